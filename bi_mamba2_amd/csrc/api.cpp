@@ -1,0 +1,266 @@
+// C ABI of libbimamba2_hip.so: argument checks, workspace carving and the forward / backward pipelines.
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+
+#include "../../include/bimamba2.h"
+#include "launch.hpp"
+
+using namespace bm2;
+
+namespace {
+
+inline int nchunks(const bimamba2_params *p) { return (p->seqlen + p->chunk_size - 1) / p->chunk_size; }
+inline hipStream_t stream_of(const bimamba2_params *p) { return reinterpret_cast<hipStream_t>(p->stream); }
+inline size_t elem_size(int dtype) { return dtype == BIMAMBA2_F32 ? 4 : 2; }
+inline int sp_nsplit(const bimamba2_params *p) { return (p->headdim * p->dstate + 1023) / 1024; }
+
+int check_problem(const bimamba2_params *p) {
+    if (!p) return BIMAMBA2_EINVAL;
+    if (p->batch <= 0 || p->seqlen <= 0 || p->nheads <= 0 || p->headdim <= 0 || p->ngroups <= 0 || p->dstate <= 0)
+        return BIMAMBA2_EINVAL;
+    if (p->nheads % p->ngroups) return BIMAMBA2_EINVAL;
+    if (p->dtype < BIMAMBA2_F32 || p->dtype > BIMAMBA2_F16) return BIMAMBA2_EUNSUPPORTED;
+    if (p->dt_dtype < BIMAMBA2_F32 || p->dt_dtype > BIMAMBA2_F16) return BIMAMBA2_EUNSUPPORTED;
+    if (p->chunk_size < BIMAMBA2_MIN_CHUNK || p->chunk_size > BIMAMBA2_MAX_CHUNK) return BIMAMBA2_EUNSUPPORTED;
+    if (p->headdim > BIMAMBA2_MAX_HEADDIM || p->dstate > BIMAMBA2_MAX_DSTATE) return BIMAMBA2_EUNSUPPORTED;
+    // grid.z = batch * nchunks * nheads must fit the launch limits
+    const int64_t z = (int64_t)p->batch * nchunks(p) * p->nheads;
+    if (z > 2147483647LL / 2) return BIMAMBA2_EUNSUPPORTED;
+    return BIMAMBA2_OK;
+}
+
+#define REQUIRE(ptr)                        \
+    do {                                    \
+        if (!(ptr)) return BIMAMBA2_EINVAL; \
+    } while (0)
+#define TRY(expr)              \
+    do {                       \
+        int rc_ = (expr);      \
+        if (rc_) return rc_;   \
+    } while (0)
+
+struct Carver {
+    char *base;
+    size_t off = 0;
+    explicit Carver(void *b) : base(static_cast<char *>(b)) {}
+    template <typename T> T *take(size_t n) {
+        off = (off + 255) & ~size_t(255);
+        T *r = base ? reinterpret_cast<T *>(base + off) : nullptr;
+        off += n * sizeof(T);
+        return r;
+    }
+};
+
+// Assigns every intermediate that is NULL in `q` from the workspace; returns the bytes used.
+size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
+    Carver cv(ws);
+    const size_t nc = nchunks(q), Q = q->chunk_size;
+    const size_t bhcq = (size_t)q->batch * q->nheads * nc * Q;
+    const size_t cbn = (size_t)q->batch * nc * q->ngroups * Q * Q;
+    const size_t stn = (size_t)q->batch * nc * q->nheads * q->headdim * q->dstate;
+    auto need_f = [&](float *&ptr, size_t n) { if (!ptr) ptr = cv.take<float>(n); };
+    need_f(q->dt_out, bhcq);
+    need_f(q->cs_f, bhcq);
+    need_f(q->cs_b, bhcq);
+    need_f(q->CB, cbn);
+    need_f(q->states_f, stn);
+    need_f(q->states_b, stn);
+    if (is_bwd) {
+        const size_t nqt = (Q + 63) / 64, rt = nqt;
+        need_f(q->dCB, cbn);
+        need_f(q->dstates_f, stn);
+        need_f(q->dstates_b, stn);
+        if (q->has_z && !q->dout_x)
+            q->dout_x = cv.take<char>((size_t)q->batch * q->seqlen * q->nheads * q->headdim * elem_size(q->dtype));
+        need_f(q->ddt_direct, bhcq);
+        need_f(q->u_f, bhcq);
+        need_f(q->u_b, bhcq);
+        need_f(q->v_f, bhcq);
+        need_f(q->v_b, bhcq);
+        need_f(q->da_intra, bhcq * nqt);
+        need_f(q->ddA_chunk_f, (size_t)q->batch * q->nheads * nc * sp_nsplit(q));
+        need_f(q->ddA_chunk_b, (size_t)q->batch * q->nheads * nc * sp_nsplit(q));
+        const size_t bn = (size_t)q->batch * q->seqlen * q->ngroups * q->dstate;
+        need_f(q->dBs, bn);
+        need_f(q->dCs, bn);
+        const size_t red = std::max((size_t)q->batch * nc * rt * q->nheads * q->headdim, (size_t)2 * q->batch * nc * q->nheads);
+        need_f(q->red, red);
+    }
+    return (cv.off + 255) & ~size_t(255);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *bimamba2_strerror(int code) {
+    switch (code) {
+        case BIMAMBA2_OK: return "ok";
+        case BIMAMBA2_EINVAL: return "invalid argument (null pointer or inconsistent dimensions)";
+        case BIMAMBA2_EUNSUPPORTED:
+            return "unsupported problem (need 32 <= chunk_size <= 256, headdim <= 128, dstate <= 256, dtype f32/bf16/f16)";
+        case BIMAMBA2_EWORKSPACE: return "workspace missing or too small";
+        case BIMAMBA2_ELAUNCH: return "HIP kernel launch failed";
+        default: return "unknown error";
+    }
+}
+
+int bimamba2_version(void) { return 100; }
+size_t bimamba2_params_size(void) { return sizeof(bimamba2_params); }
+
+size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd) {
+    if (check_problem(p)) return 0;
+    bimamba2_params q = *p;
+    return carve(&q, is_bwd, nullptr);
+}
+
+int bimamba2_chunk_cumsum_fwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->dt); REQUIRE(p->A); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (p->has_dt_bias) REQUIRE(p->dt_bias);
+    return launch_chunk_cumsum_fwd(p);
+}
+
+int bimamba2_bmm_chunk_fwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->Bm); REQUIRE(p->Cm); REQUIRE(p->CB);
+    return launch_bmm_chunk_fwd(p);
+}
+
+int bimamba2_chunk_state_fwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->states_f); REQUIRE(p->states_b);
+    return launch_chunk_state(p, false);
+}
+
+int bimamba2_state_passing_fwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
+    return launch_state_passing_fwd(p);
+}
+
+int bimamba2_chunk_scan_fwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->x); REQUIRE(p->Cm); REQUIRE(p->CB); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->states_f); REQUIRE(p->states_b); REQUIRE(p->out);
+    if (p->has_D) REQUIRE(p->D);
+    if (p->has_z) REQUIRE(p->z);
+    return launch_chunk_scan(p, false);
+}
+
+int bimamba2_chunk_scan_bwd_dz(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    if (!p->has_z) return BIMAMBA2_EINVAL;
+    REQUIRE(p->z); REQUIRE(p->dout); REQUIRE(p->out_x); REQUIRE(p->dz); REQUIRE(p->dout_x);
+    return launch_bwd_dz(p);
+}
+
+int bimamba2_chunk_scan_bwd_dstates(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->dstates_f); REQUIRE(p->dstates_b);
+    if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
+    return launch_chunk_state(p, true);
+}
+
+int bimamba2_state_passing_bwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
+    REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->ddA_chunk_f); REQUIRE(p->ddA_chunk_b);
+    return launch_state_passing_bwd(p);
+}
+
+int bimamba2_chunk_scan_bwd_dx(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->CB); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->dx); REQUIRE(p->ddt_direct);
+    if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
+    if (p->has_D) { REQUIRE(p->D); REQUIRE(p->dD); REQUIRE(p->red); }
+    const int nc = nchunks(p);
+    if (p->headdim > 64)   // several headdim tiles add their row sums atomically
+        TRY(launch_fill(p->ddt_direct, (size_t)p->batch * p->nheads * nc * p->chunk_size, 0.f, stream_of(p)));
+    TRY(launch_chunk_scan(p, true));
+    if (p->has_D) {
+        const int rt = (p->chunk_size + 63) / 64;
+        if (p->D_has_hdim) return launch_reduce(p->red, p->dD, p->batch * nc * rt, p->nheads * p->headdim, 1, stream_of(p));
+        return launch_reduce(p->red, p->dD, p->batch * nc * rt, p->nheads, p->headdim, stream_of(p));
+    }
+    return BIMAMBA2_OK;
+}
+
+int bimamba2_chunk_state_bwd_db(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->dBs); REQUIRE(p->v_f); REQUIRE(p->v_b);
+    return launch_bwd_dbdc(p, true);
+}
+
+int bimamba2_chunk_scan_bwd_dc(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
+    REQUIRE(p->dCs); REQUIRE(p->u_f); REQUIRE(p->u_b);
+    if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
+    return launch_bwd_dbdc(p, false);
+}
+
+int bimamba2_chunk_scan_bwd_dcb(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->x); REQUIRE(p->CB); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->dCB); REQUIRE(p->da_intra);
+    if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
+    return launch_bwd_dcb(p);
+}
+
+int bimamba2_bmm_chunk_bwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->Bm); REQUIRE(p->Cm); REQUIRE(p->dCB); REQUIRE(p->dBs); REQUIRE(p->dCs); REQUIRE(p->dB); REQUIRE(p->dC);
+    return launch_bmm_chunk_bwd(p);
+}
+
+int bimamba2_chunk_cumsum_bwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    REQUIRE(p->dt); REQUIRE(p->A); REQUIRE(p->da_intra); REQUIRE(p->u_f); REQUIRE(p->u_b); REQUIRE(p->v_f); REQUIRE(p->v_b);
+    REQUIRE(p->ddA_chunk_f); REQUIRE(p->ddA_chunk_b); REQUIRE(p->ddt_direct); REQUIRE(p->ddt); REQUIRE(p->dA); REQUIRE(p->red);
+    if (p->has_dt_bias) REQUIRE(p->dt_bias);
+    return launch_chunk_cumsum_bwd(p);
+}
+
+int bimamba2_fwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    bimamba2_params q = *p;
+    const size_t need = carve(&q, 0, p->workspace);
+    if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
+    TRY(bimamba2_chunk_cumsum_fwd(&q));
+    TRY(bimamba2_bmm_chunk_fwd(&q));
+    TRY(bimamba2_chunk_state_fwd(&q));
+    TRY(bimamba2_state_passing_fwd(&q));
+    TRY(bimamba2_chunk_scan_fwd(&q));
+    return BIMAMBA2_OK;
+}
+
+int bimamba2_bwd(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    bimamba2_params q = *p;
+    q.final_f = q.final_b = nullptr;
+    const size_t need = carve(&q, 1, p->workspace);
+    if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
+    // recompute the forward intermediates (the reference does the same, src/ssd/bi/ssd_combined.py:373-380)
+    TRY(bimamba2_chunk_cumsum_fwd(&q));
+    TRY(bimamba2_bmm_chunk_fwd(&q));
+    TRY(bimamba2_chunk_state_fwd(&q));
+    TRY(bimamba2_state_passing_fwd(&q));
+    if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
+    TRY(bimamba2_chunk_scan_bwd_dstates(&q));
+    TRY(bimamba2_state_passing_bwd(&q));
+    TRY(bimamba2_chunk_scan_bwd_dx(&q));
+    TRY(bimamba2_chunk_state_bwd_db(&q));
+    TRY(bimamba2_chunk_scan_bwd_dc(&q));
+    TRY(bimamba2_chunk_scan_bwd_dcb(&q));
+    TRY(bimamba2_bmm_chunk_bwd(&q));
+    TRY(bimamba2_chunk_cumsum_bwd(&q));
+    return BIMAMBA2_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,215 @@
+// Shared device helpers for the gfx950 kernels: element types, 16x16 MFMA fragments, LDS tile loaders,
+// wavefront scans.  Wave size is 64; every kernel here runs 256 threads = 4 waves per workgroup.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/bimamba2.h"
+
+namespace bm2 {
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int NTHREADS = 256;
+constexpr int BK = 32;          // K extent of one LDS tile
+
+__device__ __forceinline__ float to_f(float v) { return v; }
+__device__ __forceinline__ float to_f(bf16_t v) { return static_cast<float>(v); }
+__device__ __forceinline__ float to_f(f16_t v) { return static_cast<float>(v); }
+template <typename T> __device__ __forceinline__ T from_f(float v) { return static_cast<T>(v); }
+
+// ---- MFMA 16x16 fragments -----------------------------------------------------------------------------
+// Output tile D (16x16, f32): lane l holds rows 4*(l/16)+i (i=0..3) of column l%16.
+// A operand: lane l holds KPL consecutive k of row l%16 starting at KPL*(l/16); B operand likewise for
+// column l%16.  Both operands use the same k mapping, so any consistent mapping gives the same product.
+template <typename T> struct Mma;
+template <> struct Mma<float> {
+    static constexpr int KPL = 1, KSTEP = 4, LD = BK + 4;
+    typedef float Frag;
+    static __device__ __forceinline__ Frag load(const float *p) { return *p; }
+    static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mma<bf16_t> {
+    static constexpr int KPL = 8, KSTEP = 32, LD = BK + 8;
+    typedef bf16x8 Frag;
+    static __device__ __forceinline__ Frag load(const bf16_t *p) { return *reinterpret_cast<const bf16x8 *>(p); }
+    static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mma<f16_t> {
+    static constexpr int KPL = 8, KSTEP = 32, LD = BK + 8;
+    typedef f16x8 Frag;
+    static __device__ __forceinline__ Frag load(const f16_t *p) { return *reinterpret_cast<const f16x8 *>(p); }
+    static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// acc[j] += A(16 rows at As) * B(16 cols at Bs + 16*j rows)^T over one BK-wide LDS tile.
+// As points at the first of the wave's 16 rows ([row][k], leading dimension LD); Bs at the first of NJ*16
+// columns stored [col][k].
+template <typename T, int NJ>
+__device__ __forceinline__ void mma_tile(f32x4 (&acc)[NJ], const T *As, const T *Bs, int lane) {
+    typedef Mma<T> M;
+    const int r = lane & 15, kq = (lane >> 4) * M::KPL;
+#pragma unroll
+    for (int k0 = 0; k0 < BK; k0 += M::KSTEP) {
+        typename M::Frag a = M::load(As + r * M::LD + k0 + kq);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            typename M::Frag b = M::load(Bs + (16 * j + r) * M::LD + k0 + kq);
+            acc[j] = M::mma(a, b, acc[j]);
+        }
+    }
+}
+
+// ---- global -> LDS tile loaders -----------------------------------------------------------------------
+template <typename S> struct Vec16 {
+    static constexpr int N = 16 / sizeof(S);
+    S v[N];
+};
+
+template <typename S> __device__ __forceinline__ bool aligned16(const S *p, int64_t stride_elems) {
+    return ((reinterpret_cast<uintptr_t>(p) | static_cast<uintptr_t>(stride_elems * sizeof(S))) & 15) == 0;
+}
+
+// dst[r][k] = f(r, k, src[r*rs + k]) for r < ROWS, k < BK; elements with r >= rvalid or k >= kvalid are 0
+// (f is still applied to the 0).  Source is contiguous along k.
+template <typename T, typename S, int ROWS, class F>
+__device__ __forceinline__ void tile_load_kcontig(T *dst, const S *src, int64_t rs, int rvalid, int kvalid, F f) {
+    constexpr int VS = 16 / sizeof(S), KV = BK / VS, LD = Mma<T>::LD;
+    const bool vec = aligned16(src, rs);
+    for (int idx = threadIdx.x; idx < ROWS * KV; idx += NTHREADS) {
+        const int r = idx / KV, k0 = (idx % KV) * VS;
+        float v[VS];
+        if (vec && r < rvalid && k0 + VS <= kvalid) {
+            Vec16<S> raw = *reinterpret_cast<const Vec16<S> *>(src + r * rs + k0);
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = to_f(raw.v[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = (r < rvalid && k0 + i < kvalid) ? to_f(src[r * rs + k0 + i]) : 0.f;
+        }
+        struct alignas(sizeof(T) * VS) Out { T v[VS]; } o;
+#pragma unroll
+        for (int i = 0; i < VS; ++i) o.v[i] = from_f<T>(f(r, k0 + i, v[i]));
+        *reinterpret_cast<Out *>(dst + r * LD + k0) = o;
+    }
+}
+
+// dst[r][k] = f(r, k, src[k*ks + r]): the source is contiguous along r (transposing load).
+template <typename T, typename S, int ROWS, class F>
+__device__ __forceinline__ void tile_load_rcontig(T *dst, const S *src, int64_t ks, int rvalid, int kvalid, F f) {
+    constexpr int VS = 16 / sizeof(S), RV = ROWS / VS, LD = Mma<T>::LD;
+    const bool vec = aligned16(src, ks);
+    for (int idx = threadIdx.x; idx < BK * RV; idx += NTHREADS) {
+        const int k = idx / RV, r0 = (idx % RV) * VS;
+        float v[VS];
+        if (vec && k < kvalid && r0 + VS <= rvalid) {
+            Vec16<S> raw = *reinterpret_cast<const Vec16<S> *>(src + k * ks + r0);
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = to_f(raw.v[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = (k < kvalid && r0 + i < rvalid) ? to_f(src[k * ks + r0 + i]) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < VS; ++i) dst[(r0 + i) * LD + k] = from_f<T>(f(r0 + i, k, v[i]));
+    }
+}
+
+// same, writing two tiles with two functors from one read of the source
+template <typename T, typename S, int ROWS, class F1, class F2>
+__device__ __forceinline__ void tile_load_rcontig2(T *dst1, T *dst2, const S *src, int64_t ks, int rvalid,
+                                                   int kvalid, F1 f1, F2 f2) {
+    constexpr int VS = 16 / sizeof(S), RV = ROWS / VS, LD = Mma<T>::LD;
+    const bool vec = aligned16(src, ks);
+    for (int idx = threadIdx.x; idx < BK * RV; idx += NTHREADS) {
+        const int k = idx / RV, r0 = (idx % RV) * VS;
+        float v[VS];
+        if (vec && k < kvalid && r0 + VS <= rvalid) {
+            Vec16<S> raw = *reinterpret_cast<const Vec16<S> *>(src + k * ks + r0);
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = to_f(raw.v[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = (k < kvalid && r0 + i < rvalid) ? to_f(src[k * ks + r0 + i]) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < VS; ++i) {
+            dst1[(r0 + i) * LD + k] = from_f<T>(f1(r0 + i, k, v[i]));
+            dst2[(r0 + i) * LD + k] = from_f<T>(f2(r0 + i, k, v[i]));
+        }
+    }
+}
+
+struct Ident {
+    __device__ __forceinline__ float operator()(int, int, float v) const { return v; }
+};
+
+// ---- wavefront helpers --------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+    return v;
+}
+// sum over the 16 lanes that share l/16 (one row group of an MFMA output tile)
+__device__ __forceinline__ float row16_sum(float v) {
+#pragma unroll
+    for (int d = 8; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+    return v;
+}
+// inclusive prefix / suffix sums over the 64 lanes
+__device__ __forceinline__ float wave_incl_prefix(float v, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        float o = __shfl_up(v, d, 64);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+__device__ __forceinline__ float wave_incl_suffix(float v, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        float o = __shfl_down(v, d, 64);
+        if (lane + d < 64) v += o;
+    }
+    return v;
+}
+
+template <int CTRL> __device__ __forceinline__ float dpp_mov0(float v) {
+    // lanes whose source lies outside their row of 16 receive 0
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// inclusive prefix (towards higher lanes) / suffix sums inside each row of 16 lanes
+__device__ __forceinline__ float row16_incl_prefix(float v) {
+    v += dpp_mov0<0x111>(v);  // row_shr:1
+    v += dpp_mov0<0x112>(v);  // row_shr:2
+    v += dpp_mov0<0x114>(v);  // row_shr:4
+    v += dpp_mov0<0x118>(v);  // row_shr:8
+    return v;
+}
+__device__ __forceinline__ float row16_incl_suffix(float v) {
+    v += dpp_mov0<0x101>(v);  // row_shl:1
+    v += dpp_mov0<0x102>(v);
+    v += dpp_mov0<0x104>(v);
+    v += dpp_mov0<0x108>(v);
+    return v;
+}
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + __expf(-z)); }
+
+// chunk bookkeeping shared by all kernels
+struct ChunkIdx {
+    int b, c, h, g, limit;
+};
+
+}  // namespace bm2

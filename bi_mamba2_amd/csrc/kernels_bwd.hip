@@ -1,0 +1,646 @@
+// Backward kernels of the bidirectional SSD operator for gfx950 (the gradient of the chunk-entry states and dx
+// reuse chunk_state_kernel / chunk_scan_kernel from kernels_fwd.hip).
+//   bwd_dz             dz and dout*silu(z)
+//   state_passing_bwd  both inter-chunk adjoint recurrences in one launch + the chunk-total decay gradients
+//   bwd_dbdc           state part of dB (or dC) summed over the heads of a group + per-position decay terms
+//   bwd_dcb            G = dy.x^T once per head -> dCB (summed over heads) and the within-chunk decay gradient
+//   bmm_chunk_bwd      dB = dBs + dCB^T.C ; dC = dCs + dCB.B
+//   chunk_cumsum_bwd   assembles d(dt*A) from its pieces with wavefront scans; ddt, dA, ddt_bias
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace bm2 {
+
+static inline int nchunks(const bimamba2_params *p) { return (p->seqlen + p->chunk_size - 1) / p->chunk_size; }
+static inline hipStream_t stream_of(const bimamba2_params *p) { return reinterpret_cast<hipStream_t>(p->stream); }
+
+// =========================================================================================================
+__global__ void fill_kernel(float *ptr, size_t n, float value) {
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) ptr[i] = value;
+}
+int launch_fill(float *ptr, size_t n, float value, hipStream_t stream) {
+    if (n == 0) return BIMAMBA2_OK;
+    const int blocks = (int)std::min<size_t>((n + 255) / 256, 2048);
+    hipLaunchKernelGGL(fill_kernel, dim3(blocks), dim3(256), 0, stream, ptr, n, value);
+    return check_launch();
+}
+
+// out[j] = sum_i sum_k in[(i*nj + j)*nk + k]; one workgroup per j
+__global__ __launch_bounds__(NTHREADS) void reduce_kernel(const float *in, float *out, int ni, int nj, int nk) {
+    __shared__ float red[4];
+    const int j = blockIdx.x;
+    float s = 0.f;
+    const int total = ni * nk;
+    for (int t = threadIdx.x; t < total; t += NTHREADS) {
+        const int i = t / nk, k = t - i * nk;
+        s += in[((int64_t)i * nj + j) * nk + k];
+    }
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) out[j] = red[0] + red[1] + red[2] + red[3];
+}
+int launch_reduce(const float *in, float *out, int ni, int nj, int nk, hipStream_t stream) {
+    hipLaunchKernelGGL(reduce_kernel, dim3(nj), dim3(NTHREADS), 0, stream, in, out, ni, nj, nk);
+    return check_launch();
+}
+
+// =========================================================================================================
+// dz = dout * out_x * sigmoid(z) (1 + z (1 - sigmoid(z)));  dout_x = dout * z * sigmoid(z)
+// =========================================================================================================
+template <typename T>
+__global__ __launch_bounds__(NTHREADS) void bwd_dz_kernel(const bimamba2_params p) {
+    constexpr int VS = 16 / sizeof(T);
+    const int P = p.headdim;
+    const int pv = (P + VS - 1) / VS;
+    const int64_t nrows = (int64_t)p.batch * p.seqlen * p.nheads;
+    const T *zb = reinterpret_cast<const T *>(p.z);
+    const T *db = reinterpret_cast<const T *>(p.dout);
+    const T *ox = reinterpret_cast<const T *>(p.out_x);
+    T *dz = reinterpret_cast<T *>(p.dz);
+    T *dox = reinterpret_cast<T *>(p.dout_x);
+    for (int64_t idx = blockIdx.x * (int64_t)NTHREADS + threadIdx.x; idx < nrows * pv; idx += (int64_t)gridDim.x * NTHREADS) {
+        const int64_t row = idx / pv;
+        const int c0 = (int)(idx - row * pv) * VS;
+        const int h = (int)(row % p.nheads);
+        const int64_t bl = row / p.nheads;
+        const int l = (int)(bl % p.seqlen), b = (int)(bl / p.seqlen);
+        const T *zp = zb + b * p.z_sb + l * p.z_sl + h * p.z_sh + c0;
+        const T *dp = db + b * p.dout_sb + l * p.dout_sl + h * p.dout_sh + c0;
+        const int64_t o = row * P + c0;
+        const bool vec = (c0 + VS <= P) && aligned16(zp, 0) && aligned16(dp, 0) && aligned16(ox + o, 0);
+        float zv[VS], dv[VS], ov[VS];
+        if (vec) {
+            Vec16<T> a = *reinterpret_cast<const Vec16<T> *>(zp), d = *reinterpret_cast<const Vec16<T> *>(dp),
+                     e = *reinterpret_cast<const Vec16<T> *>(ox + o);
+#pragma unroll
+            for (int i = 0; i < VS; ++i) { zv[i] = to_f(a.v[i]); dv[i] = to_f(d.v[i]); ov[i] = to_f(e.v[i]); }
+        } else {
+#pragma unroll
+            for (int i = 0; i < VS; ++i) {
+                const bool ok = c0 + i < P;
+                zv[i] = ok ? to_f(zp[i]) : 0.f; dv[i] = ok ? to_f(dp[i]) : 0.f; ov[i] = ok ? to_f(ox[o + i]) : 0.f;
+            }
+        }
+        Vec16<T> r1, r2;
+#pragma unroll
+        for (int i = 0; i < VS; ++i) {
+            const float sg = sigmoid_f(zv[i]);
+            r1.v[i] = from_f<T>(dv[i] * ov[i] * sg * (1.f + zv[i] * (1.f - sg)));
+            r2.v[i] = from_f<T>(dv[i] * zv[i] * sg);
+        }
+        if (vec) {
+            *reinterpret_cast<Vec16<T> *>(dz + o) = r1;
+            *reinterpret_cast<Vec16<T> *>(dox + o) = r2;
+        } else {
+#pragma unroll
+            for (int i = 0; i < VS; ++i)
+                if (c0 + i < P) { dz[o + i] = r1.v[i]; dox[o + i] = r2.v[i]; }
+        }
+    }
+}
+
+int launch_bwd_dz(const bimamba2_params *p) {
+    const int64_t n = (int64_t)p->batch * p->seqlen * p->nheads * ((p->headdim + 3) / 4);
+    const int blocks = (int)std::min<int64_t>((n + NTHREADS - 1) / NTHREADS, 8192);
+    switch (p->dtype) {
+        case BIMAMBA2_F32: hipLaunchKernelGGL(bwd_dz_kernel<float>, dim3(blocks), dim3(NTHREADS), 0, stream_of(p), *p); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL(bwd_dz_kernel<bf16_t>, dim3(blocks), dim3(NTHREADS), 0, stream_of(p), *p); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL(bwd_dz_kernel<f16_t>, dim3(blocks), dim3(NTHREADS), 0, stream_of(p), *p); break;
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+    return check_launch();
+}
+
+// =========================================================================================================
+// adjoint of the inter-chunk recurrences.  On entry dstates_* hold the gradient w.r.t. the state entering
+// each chunk (dprev); on exit they hold the gradient w.r.t. each chunk's own state S[c]:
+//   forward dir : g = 0; for c = nc-1..0 : dS_f[c] = g; ddA_chunk_f[c] = e^{tot_c} <g, prev_f[c]>; g = dprev_f[c] + e^{tot_c} g
+//   reverse dir : g = 0; for c = 0..nc-1 : dS_b[c] = g; ddA_chunk_b[c] = e^{tot_c} <g, prev_b[c]>; g = dprev_b[c] + e^{tot_c} g
+// A workgroup owns SP_EPT*256 of the P*N elements of one (b, h); its partial inner products go to
+// ddA_chunk_*[b, h, c, split].
+// =========================================================================================================
+constexpr int SP_EPT = 4;
+__global__ __launch_bounds__(NTHREADS) void state_passing_bwd_kernel(const bimamba2_params p, int nc, int nsplit) {
+    __shared__ float red[2][4];
+    const int PN = p.headdim * p.dstate;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int Q = p.chunk_size;
+    const float *csf = p.cs_f + ((int64_t)b * p.nheads + h) * nc * Q;
+    const float *csb = p.cs_b + ((int64_t)b * p.nheads + h) * nc * Q;
+    const int64_t cstride = (int64_t)p.nheads * PN;
+    const int64_t base = ((int64_t)b * nc * p.nheads + h) * PN;
+    const int e0 = split * SP_EPT * NTHREADS + threadIdx.x;
+    for (int dir = 0; dir < 2; ++dir) {
+        const float *prev = (dir == 0 ? p.states_f : p.states_b) + base;
+        float *ds = (dir == 0 ? p.dstates_f : p.dstates_b) + base;
+        float *dda = (dir == 0 ? p.ddA_chunk_f : p.ddA_chunk_b) + ((int64_t)b * p.nheads + h) * nc * nsplit + split;
+        float g[SP_EPT];
+#pragma unroll
+        for (int i = 0; i < SP_EPT; ++i) g[i] = 0.f;
+        for (int step = 0; step < nc; ++step) {
+            const int c = dir == 0 ? nc - 1 - step : step;
+            const float dec = __expf(dir == 0 ? csf[(int64_t)c * Q + Q - 1] : csb[(int64_t)c * Q]);
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < SP_EPT; ++i) {
+                const int e = e0 + i * NTHREADS;
+                if (e < PN) {
+                    const int64_t a = c * cstride + e;
+                    const float dp = ds[a];
+                    dot += g[i] * prev[a];
+                    ds[a] = g[i];
+                    g[i] = dp + dec * g[i];
+                }
+            }
+            dot = wave_sum(dot);
+            if (lane == 0) red[step & 1][wave] = dot;
+            __syncthreads();
+            if (threadIdx.x == 0) dda[(int64_t)c * nsplit] = dec * (red[step & 1][0] + red[step & 1][1] + red[step & 1][2] + red[step & 1][3]);
+        }
+        __syncthreads();
+    }
+}
+
+int launch_state_passing_bwd(const bimamba2_params *p) {
+    const int nc = nchunks(p), PN = p->headdim * p->dstate;
+    const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS);
+    dim3 grid(nsplit, p->nheads, p->batch);
+    hipLaunchKernelGGL(state_passing_bwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit);
+    return check_launch();
+}
+
+// =========================================================================================================
+// state part of dC (IS_DB = false), rows r = positions t of a 64-row tile, summed over the heads of a group:
+//   tmp_f = dy_h[r,:] . prev_f[h]  (K = headdim),  dCs[r,n] += e^{cs_f[r]} tmp_f + e^{cs_b[r]} tmp_b
+//   u_f[h,r] = e^{cs_f[r]} sum_n tmp_f[r,n] C[r,n]      (same for b)
+// state part of dB (IS_DB = true), rows r = positions s:
+//   tmp_f = x_h[r,:] . dS_f[h],  dBs[r,n] += dt[r] (e^{cs_f[Q-1]-cs_f[r]} tmp_f + e^{cs_b[0]-cs_b[r]} tmp_b)
+//   v_f[h,r] = dt[r] e^{cs_f[Q-1]-cs_f[r]} sum_n tmp_f[r,n] B[r,n]
+// =========================================================================================================
+template <typename T, int NT, bool IS_DB>
+__global__ __launch_bounds__(NTHREADS) void bwd_dbdc_kernel(const bimamba2_params p, int nc) {
+    constexpr int LD = Mma<T>::LD;
+    __shared__ __attribute__((aligned(16))) T As[64 * LD];
+    __shared__ __attribute__((aligned(16))) T Bf[64 * LD];
+    __shared__ __attribute__((aligned(16))) T Bb[64 * LD];
+    __shared__ float sfs[64], sbs[64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rt = blockIdx.x;
+    const int g = blockIdx.y % p.ngroups, bc = blockIdx.y / p.ngroups, c = bc % nc, b = bc / nc;
+    const int Q = p.chunk_size, N = p.dstate, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int r0 = rt * 64;
+    // B or C values of this lane's output elements
+    const T *cbp;
+    int64_t cbs;
+    if (IS_DB) { cbs = p.B_sl; cbp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + ((int64_t)c * Q + r0) * cbs + g * p.B_sg; }
+    else { cbs = p.C_sl; cbp = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + ((int64_t)c * Q + r0) * cbs + g * p.C_sg; }
+    float creg[NT][4][4];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int rl = wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
+                creg[nt][j][i] = (r0 + rl < limit && n < N) ? to_f(cbp[(int64_t)rl * cbs + n]) : 0.f;
+            }
+    f32x4 tot[NT][4] = {};
+    for (int hh = 0; hh < hpg; ++hh) {
+        const int h = g * hpg + hh;
+        const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            const int r = r0 + threadIdx.x;
+            float f = 0.f, s = 0.f;
+            if (r < limit) {
+                if (IS_DB) {
+                    const float d = p.dt_out[o + r];
+                    f = d * __expf(p.cs_f[o + Q - 1] - p.cs_f[o + r]);
+                    s = d * __expf(p.cs_b[o] - p.cs_b[o + r]);
+                } else {
+                    f = __expf(p.cs_f[o + r]);
+                    s = __expf(p.cs_b[o + r]);
+                }
+            }
+            sfs[threadIdx.x] = f;
+            sbs[threadIdx.x] = s;
+        }
+        const T *ap;
+        int64_t as;
+        if (IS_DB) { as = p.x_sl; ap = reinterpret_cast<const T *>(p.x) + b * p.x_sb + ((int64_t)c * Q + r0) * as + h * p.x_sh; }
+        else if (p.has_z) { as = (int64_t)H * P; ap = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q + r0) * as + (int64_t)h * P; }
+        else { as = p.dout_sl; ap = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + ((int64_t)c * Q + r0) * as + h * p.dout_sh; }
+        const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * N;
+        const float *s1 = (IS_DB ? p.dstates_f : p.states_f) + so;
+        const float *s2 = (IS_DB ? p.dstates_b : p.states_b) + so;
+        float uf[4] = {0.f, 0.f, 0.f, 0.f}, ub[4] = {0.f, 0.f, 0.f, 0.f};
+        float sfr[4], sbr[4];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            if (nt * 64 >= N) break;
+            f32x4 tf[4] = {}, tb[4] = {};
+            for (int k0 = 0; k0 < P; k0 += BK) {
+                __syncthreads();
+                tile_load_kcontig<T, T, 64>(As, ap + k0, as, limit - r0, P - k0, Ident());
+                // state[p][n] -> [n][p]: element (r = n, k = p) at s + k*N + n
+                tile_load_rcontig<T, float, 64>(Bf, s1 + (int64_t)k0 * N + nt * 64, N, N - nt * 64, P - k0, Ident());
+                tile_load_rcontig<T, float, 64>(Bb, s2 + (int64_t)k0 * N + nt * 64, N, N - nt * 64, P - k0, Ident());
+                __syncthreads();
+                mma_tile<T, 4>(tf, As + wave * 16 * LD, Bf, lane);
+                mma_tile<T, 4>(tb, As + wave * 16 * LD, Bb, lane);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int rl = wave * 16 + (lane >> 4) * 4 + i;
+                sfr[i] = sfs[rl];
+                sbr[i] = sbs[rl];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    uf[i] += tf[j][i] * creg[nt][j][i];
+                    ub[i] += tb[j][i] * creg[nt][j][i];
+                    tot[nt][j][i] += sfr[i] * tf[j][i] + sbr[i] * tb[j][i];
+                }
+            }
+        }
+        float *of = IS_DB ? p.v_f : p.u_f, *ob = IS_DB ? p.v_b : p.u_b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = r0 + wave * 16 + (lane >> 4) * 4 + i;
+            const float a = row16_sum(uf[i]) * sfr[i], bb = row16_sum(ub[i]) * sbr[i];
+            if ((lane & 15) == 0 && r < Q) {
+                of[o + r] = a;
+                ob[o + r] = bb;
+            }
+        }
+    }
+    float *out = (IS_DB ? p.dBs : p.dCs);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = r0 + wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
+                if (r < limit && n < N)
+                    out[(((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n] = tot[nt][j][i];
+            }
+}
+
+template <typename T, bool IS_DB>
+static int launch_dbdc_t(const bimamba2_params *p) {
+    const int nc = nchunks(p);
+    dim3 grid((p->chunk_size + 63) / 64, p->batch * nc * p->ngroups);
+    const int nt = (p->dstate + 63) / 64;
+    if (nt == 1) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 1, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    else if (nt == 2) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 2, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    else if (nt <= 4) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 4, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    else return BIMAMBA2_EUNSUPPORTED;
+    return check_launch();
+}
+
+int launch_bwd_dbdc(const bimamba2_params *p, bool is_db) {
+    switch (p->dtype) {
+        case BIMAMBA2_F32: return is_db ? launch_dbdc_t<float, true>(p) : launch_dbdc_t<float, false>(p);
+        case BIMAMBA2_BF16: return is_db ? launch_dbdc_t<bf16_t, true>(p) : launch_dbdc_t<bf16_t, false>(p);
+        case BIMAMBA2_F16: return is_db ? launch_dbdc_t<f16_t, true>(p) : launch_dbdc_t<f16_t, false>(p);
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+}
+
+// =========================================================================================================
+// G[t,s] = dy_h[t,:] . x_h[s,:]  (K = headdim) for a 64-row tile of t and all s of the chunk, per head:
+//   f[t,s] = 1[s<=t] G dt[s] e^{cs_f[t]-cs_f[s]},  b[t,s] = 1[s>=t] G dt[s] e^{cs_b[t]-cs_b[s]}
+//   dCB[t,s] = sum_{h in group} (f + b)
+//   da_intra[h, i] = sum_{t>=i} sum_{s<i} f[t,s] CB[t,s]  +  sum_{t<=i} sum_{s>i} b[t,s] CB[t,s]
+// The row prefix (resp. suffix) over s runs across the 16 lanes of an MFMA row group with DPP adds and is
+// carried from column tile to column tile, ascending s for the forward direction, descending for the reverse.
+// Output da_intra[b, h, c, tt, Q] holds this row tile's share; the consumer sums over tt.
+// =========================================================================================================
+template <typename T, int QT>
+__global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params p, int nc) {
+    constexpr int LD = Mma<T>::LD;
+    __shared__ __attribute__((aligned(16))) T As[64 * LD];
+    __shared__ __attribute__((aligned(16))) T Bs[64 * LD];
+    __shared__ float csf[BIMAMBA2_MAX_CHUNK], csb[BIMAMBA2_MAX_CHUNK], dts[BIMAMBA2_MAX_CHUNK];
+    __shared__ float red[4][QT * 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tt = blockIdx.x;
+    const int g = blockIdx.y % p.ngroups, bc = blockIdx.y / p.ngroups, c = bc % nc, b = bc / nc;
+    const int Q = p.chunk_size, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int t0 = tt * 64;
+    const int nqt = (Q + 63) / 64;
+    const float *cbg = p.CB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    int trow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) trow[i] = t0 + wave * 16 + (lane >> 4) * 4 + i;
+    f32x4 cbr[QT][4], dcb[QT][4] = {};
+#pragma unroll
+    for (int st = 0; st < QT; ++st)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int s = st * 64 + j * 16 + (lane & 15);
+                cbr[st][j][i] = (trow[i] < Q && s < Q) ? cbg[(int64_t)trow[i] * Q + s] : 0.f;
+            }
+    for (int hh = 0; hh < hpg; ++hh) {
+        const int h = g * hpg + hh;
+        const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
+        __syncthreads();
+        for (int q = threadIdx.x; q < Q; q += NTHREADS) {
+            csf[q] = p.cs_f[o + q];
+            csb[q] = p.cs_b[o + q];
+            dts[q] = p.dt_out[o + q];
+        }
+        const T *yp;
+        int64_t ys;
+        if (p.has_z) { ys = (int64_t)H * P; yp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * ys + (int64_t)h * P; }
+        else { ys = p.dout_sl; yp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * ys + h * p.dout_sh; }
+        const T *xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh;
+        float col[QT][4];
+#pragma unroll
+        for (int st = 0; st < QT; ++st)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) col[st][j] = 0.f;
+
+        auto gtile = [&](int st, f32x4(&acc)[4]) {
+            for (int k0 = 0; k0 < P; k0 += BK) {
+                __syncthreads();
+                tile_load_kcontig<T, T, 64>(As, yp + (int64_t)t0 * ys + k0, ys, limit - t0, P - k0, Ident());
+                tile_load_kcontig<T, T, 64>(Bs, xp + (int64_t)st * 64 * p.x_sl + k0, p.x_sl, limit - st * 64, P - k0, Ident());
+                __syncthreads();
+                mma_tile<T, 4>(acc, As + wave * 16 * LD, Bs, lane);
+            }
+        };
+        float csft[4], csbt[4];
+        // (cs vectors were written before the first barrier inside gtile; read them after it)
+        // ---- ascending pass: forward direction, column tiles st <= tt ----
+        float carry[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int st = 0; st < QT; ++st) {
+            if (st > tt || st * 64 >= limit) continue;
+            f32x4 acc[4] = {};
+            gtile(st, acc);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { csft[i] = csf[min(trow[i], Q - 1)]; csbt[i] = csb[min(trow[i], Q - 1)]; }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int s = st * 64 + j * 16 + (lane & 15);
+                const int sc = min(s, Q - 1);
+                const float dtv = dts[sc], cfs = csf[sc], cbs_ = csb[sc];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int t = trow[i];
+                    const float gv = acc[j][i] * dtv;
+                    const float f = (s <= t) ? gv * __expf(csft[i] - cfs) : 0.f;
+                    float both = f;
+                    if (st == tt) both += (s >= t) ? gv * __expf(csbt[i] - cbs_) : 0.f;
+                    dcb[st][j][i] += both;
+                    const float w = (s < t) ? f * cbr[st][j][i] : 0.f;
+                    const float incl = row16_incl_prefix(w);
+                    const float excl = carry[i] + incl - w;
+                    if (t >= s) col[st][j] += excl;
+                    carry[i] += row16_sum(w);
+                }
+            }
+        }
+        // ---- descending pass: reverse direction, column tiles st >= tt ----
+#pragma unroll
+        for (int i = 0; i < 4; ++i) carry[i] = 0.f;
+#pragma unroll
+        for (int st = QT - 1; st >= 0; --st) {
+            if (st < tt || st * 64 >= limit) continue;
+            f32x4 acc[4] = {};
+            gtile(st, acc);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) csbt[i] = csb[min(trow[i], Q - 1)];
+#pragma unroll
+            for (int j = 3; j >= 0; --j) {
+                const int s = st * 64 + j * 16 + (lane & 15);
+                const int sc = min(s, Q - 1);
+                const float dtv = dts[sc], cbs_ = csb[sc];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int t = trow[i];
+                    const float gv = acc[j][i] * dtv;
+                    const float bv = (s >= t) ? gv * __expf(csbt[i] - cbs_) : 0.f;
+                    if (st != tt) dcb[st][j][i] += bv;
+                    const float w = (s > t) ? bv * cbr[st][j][i] : 0.f;
+                    const float incl = row16_incl_suffix(w);
+                    const float excl = carry[i] + incl - w;
+                    if (t <= s) col[st][j] += excl;
+                    carry[i] += row16_sum(w);
+                }
+            }
+        }
+        // ---- column sums over the 64 rows of this tile ----
+#pragma unroll
+        for (int st = 0; st < QT; ++st)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v = col[st][j];
+                v += __shfl_xor(v, 16, 64);
+                v += __shfl_xor(v, 32, 64);
+                if (lane < 16) red[wave][st * 64 + j * 16 + lane] = v;
+            }
+        __syncthreads();
+        for (int q = threadIdx.x; q < Q; q += NTHREADS)
+            p.da_intra[(o * nqt) + (int64_t)tt * Q + q] = red[0][q] + red[1][q] + red[2][q] + red[3][q];
+    }
+    float *out = p.dCB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+#pragma unroll
+    for (int st = 0; st < QT; ++st)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int s = st * 64 + j * 16 + (lane & 15);
+                if (trow[i] < Q && s < Q) out[(int64_t)trow[i] * Q + s] = dcb[st][j][i];
+            }
+}
+
+template <typename T>
+static int launch_dcb_t(const bimamba2_params *p) {
+    const int nc = nchunks(p), qt = (p->chunk_size + 63) / 64;
+    dim3 grid(qt, p->batch * nc * p->ngroups);
+    if (qt == 1) hipLaunchKernelGGL((bwd_dcb_kernel<T, 1>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    else if (qt == 2) hipLaunchKernelGGL((bwd_dcb_kernel<T, 2>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    else if (qt <= 4) hipLaunchKernelGGL((bwd_dcb_kernel<T, 4>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    else return BIMAMBA2_EUNSUPPORTED;
+    return check_launch();
+}
+
+int launch_bwd_dcb(const bimamba2_params *p) {
+    switch (p->dtype) {
+        case BIMAMBA2_F32: return launch_dcb_t<float>(p);
+        case BIMAMBA2_BF16: return launch_dcb_t<bf16_t>(p);
+        case BIMAMBA2_F16: return launch_dcb_t<f16_t>(p);
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+}
+
+// =========================================================================================================
+// which = 0 : dB[s,n] = dBs[s,n] + sum_t dCB[t,s] C[t,n]      which = 1 : dC[t,n] = dCs[t,n] + sum_s dCB[t,s] B[s,n]
+// =========================================================================================================
+template <typename T>
+__global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_params p, int nc) {
+    constexpr int LD = Mma<T>::LD;
+    __shared__ __attribute__((aligned(16))) T As[64 * LD];
+    __shared__ __attribute__((aligned(16))) T Bs[64 * LD];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nt = blockIdx.x, rt = blockIdx.y;
+    const int which = blockIdx.z & 1, bcg = blockIdx.z >> 1;
+    const int g = bcg % p.ngroups, bc = bcg / p.ngroups, c = bc % nc, b = bc / nc;
+    const int Q = p.chunk_size, N = p.dstate;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int r0 = rt * 64;
+    const float *dcb = p.dCB + (int64_t)bcg * Q * Q;
+    const T *op;
+    int64_t os;
+    if (which == 0) { os = p.C_sl; op = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * os + g * p.C_sg + nt * 64; }
+    else { os = p.B_sl; op = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * os + g * p.B_sg + nt * 64; }
+    f32x4 acc[4] = {};
+    for (int k0 = 0; k0 < limit; k0 += BK) {
+        __syncthreads();
+        if (which == 0) tile_load_rcontig<T, float, 64>(As, dcb + (int64_t)k0 * Q + r0, Q, Q - r0, Q - k0, Ident());
+        else tile_load_kcontig<T, float, 64>(As, dcb + (int64_t)r0 * Q + k0, Q, Q - r0, Q - k0, Ident());
+        tile_load_rcontig<T, T, 64>(Bs, op + k0 * os, os, N - nt * 64, limit - k0, Ident());
+        __syncthreads();
+        mma_tile<T, 4>(acc, As + wave * 16 * LD, Bs, lane);
+    }
+    const float *res = which == 0 ? p.dBs : p.dCs;
+    T *out = reinterpret_cast<T *>(which == 0 ? p.dB : p.dC);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = r0 + wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
+            if (r < limit && n < N) {
+                const int64_t a = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n;
+                out[a] = from_f<T>(acc[j][i] + res[a]);
+            }
+        }
+}
+
+int launch_bmm_chunk_bwd(const bimamba2_params *p) {
+    const int nc = nchunks(p);
+    dim3 grid((p->dstate + 63) / 64, (p->chunk_size + 63) / 64, p->batch * nc * p->ngroups * 2);
+    switch (p->dtype) {
+        case BIMAMBA2_F32: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+    return check_launch();
+}
+
+// =========================================================================================================
+// one wave per (b, c, h); lane i owns positions 4i..4i+3.
+//   da[q] = sum_tt da_intra[tt][q] + sum_{s<q} v_f[s] + sum_{s>q} v_b[s] + sum_{t>=q} u_f[t] + sum_{t<=q} u_b[t]
+//           + ddA_chunk_f + ddA_chunk_b
+//   ddt' = da*A + ddt_direct ; through clamp and softplus -> ddt ; dA += sum da*dt' ; ddt_bias += sum ddt
+// Partials per (b, c) go to red[(b*nc + c)*H + h] (dA) and red[B*nc*H + ...] (ddt_bias).
+// =========================================================================================================
+template <typename DT>
+__global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamba2_params p, int nc, int nqt, int nsplit) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = blockIdx.x * 4 + wave, c = blockIdx.y, b = blockIdx.z;
+    if (h >= p.nheads) return;
+    const int Q = p.chunk_size, H = p.nheads;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
+    float vf[4], vb[4], uf[4], ub[4], di[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int q = lane * 4 + e;
+        const bool ok = q < limit;
+        vf[e] = ok ? p.v_f[o + q] : 0.f;
+        vb[e] = ok ? p.v_b[o + q] : 0.f;
+        uf[e] = ok ? p.u_f[o + q] : 0.f;
+        ub[e] = ok ? p.u_b[o + q] : 0.f;
+        float s = 0.f;
+        if (ok) for (int t = 0; t < nqt; ++t) s += p.da_intra[o * nqt + (int64_t)t * Q + q];
+        di[e] = s;
+    }
+    float chunk_term = 0.f;
+    for (int s = 0; s < nsplit; ++s)
+        chunk_term += p.ddA_chunk_f[(((int64_t)b * H + h) * nc + c) * nsplit + s] + p.ddA_chunk_b[(((int64_t)b * H + h) * nc + c) * nsplit + s];
+    // lane totals and cross-lane scans
+    const float tvf = vf[0] + vf[1] + vf[2] + vf[3], tvb = vb[0] + vb[1] + vb[2] + vb[3];
+    const float tuf = uf[0] + uf[1] + uf[2] + uf[3], tub = ub[0] + ub[1] + ub[2] + ub[3];
+    const float vf_before = wave_incl_prefix(tvf, lane) - tvf;     // sum over lower lanes
+    const float ub_before = wave_incl_prefix(tub, lane) - tub;
+    const float vb_after = wave_incl_suffix(tvb, lane) - tvb;      // sum over higher lanes
+    const float uf_after = wave_incl_suffix(tuf, lane) - tuf;
+    float da[4];
+    {
+        float ex_vf = vf_before, in_ub = ub_before;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            in_ub += ub[e];
+            da[e] = di[e] + ex_vf + in_ub + chunk_term;
+            ex_vf += vf[e];
+        }
+        float ex_vb = vb_after, in_uf = uf_after;
+#pragma unroll
+        for (int e = 3; e >= 0; --e) {
+            in_uf += uf[e];
+            da[e] += ex_vb + in_uf;
+            ex_vb += vb[e];
+        }
+    }
+    const float A = p.A[h];
+    const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
+    const DT *dt = reinterpret_cast<const DT *>(p.dt) + b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
+    DT *ddt = reinterpret_cast<DT *>(p.ddt);
+    float sA = 0.f, sb = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int q = lane * 4 + e;
+        if (q < limit) {
+            const float pre = to_f(dt[(int64_t)q * p.dt_sl]) + bias;
+            float d = pre;
+            if (p.dt_softplus) d = d > 20.f ? d : log1pf(expf(d));
+            const bool clamped = d < p.dt_min || d > p.dt_max;
+            d = fminf(fmaxf(d, p.dt_min), p.dt_max);
+            float g = da[e] * A + p.ddt_direct[o + q];
+            if (clamped) g = 0.f;
+            if (p.dt_softplus && pre <= 20.f) g *= 1.f / (1.f + expf(-pre));
+            ddt[((int64_t)b * p.seqlen + (int64_t)c * Q + q) * H + h] = from_f<DT>(g);
+            sA += da[e] * d;
+            sb += g;
+        }
+    }
+    sA = wave_sum(sA);
+    sb = wave_sum(sb);
+    if (lane == 0) {
+        p.red[(int64_t)(b * nc + c) * H + h] = sA;
+        p.red[(int64_t)p.batch * nc * H + (int64_t)(b * nc + c) * H + h] = sb;
+    }
+}
+
+int launch_chunk_cumsum_bwd(const bimamba2_params *p) {
+    const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
+    const int PN = p->headdim * p->dstate;
+    const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS);
+    dim3 grid((p->nheads + 3) / 4, nc, p->batch);
+    switch (p->dt_dtype) {
+        case BIMAMBA2_F32: hipLaunchKernelGGL(chunk_cumsum_bwd_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, nsplit); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL(chunk_cumsum_bwd_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, nsplit); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL(chunk_cumsum_bwd_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, nsplit); break;
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+    int rc = check_launch();
+    if (rc) return rc;
+    const int ni = p->batch * nc;
+    rc = launch_reduce(p->red, p->dA, ni, p->nheads, 1, stream_of(p));
+    if (rc) return rc;
+    if (p->has_dt_bias && p->ddt_bias) rc = launch_reduce(p->red + (int64_t)ni * p->nheads, p->ddt_bias, ni, p->nheads, 1, stream_of(p));
+    return rc;
+}
+
+}  // namespace bm2

@@ -1,0 +1,459 @@
+// Forward kernels of the bidirectional SSD operator for gfx950.
+//   chunk_cumsum_fwd   dt -> dt', forward and reverse within-chunk cumulative sums of dt'*A
+//   bmm_chunk_fwd      CB = C . B^T per chunk and group
+//   chunk_state        per chunk and head: x^T . (B * decay * dt) for both directions (also used, with other
+//                      operands and weights, for the gradient of the chunk-entry states)
+//   state_passing_fwd  forward and reverse inter-chunk recurrences in one launch, in place
+//   chunk_scan         y = C.prev_f e^{cs_f} + C.prev_b e^{cs_b} + (CB * decay * dt) . x + D x, z gate
+//                      (its mirrored form computes dx in the backward pass)
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace bm2 {
+
+// =========================================================================================================
+// chunk cumsum: one wave per (b, c, h); lane i owns positions 4i..4i+3 of the chunk (Q <= 256)
+// =========================================================================================================
+template <typename DT>
+__global__ __launch_bounds__(NTHREADS) void chunk_cumsum_fwd_kernel(const bimamba2_params p, int nc) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = blockIdx.x * 4 + wave, c = blockIdx.y, b = blockIdx.z;
+    if (h >= p.nheads) return;
+    const int Q = p.chunk_size;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const DT *dt = reinterpret_cast<const DT *>(p.dt) + b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
+    const float A = p.A[h];
+    const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
+    float v[4], a[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int q = lane * 4 + e;
+        float d = 0.f;
+        if (q < limit) {
+            d = to_f(dt[(int64_t)q * p.dt_sl]) + bias;
+            if (p.dt_softplus) d = d > 20.f ? d : log1pf(expf(d));
+            d = fminf(fmaxf(d, p.dt_min), p.dt_max);
+        }
+        v[e] = d;
+        a[e] = d * A;
+    }
+    // forward inclusive scan
+    float pf[4], sb[4];
+    pf[0] = a[0]; pf[1] = pf[0] + a[1]; pf[2] = pf[1] + a[2]; pf[3] = pf[2] + a[3];
+    sb[3] = a[3]; sb[2] = sb[3] + a[2]; sb[1] = sb[2] + a[1]; sb[0] = sb[1] + a[0];
+    const float tot = pf[3];
+    const float incl = wave_incl_prefix(tot, lane);
+    const float before = incl - tot;
+    const float incl_s = wave_incl_suffix(tot, lane);
+    const float after = incl_s - tot;
+    const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int q = lane * 4 + e;
+        if (q < Q) {
+            p.dt_out[o + q] = v[e];
+            p.cs_f[o + q] = before + pf[e];
+            p.cs_b[o + q] = after + sb[e];
+        }
+    }
+}
+
+// =========================================================================================================
+// CB[t, s] = sum_n C[t, n] B[s, n]
+// =========================================================================================================
+template <typename T>
+__global__ __launch_bounds__(NTHREADS) void bmm_chunk_fwd_kernel(const bimamba2_params p, int nc) {
+    constexpr int LD = Mma<T>::LD;
+    __shared__ __attribute__((aligned(16))) T As[64 * LD];
+    __shared__ __attribute__((aligned(16))) T Bs[64 * LD];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int st = blockIdx.x, tt = blockIdx.y;
+    const int g = blockIdx.z % p.ngroups, bc = blockIdx.z / p.ngroups, c = bc % nc, b = bc / nc;
+    const int Q = p.chunk_size, N = p.dstate;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const T *Cp = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + ((int64_t)c * Q + tt * 64) * p.C_sl + g * p.C_sg;
+    const T *Bp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + ((int64_t)c * Q + st * 64) * p.B_sl + g * p.B_sg;
+    f32x4 acc[4] = {};
+    for (int k0 = 0; k0 < N; k0 += BK) {
+        __syncthreads();
+        tile_load_kcontig<T, T, 64>(As, Cp + k0, p.C_sl, limit - tt * 64, N - k0, Ident());
+        tile_load_kcontig<T, T, 64>(Bs, Bp + k0, p.B_sl, limit - st * 64, N - k0, Ident());
+        __syncthreads();
+        mma_tile<T, 4>(acc, As + wave * 16 * LD, Bs, lane);
+    }
+    float *out = p.CB + (int64_t)blockIdx.z * Q * Q;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = tt * 64 + wave * 16 + (lane >> 4) * 4 + i, s = st * 64 + j * 16 + (lane & 15);
+            if (t < Q && s < Q) out[(int64_t)t * Q + s] = acc[j][i];
+        }
+}
+
+// =========================================================================================================
+// chunk state (DSTATES = false):  S_f[p,n] = sum_k x[k,p] B[k,n] e^{cs_f[Q-1]-cs_f[k]} dt[k],  S_b with
+//                                 e^{cs_b[0]-cs_b[k]}
+// gradient of the chunk-entry states (DSTATES = true):  dprev_f[p,n] = sum_k dy[k,p] C[k,n] e^{cs_f[k]},
+//                                 dprev_b with e^{cs_b[k]}
+// =========================================================================================================
+template <typename T, bool DSTATES>
+__global__ __launch_bounds__(NTHREADS) void chunk_state_kernel(const bimamba2_params p, int nc) {
+    constexpr int LD = Mma<T>::LD;
+    __shared__ __attribute__((aligned(16))) T As[64 * LD];
+    __shared__ __attribute__((aligned(16))) T Bf[64 * LD];
+    __shared__ __attribute__((aligned(16))) T Bb[64 * LD];
+    __shared__ float wf[BIMAMBA2_MAX_CHUNK], wb[BIMAMBA2_MAX_CHUNK];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nt = blockIdx.x, pt = blockIdx.y;
+    const int h = blockIdx.z % p.nheads, bc = blockIdx.z / p.nheads, c = bc % nc, b = bc / nc;
+    const int g = h / (p.nheads / p.ngroups);
+    const int Q = p.chunk_size, N = p.dstate, P = p.headdim;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
+    for (int q = threadIdx.x; q < Q; q += NTHREADS) {
+        float f = 0.f, r = 0.f;
+        if (q < limit) {
+            if (DSTATES) {
+                f = __expf(p.cs_f[o + q]);
+                r = __expf(p.cs_b[o + q]);
+            } else {
+                const float d = p.dt_out[o + q];
+                f = __expf(p.cs_f[o + Q - 1] - p.cs_f[o + q]) * d;
+                r = __expf(p.cs_b[o] - p.cs_b[o + q]) * d;
+            }
+        }
+        wf[q] = f;
+        wb[q] = r;
+    }
+    const T *xp;
+    int64_t xs;
+    if (DSTATES) {
+        const T *src = reinterpret_cast<const T *>(p.has_z ? p.dout_x : p.dout);
+        if (p.has_z) { xs = (int64_t)p.nheads * P; xp = src + ((int64_t)b * p.seqlen + (int64_t)c * Q) * xs + (int64_t)h * P; }
+        else { xs = p.dout_sl; xp = src + b * p.dout_sb + (int64_t)c * Q * xs + h * p.dout_sh; }
+    } else {
+        xs = p.x_sl;
+        xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * xs + h * p.x_sh;
+    }
+    xp += pt * 64;
+    const T *bp;
+    int64_t bs;
+    if (DSTATES) { bs = p.C_sl; bp = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * bs + g * p.C_sg; }
+    else { bs = p.B_sl; bp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * bs + g * p.B_sg; }
+    bp += nt * 64;
+    f32x4 accf[4] = {}, accb[4] = {};
+    for (int k0 = 0; k0 < limit; k0 += BK) {
+        __syncthreads();
+        tile_load_rcontig<T, T, 64>(As, xp + k0 * xs, xs, P - pt * 64, limit - k0, Ident());
+        tile_load_rcontig2<T, T, 64>(
+            Bf, Bb, bp + k0 * bs, bs, N - nt * 64, limit - k0,
+            [&](int, int k, float v) { return v * wf[k0 + k]; }, [&](int, int k, float v) { return v * wb[k0 + k]; });
+        __syncthreads();
+        mma_tile<T, 4>(accf, As + wave * 16 * LD, Bf, lane);
+        mma_tile<T, 4>(accb, As + wave * 16 * LD, Bb, lane);
+    }
+    float *of = (DSTATES ? p.dstates_f : p.states_f) + (int64_t)blockIdx.z * P * N;
+    float *ob = (DSTATES ? p.dstates_b : p.states_b) + (int64_t)blockIdx.z * P * N;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int pp = pt * 64 + wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
+            if (pp < P && n < N) {
+                of[(int64_t)pp * N + n] = accf[j][i];
+                ob[(int64_t)pp * N + n] = accb[j][i];
+            }
+        }
+}
+
+// =========================================================================================================
+// inter-chunk recurrences, both directions, in place:
+//   forward : prev_f[0] = 0, prev_f[c+1] = e^{tot_c} prev_f[c] + S_f[c]   (final_f = value after the last chunk)
+//   reverse : prev_b[nc-1] = 0, prev_b[c-1] = e^{tot_c} prev_b[c] + S_b[c] (final_b = value after chunk 0)
+// One thread owns one (b, h, p, n) element; the chunk loop is unrolled by 8 so that 8 loads are in flight.
+// =========================================================================================================
+__global__ __launch_bounds__(NTHREADS) void state_passing_fwd_kernel(const bimamba2_params p, int nc) {
+    const int PN = p.headdim * p.dstate;
+    const int e = blockIdx.x * NTHREADS + threadIdx.x;
+    const int h = blockIdx.y, b = blockIdx.z;
+    if (e >= PN) return;
+    const int Q = p.chunk_size;
+    const float *csf = p.cs_f + ((int64_t)b * p.nheads + h) * nc * Q;
+    const float *csb = p.cs_b + ((int64_t)b * p.nheads + h) * nc * Q;
+    const int64_t cstride = (int64_t)p.nheads * PN;
+    float *sf = p.states_f + ((int64_t)b * nc * p.nheads + h) * PN + e;
+    float *sb = p.states_b + ((int64_t)b * nc * p.nheads + h) * PN + e;
+    float s = 0.f;
+    for (int c0 = 0; c0 < nc; c0 += 8) {
+        float v[8], d[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (c0 + i < nc) {
+                v[i] = sf[(c0 + i) * cstride];
+                d[i] = __expf(csf[(int64_t)(c0 + i) * Q + Q - 1]);
+            }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (c0 + i < nc) {
+                sf[(c0 + i) * cstride] = s;
+                s = d[i] * s + v[i];
+            }
+    }
+    if (p.final_f) p.final_f[((int64_t)b * p.nheads + h) * PN + e] = s;
+    s = 0.f;
+    for (int c0 = nc - 1; c0 >= 0; c0 -= 8) {
+        float v[8], d[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (c0 - i >= 0) {
+                v[i] = sb[(c0 - i) * cstride];
+                d[i] = __expf(csb[(int64_t)(c0 - i) * Q]);
+            }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (c0 - i >= 0) {
+                sb[(c0 - i) * cstride] = s;
+                s = d[i] * s + v[i];
+            }
+    }
+    if (p.final_b) p.final_b[((int64_t)b * p.nheads + h) * PN + e] = s;
+}
+
+// =========================================================================================================
+// chunk scan (BWD = false), rows r = output positions t:
+//   acc[r,p] = e^{cs_f[r]} C_r.prev_f[p,:] + e^{cs_b[r]} C_r.prev_b[p,:]
+//            + sum_k CB[r,k] (1[k<=r] e^{cs_f[r]-cs_f[k]} + 1[k>=r] e^{cs_b[r]-cs_b[k]}) dt[k] x[k,p]
+//   out_x = acc + D x[r,p];  out = out_x * silu(z)
+// its mirror (BWD = true), rows r = input positions s:
+//   acc[r,p] = e^{cs_f[Q-1]-cs_f[r]} B_r.dS_f[p,:] + e^{cs_b[0]-cs_b[r]} B_r.dS_b[p,:]
+//            + sum_k CB[k,r] (1[k>=r] e^{cs_f[k]-cs_f[r]} + 1[k<=r] e^{cs_b[k]-cs_b[r]}) dy[k,p]
+//   dx = acc dt[r] + D dy[r,p];  ddt_direct[r] = sum_p acc x[r,p];  dD partial = sum_r dy x
+// =========================================================================================================
+template <typename T, bool BWD>
+__global__ __launch_bounds__(NTHREADS) void chunk_scan_kernel(const bimamba2_params p, int nc) {
+    constexpr int LD = Mma<T>::LD;
+    __shared__ __attribute__((aligned(16))) T As[64 * LD];
+    __shared__ __attribute__((aligned(16))) T B1[64 * LD];
+    __shared__ __attribute__((aligned(16))) T B2[64 * LD];
+    __shared__ float csf[BIMAMBA2_MAX_CHUNK], csb[BIMAMBA2_MAX_CHUNK], dts[BIMAMBA2_MAX_CHUNK];
+    __shared__ float red[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pt = blockIdx.x, rt = blockIdx.y;
+    const int h = blockIdx.z % p.nheads, bc = blockIdx.z / p.nheads, c = bc % nc, b = bc / nc;
+    const int g = h / (p.nheads / p.ngroups);
+    const int Q = p.chunk_size, N = p.dstate, P = p.headdim;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
+    for (int q = threadIdx.x; q < Q; q += NTHREADS) {
+        csf[q] = p.cs_f[o + q];
+        csb[q] = p.cs_b[o + q];
+        dts[q] = p.dt_out[o + q];
+    }
+    // ---- part 1: contribution of the states, K = dstate ----
+    const T *ap;
+    int64_t as;
+    if (BWD) { as = p.B_sl; ap = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + ((int64_t)c * Q + rt * 64) * as + g * p.B_sg; }
+    else { as = p.C_sl; ap = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + ((int64_t)c * Q + rt * 64) * as + g * p.C_sg; }
+    const float *s1 = (BWD ? p.dstates_f : p.states_f) + (int64_t)blockIdx.z * P * N + (int64_t)pt * 64 * N;
+    const float *s2 = (BWD ? p.dstates_b : p.states_b) + (int64_t)blockIdx.z * P * N + (int64_t)pt * 64 * N;
+    f32x4 acc[4] = {};
+    {
+        f32x4 accf[4] = {}, accb[4] = {};
+        for (int k0 = 0; k0 < N; k0 += BK) {
+            __syncthreads();
+            tile_load_kcontig<T, T, 64>(As, ap + k0, as, limit - rt * 64, N - k0, Ident());
+            tile_load_kcontig<T, float, 64>(B1, s1 + k0, N, P - pt * 64, N - k0, Ident());
+            tile_load_kcontig<T, float, 64>(B2, s2 + k0, N, P - pt * 64, N - k0, Ident());
+            __syncthreads();
+            mma_tile<T, 4>(accf, As + wave * 16 * LD, B1, lane);
+            mma_tile<T, 4>(accb, As + wave * 16 * LD, B2, lane);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = rt * 64 + wave * 16 + (lane >> 4) * 4 + i;
+            float sf = 0.f, sb = 0.f;
+            if (r < limit) {
+                sf = BWD ? __expf(csf[Q - 1] - csf[r]) : __expf(csf[r]);
+                sb = BWD ? __expf(csb[0] - csb[r]) : __expf(csb[r]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j][i] = accf[j][i] * sf + accb[j][i] * sb;
+        }
+    }
+    // ---- part 2: inside the chunk, K = chunk positions ----
+    const float *cb = p.CB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    const T *kp;
+    int64_t ks;
+    if (!BWD) { ks = p.x_sl; kp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * ks + h * p.x_sh; }
+    else if (p.has_z) { ks = (int64_t)p.nheads * P; kp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * ks + (int64_t)h * P; }
+    else { ks = p.dout_sl; kp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * ks + h * p.dout_sh; }
+    const T *kp_tile = kp + pt * 64;
+    const int r0 = rt * 64;
+    for (int k0 = 0; k0 < limit; k0 += BK) {
+        __syncthreads();
+        if (!BWD) {
+            tile_load_kcontig<T, float, 64>(As, cb + (int64_t)r0 * Q + k0, Q, Q - r0, Q - k0, [&](int rl, int kl, float v) {
+                const int r = r0 + rl, k = k0 + kl;
+                if (r >= limit || k >= limit) return 0.f;
+                float m = 0.f;
+                if (k <= r) m += __expf(csf[r] - csf[k]);
+                if (k >= r) m += __expf(csb[r] - csb[k]);
+                return v * m * dts[k];
+            });
+        } else {
+            tile_load_rcontig<T, float, 64>(As, cb + (int64_t)k0 * Q + r0, Q, Q - r0, Q - k0, [&](int rl, int kl, float v) {
+                const int r = r0 + rl, k = k0 + kl;
+                if (r >= limit || k >= limit) return 0.f;
+                float m = 0.f;
+                if (k >= r) m += __expf(csf[k] - csf[r]);
+                if (k <= r) m += __expf(csb[k] - csb[r]);
+                return v * m;
+            });
+        }
+        tile_load_rcontig<T, T, 64>(B1, kp_tile + k0 * ks, ks, P - pt * 64, limit - k0, Ident());
+        __syncthreads();
+        mma_tile<T, 4>(acc, As + wave * 16 * LD, B1, lane);
+    }
+    // ---- epilogue ----
+    const int col0 = pt * 64 + (lane & 15);
+    if (!BWD) {
+        T *outp = reinterpret_cast<T *>(p.out);
+        T *outx = reinterpret_cast<T *>(p.out_x);
+        const T *xrow = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh;
+        const T *zrow = p.has_z ? reinterpret_cast<const T *>(p.z) + b * p.z_sb + (int64_t)c * Q * p.z_sl + h * p.z_sh : nullptr;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = r0 + wave * 16 + (lane >> 4) * 4 + i;
+            if (r >= limit) continue;
+            const int64_t orow = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.nheads + h) * P;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = col0 + j * 16;
+                if (col >= P) continue;
+                float v = acc[j][i];
+                if (p.has_D) v += (p.D_has_hdim ? p.D[h * P + col] : p.D[h]) * to_f(xrow[(int64_t)r * p.x_sl + col]);
+                if (p.has_z) {
+                    if (outx) outx[orow + col] = from_f<T>(v);
+                    v *= silu_f(to_f(zrow[(int64_t)r * p.z_sl + col]));
+                }
+                outp[orow + col] = from_f<T>(v);
+            }
+        }
+    } else {
+        T *dxp = reinterpret_cast<T *>(p.dx);
+        const T *xrow = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh;
+        float dsum[4] = {0.f, 0.f, 0.f, 0.f};   // per column tile j: sum over this lane's rows of dy*x
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = r0 + wave * 16 + (lane >> 4) * 4 + i;
+            const bool rok = r < limit;
+            const float dtr = rok ? dts[r] : 0.f;
+            const int64_t orow = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.nheads + h) * P;
+            float rs = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = col0 + j * 16;
+                if (rok && col < P) {
+                    const float xv = to_f(xrow[(int64_t)r * p.x_sl + col]);
+                    const float a = acc[j][i];
+                    rs += a * xv;
+                    float v = a * dtr;
+                    if (p.has_D) {
+                        const float dy = to_f(kp[(int64_t)r * ks + col]);
+                        v += (p.D_has_hdim ? p.D[h * P + col] : p.D[h]) * dy;
+                        dsum[j] += dy * xv;
+                    }
+                    dxp[orow + col] = from_f<T>(v);
+                }
+            }
+            rs = row16_sum(rs);
+            if (rok && (lane & 15) == 0) {
+                // with more than one headdim tile the partial row sums are added atomically
+                if (gridDim.x == 1) p.ddt_direct[o + r] = rs;
+                else atomicAdd(p.ddt_direct + o + r, rs);
+            }
+        }
+        if (p.has_D) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v = dsum[j];
+                v += __shfl_xor(v, 16, 64);
+                v += __shfl_xor(v, 32, 64);
+                if (lane < 16) red[wave][j * 16 + lane] = v;
+            }
+            __syncthreads();
+            if (threadIdx.x < 64) {
+                const int col = pt * 64 + threadIdx.x;
+                if (col < P) {
+                    const float v = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
+                    // partials: [(b*nc + c)*RT + rt][h][P]
+                    p.red[(((int64_t)(b * nc + c) * gridDim.y + rt) * p.nheads + h) * P + col] = v;
+                }
+            }
+        }
+    }
+}
+
+// =========================================================================================================
+// launchers
+// =========================================================================================================
+static inline int nchunks(const bimamba2_params *p) { return (p->seqlen + p->chunk_size - 1) / p->chunk_size; }
+static inline hipStream_t stream_of(const bimamba2_params *p) { return reinterpret_cast<hipStream_t>(p->stream); }
+
+int launch_chunk_cumsum_fwd(const bimamba2_params *p) {
+    const int nc = nchunks(p);
+    dim3 grid((p->nheads + 3) / 4, nc, p->batch);
+    switch (p->dt_dtype) {
+        case BIMAMBA2_F32: hipLaunchKernelGGL(chunk_cumsum_fwd_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL(chunk_cumsum_fwd_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL(chunk_cumsum_fwd_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+    return check_launch();
+}
+
+#define BM2_DISPATCH_T(p, KERNEL, grid, ...)                                                                          \
+    switch ((p)->dtype) {                                                                                             \
+        case BIMAMBA2_F32: hipLaunchKernelGGL((KERNEL<float, ##__VA_ARGS__>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;   \
+        case BIMAMBA2_BF16: hipLaunchKernelGGL((KERNEL<bf16_t, ##__VA_ARGS__>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break; \
+        case BIMAMBA2_F16: hipLaunchKernelGGL((KERNEL<f16_t, ##__VA_ARGS__>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;   \
+        default: return BIMAMBA2_EUNSUPPORTED;                                                                        \
+    }
+
+int launch_bmm_chunk_fwd(const bimamba2_params *p) {
+    const int nc = nchunks(p), qt = (p->chunk_size + 63) / 64;
+    dim3 grid(qt, qt, p->batch * nc * p->ngroups);
+    switch (p->dtype) {
+        case BIMAMBA2_F32: hipLaunchKernelGGL(bmm_chunk_fwd_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL(bmm_chunk_fwd_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL(bmm_chunk_fwd_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+    return check_launch();
+}
+
+int launch_chunk_state(const bimamba2_params *p, bool dstates) {
+    const int nc = nchunks(p);
+    dim3 grid((p->dstate + 63) / 64, (p->headdim + 63) / 64, p->batch * nc * p->nheads);
+    if (dstates) { BM2_DISPATCH_T(p, chunk_state_kernel, grid, true) }
+    else { BM2_DISPATCH_T(p, chunk_state_kernel, grid, false) }
+    return check_launch();
+}
+
+int launch_state_passing_fwd(const bimamba2_params *p) {
+    const int nc = nchunks(p), PN = p->headdim * p->dstate;
+    dim3 grid((PN + NTHREADS - 1) / NTHREADS, p->nheads, p->batch);
+    hipLaunchKernelGGL(state_passing_fwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    return check_launch();
+}
+
+int launch_chunk_scan(const bimamba2_params *p, bool bwd) {
+    const int nc = nchunks(p);
+    dim3 grid((p->headdim + 63) / 64, (p->chunk_size + 63) / 64, p->batch * nc * p->nheads);
+    if (bwd) { BM2_DISPATCH_T(p, chunk_scan_kernel, grid, true) }
+    else { BM2_DISPATCH_T(p, chunk_scan_kernel, grid, false) }
+    return check_launch();
+}
+
+}  // namespace bm2

@@ -1,0 +1,27 @@
+// Host-side declarations shared by the kernel files and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "../../include/bimamba2.h"
+
+namespace bm2 {
+
+static inline int check_launch() { return hipGetLastError() == hipSuccess ? BIMAMBA2_OK : BIMAMBA2_ELAUNCH; }
+
+int launch_chunk_cumsum_fwd(const bimamba2_params *p);
+int launch_bmm_chunk_fwd(const bimamba2_params *p);
+int launch_chunk_state(const bimamba2_params *p, bool dstates);
+int launch_state_passing_fwd(const bimamba2_params *p);
+int launch_chunk_scan(const bimamba2_params *p, bool bwd);
+
+int launch_bwd_dz(const bimamba2_params *p);
+int launch_state_passing_bwd(const bimamba2_params *p);
+int launch_bwd_dbdc(const bimamba2_params *p, bool is_db);
+int launch_bwd_dcb(const bimamba2_params *p);
+int launch_bmm_chunk_bwd(const bimamba2_params *p);
+int launch_chunk_cumsum_bwd(const bimamba2_params *p);
+int launch_fill(float *ptr, size_t n, float value, hipStream_t stream);
+// out[j] = sum_{i<ni} sum_{k<nk} in[(i*nj + j)*nk + k]
+int launch_reduce(const float *in, float *out, int ni, int nj, int nk, hipStream_t stream);
+
+}  // namespace bm2

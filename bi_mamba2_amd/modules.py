@@ -1,0 +1,111 @@
+"""``BiMamba2`` layer around the bidirectional SSD operator.
+
+Same constructor keywords, parameter names/shapes (so state_dicts interchange) and forward math as the
+reference layer (src/ssd/modules.py:17-187): in_proj -> split [z | xBC | dt] -> softplus(dt + dt_bias) ->
+non-causal depthwise conv1d + SiLU -> split x, B, C -> bidirectional SSD with D -> gated RMSNorm(y, z) ->
+out_proj.  Parameters are created in the reference's order, so a seeded construction draws the same values.
+The projections, the convolution and the norm are ordinary torch ops; the SSD is the HIP operator.
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .ops import bimamba_chunk_scan_combined
+
+
+class RMSNormGated(nn.Module):
+    """RMSNorm over the last dim with an optional silu(z) gate, norm first then gate by default (the math of
+    the reference's ``rms_norm_ref``, src/ssd/bi/layernorm_gated.py:18-39), computed in float32."""
+
+    def __init__(self, hidden_size, eps=1e-5, group_size=None, norm_before_gate=True, device=None, dtype=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(hidden_size, device=device, dtype=dtype))
+        self.register_parameter("bias", None)
+        self.group_size = group_size
+        self.norm_before_gate = norm_before_gate
+
+    def forward(self, x, z=None):
+        dtype = x.dtype
+        xf = x.float()
+        zf = z.float() if z is not None else None
+        if zf is not None and not self.norm_before_gate:
+            xf = xf * F.silu(zf)
+        if self.group_size is None:
+            y = xf * torch.rsqrt(xf.square().mean(-1, keepdim=True) + self.eps)
+        else:
+            xg = xf.unflatten(-1, (-1, self.group_size))
+            y = (xg * torch.rsqrt(xg.square().mean(-1, keepdim=True) + self.eps)).flatten(-2)
+        y = y * self.weight.float()
+        if zf is not None and self.norm_before_gate:
+            y = y * F.silu(zf)
+        return y.to(dtype)
+
+
+class BiMamba2(nn.Module):
+    """Bidirectional Mamba-2 mixer layer; ``forward(u)`` maps (batch, seqlen, d_model) to the same shape."""
+
+    def __init__(self, d_model, d_state=64, d_conv=7, conv_init=None, expand=2, headdim=64, ngroups=1,
+                 dt_min=0.001, dt_max=0.1, dt_init_floor=1e-4, dt_limit=(0.0, float("inf")),
+                 learnable_init_states=False, activation="swish", bias=False, conv_bias=True, chunk_size=256,
+                 use_mem_eff_path=False, layer_idx=None, device=None, dtype=None):
+        super().__init__()
+        fk = {"device": device, "dtype": dtype}
+        assert not use_mem_eff_path, "Mem Eff Path is not implemented yet."
+        assert activation in ("silu", "swish")
+        self.d_model, self.d_state, self.d_conv, self.conv_init = d_model, d_state, d_conv, conv_init
+        self.expand, self.headdim, self.ngroups = expand, headdim, ngroups
+        self.d_inner = expand * d_model
+        assert self.d_inner % headdim == 0
+        self.nheads = self.d_inner // headdim
+        self.dt_limit = dt_limit
+        self.learnable_init_states = learnable_init_states
+        self.activation = activation
+        self.chunk_size = chunk_size
+        self.use_mem_eff_path = use_mem_eff_path
+        self.layer_idx = layer_idx
+
+        bc = 2 * ngroups * d_state
+        # in_proj output order: [z, x, B, C, dt]
+        self.in_proj = nn.Linear(d_model, 2 * self.d_inner + bc + self.nheads, bias=bias, **fk)
+        conv_dim = self.d_inner + bc
+        self.conv1d = nn.Conv1d(conv_dim, conv_dim, kernel_size=d_conv, groups=conv_dim, padding=d_conv // 2,
+                                bias=conv_bias, **fk)
+        if conv_init is not None:
+            nn.init.uniform_(self.conv1d.weight, -conv_init, conv_init)
+        if learnable_init_states:   # kept for state_dict compatibility; the bidirectional path has no initial state
+            self.init_states = nn.Parameter(torch.zeros(self.nheads, headdim, d_state, **fk))
+            self.init_states._no_weight_decay = True
+        self.act = nn.SiLU()
+
+        # dt_bias = softplus^-1 of a log-uniform sample in [dt_min, dt_max]
+        dt0 = torch.exp(torch.rand(self.nheads, **fk) * (math.log(dt_max) - math.log(dt_min)) + math.log(dt_min))
+        dt0 = torch.clamp(dt0, min=dt_init_floor)
+        self.dt_bias = nn.Parameter(dt0 + torch.log(-torch.expm1(-dt0)))
+        self.dt_bias._no_weight_decay = True
+
+        self.A_log = nn.Parameter(torch.log(torch.ones(self.nheads, dtype=torch.float32, device=device)).to(dtype=dtype))
+        self.A_log._no_weight_decay = True
+        self.D = nn.Parameter(torch.ones(self.nheads, device=device))
+        self.D._no_weight_decay = True
+        self.fc_D = nn.Linear(self.d_inner, self.nheads, bias=False, **fk)   # present in the reference, unused there too
+        self.norm = RMSNormGated(self.d_inner, eps=1e-5, norm_before_gate=True, **fk)
+        self.out_proj = nn.Linear(self.d_inner, d_model, bias=bias, **fk)
+
+    def forward(self, u):
+        bc = self.ngroups * self.d_state
+        zxbcdt = self.in_proj(u)
+        A = -torch.exp(self.A_log.float())
+        z, xBC, dt = torch.split(zxbcdt, [self.d_inner, self.d_inner + 2 * bc, self.nheads], dim=-1)
+        dt = F.softplus(dt + self.dt_bias)
+        xBC = self.act(self.conv1d(xBC.transpose(1, 2)).transpose(1, 2))
+        x, B, C = torch.split(xBC, [self.d_inner, bc, bc], dim=-1)
+        kw = {} if tuple(self.dt_limit) == (0.0, float("inf")) else {"dt_limit": tuple(self.dt_limit)}
+        y = bimamba_chunk_scan_combined(
+            x.unflatten(-1, (self.nheads, self.headdim)), dt, A,
+            B.unflatten(-1, (self.ngroups, self.d_state)), C.unflatten(-1, (self.ngroups, self.d_state)),
+            chunk_size=self.chunk_size, D=self.D, z=None, **kw)
+        y = self.norm(y.flatten(-2), z)
+        return self.out_proj(y)

@@ -1,0 +1,492 @@
+"""Host side of the bidirectional SSD operator: the functions of the reference's ``ssd.bi.ssd_combined`` and of its
+stage wrappers, with the same names, argument meaning and error behaviour, on top of the C ABI of
+libbimamba2_hip.so (include/bimamba2.h).  PyTorch is used for device memory and streams only; every device
+computation is a hand-written HIP kernel.  There is no CPU path: tensors must live on a GPU.
+
+Reference interface mirrored here (paths relative to the reference's root):
+  bimamba_chunk_scan_combined / MambaChunkScanCombinedFn      src/ssd/bi/ssd_combined.py:555-593
+  _mamba_chunk_scan_combined_fwd / _bwd                       src/ssd/bi/ssd_combined.py:297-475
+  _chunk_cumsum_fwd, _chunk_state_fwd, _chunk_state_bwd_db,
+  _chunk_cumsum_bwd                                           src/ssd/bi/ssd_chunk_state.py:699-894
+  _state_passing_fwd / _bwd                                   src/ssd/bi/ssd_state_passing.py:190-248
+  _bmm_chunk_fwd / _bwd                                       src/ssd/bi/ssd_bmm.py:163-262
+  _chunk_scan_fwd, _chunk_scan_bwd_dz/_dstates/_dC/_dcb       src/ssd/bi/ssd_chunk_scan.py:1638-1909
+"""
+import math
+
+import torch
+
+from . import _lib
+from ._lib import Params
+
+_DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+_INF = float("inf")
+
+
+def _require_gpu(t, name):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} is on {t.device}: the bidirectional SSD kernels run on an AMD GPU only "
+                           "(there is no CPU fallback)")
+
+
+def _rowmajor_last(t):
+    """Last dim must be contiguous for the kernels; anything else is copied."""
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _f32c(t):
+    return t.detach().to(torch.float32).contiguous()
+
+
+class _Call:
+    """Collects tensors into a ``bimamba2_params`` and keeps them alive until the launch has been enqueued."""
+
+    def __init__(self, batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, dtype, device,
+                 dt_dtype=torch.float32, dt_softplus=False, dt_limit=(0.0, _INF)):
+        if dtype not in _DT:
+            raise ValueError(f"unsupported dtype {dtype} (need float32, bfloat16 or float16)")
+        if dt_dtype not in _DT:
+            raise ValueError(f"unsupported dt dtype {dt_dtype}")
+        p = Params()
+        p.batch, p.seqlen, p.nheads, p.headdim = batch, seqlen, nheads, headdim
+        p.ngroups, p.dstate, p.chunk_size = ngroups, dstate, chunk_size
+        p.dtype, p.dt_dtype = _DT[dtype], _DT[dt_dtype]
+        p.dt_softplus = int(bool(dt_softplus))
+        p.dt_min, p.dt_max = float(dt_limit[0]), float(dt_limit[1])
+        self.p, self.keep, self.device, self.dtype, self.dt_dtype = p, [], device, dtype, dt_dtype
+        self.nchunks = (seqlen + chunk_size - 1) // chunk_size
+
+    # ---- raw pointer fields -------------------------------------------------------------------------
+    def put(self, field, t, dtype=None):
+        if t is None:
+            return None
+        _require_gpu(t, field)
+        if dtype is not None and t.dtype != dtype:
+            raise TypeError(f"{field} must be {dtype}, got {t.dtype}")
+        if not t.is_contiguous():
+            raise ValueError(f"{field} must be contiguous")
+        self.keep.append(t)
+        setattr(self.p, field, t.data_ptr())
+        return t
+
+    def new(self, field, shape, dtype=torch.float32):
+        t = torch.empty(shape, device=self.device, dtype=dtype)
+        return self.put(field, t)
+
+    # ---- strided inputs -----------------------------------------------------------------------------
+    def _strided(self, field, prefix, t, dtype):
+        _require_gpu(t, field)
+        if t.dtype != dtype:
+            t = t.to(dtype)
+        t = _rowmajor_last(t)
+        self.keep.append(t)
+        setattr(self.p, field, t.data_ptr())
+        for name, s in zip(prefix, t.stride()[:3]):
+            setattr(self.p, name, s)
+        return t
+
+    def set_x(self, x):
+        return self._strided("x", ("x_sb", "x_sl", "x_sh"), x, self.dtype)
+
+    def set_z(self, z):
+        if z is None:
+            return None
+        self.p.has_z = 1
+        return self._strided("z", ("z_sb", "z_sl", "z_sh"), z, self.dtype)
+
+    def set_dout(self, dout):
+        return self._strided("dout", ("dout_sb", "dout_sl", "dout_sh"), dout, self.dtype)
+
+    def set_B(self, B):
+        return self._strided("Bm", ("B_sb", "B_sl", "B_sg"), B, self.dtype)
+
+    def set_C(self, C):
+        return self._strided("Cm", ("C_sb", "C_sl", "C_sg"), C, self.dtype)
+
+    def set_dt(self, dt):
+        _require_gpu(dt, "dt")
+        self.keep.append(dt)
+        self.p.dt = dt.data_ptr()
+        self.p.dt_sb, self.p.dt_sl, self.p.dt_sh = dt.stride()
+        return dt
+
+    def set_A(self, A):
+        return self.put("A", _f32c(A))
+
+    def set_D(self, D):
+        if D is None:
+            return None
+        self.p.has_D = 1
+        self.p.D_has_hdim = int(D.dim() == 2)
+        return self.put("D", _f32c(D))
+
+    def set_dt_bias(self, dt_bias):
+        if dt_bias is None:
+            return None
+        self.p.has_dt_bias = 1
+        return self.put("dt_bias", _f32c(dt_bias))
+
+    def workspace(self, is_bwd):
+        n = _lib.load().bimamba2_workspace_bytes(self.p, int(is_bwd))
+        ws = torch.empty(max(int(n), 1), device=self.device, dtype=torch.uint8)
+        self.keep.append(ws)
+        self.p.workspace = ws.data_ptr()
+        self.p.workspace_bytes = ws.numel()
+
+    def run(self, entry):
+        with torch.cuda.device(self.device):
+            self.p.stream = torch.cuda.current_stream().cuda_stream
+            _lib.call(entry, self.p)
+
+
+def _check_chunk(chunk_size):
+    assert chunk_size >= 32, "chunk_size must be at least 32 (as in the reference) and at most 256"
+
+
+def _bhcq(c):
+    return (c.p.batch, c.p.nheads, c.nchunks, c.p.chunk_size)
+
+
+# =============================================================================================================
+# stage wrappers
+# =============================================================================================================
+def _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_limit=(0.0, _INF)):
+    """-> dA_cumsum_f, dA_cumsum_b, dt_out, each (batch, nheads, nchunks, chunk_size) float32."""
+    batch, seqlen, nheads = dt.shape
+    assert A.shape == (nheads,)
+    if dt_bias is not None:
+        assert dt_bias.shape == (nheads,)
+    c = _Call(batch, seqlen, nheads, 1, 1, 1, chunk_size, torch.float32, dt.device, dt.dtype, dt_softplus, dt_limit)
+    c.set_dt(dt); c.set_A(A); c.set_dt_bias(dt_bias)
+    dt_out = c.new("dt_out", _bhcq(c)); cs_f = c.new("cs_f", _bhcq(c)); cs_b = c.new("cs_b", _bhcq(c))
+    c.run("bimamba2_chunk_cumsum_fwd")
+    return cs_f, cs_b, dt_out
+
+
+def _bmm_chunk_fwd(C, B, chunk_size, output_dtype=torch.float32):
+    """CB (batch, nchunks, ngroups, chunk_size, chunk_size); kept in float32 (the reference's choice too)."""
+    batch, seqlen, ngroups, dstate = B.shape
+    assert C.shape == B.shape
+    c = _Call(batch, seqlen, ngroups, 1, ngroups, dstate, chunk_size, C.dtype, C.device)
+    c.set_B(B); c.set_C(C)
+    CB = c.new("CB", (batch, c.nchunks, ngroups, chunk_size, chunk_size))
+    c.run("bimamba2_bmm_chunk_fwd")
+    return CB if output_dtype in (None, torch.float32) else CB.to(output_dtype)
+
+
+def _chunk_state_fwd(B, x, dt, dA_cumsum_f, dA_cumsum_b, states_in_fp32=True):
+    """-> states_f, states_b (batch, nchunks, nheads, headdim, dstate) float32."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert dt.shape == (batch, nheads, nchunks, chunk_size)
+    assert dA_cumsum_f.shape == dt.shape and dA_cumsum_b.shape == dt.shape
+    c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, x.dtype, x.device)
+    c.set_x(x); c.set_B(B)
+    c.put("dt_out", dt, torch.float32); c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    shape = (batch, nchunks, nheads, headdim, dstate)
+    sf = c.new("states_f", shape); sb = c.new("states_b", shape)
+    c.run("bimamba2_chunk_state_fwd")
+    return sf, sb
+
+
+def _state_passing_fwd(states_f, states_b, dA_cumsum_f, dA_cumsum_b, return_final_states=True):
+    """Both inter-chunk recurrences in one launch.  states_* are (batch, nchunks, nheads, headdim, dstate) float32
+    chunk states; returns the states entering each chunk (new tensors) and the two final states."""
+    batch, nchunks, nheads, headdim, dstate = states_f.shape
+    chunk_size = dA_cumsum_f.shape[-1]
+    assert states_b.shape == states_f.shape
+    assert dA_cumsum_f.shape == (batch, nheads, nchunks, chunk_size) and dA_cumsum_b.shape == dA_cumsum_f.shape
+    c = _Call(batch, nchunks * chunk_size, nheads, headdim, 1, dstate, chunk_size, torch.float32, states_f.device)
+    c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    pf = c.put("states_f", states_f.clone(), torch.float32); pb = c.put("states_b", states_b.clone(), torch.float32)
+    ff = fb = None
+    if return_final_states:
+        ff = c.new("final_f", (batch, nheads, headdim, dstate)); fb = c.new("final_b", (batch, nheads, headdim, dstate))
+    c.run("bimamba2_state_passing_fwd")
+    return pf, pb, ff, fb
+
+
+def _chunk_scan_fwd(CB, x, dt, dA_cumsum_f, dA_cumsum_b, C, states_f, states_b, D=None, z=None):
+    """-> out, out_x (out_x is None without z)."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = C.shape
+    assert nheads % ngroups == 0
+    assert C.shape == (batch, seqlen, ngroups, dstate)
+    assert CB.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    if z is not None:
+        assert z.shape == x.shape
+    if D is not None:
+        assert D.shape == (nheads, headdim) or D.shape == (nheads,)
+    assert dt.shape == (batch, nheads, nchunks, chunk_size)
+    assert states_f.shape == (batch, nchunks, nheads, headdim, dstate) and states_b.shape == states_f.shape
+    c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, x.dtype, x.device)
+    c.set_x(x); c.set_C(C); c.set_z(z); c.set_D(D)
+    c.put("CB", CB, torch.float32); c.put("dt_out", dt, torch.float32)
+    c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    c.put("states_f", states_f, torch.float32); c.put("states_b", states_b, torch.float32)
+    out = c.new("out", x.shape, x.dtype)
+    out_x = c.new("out_x", x.shape, x.dtype) if z is not None else None
+    c.run("bimamba2_chunk_scan_fwd")
+    return out, out_x
+
+
+def _chunk_scan_bwd_dz(x, z, out_x, dout, chunk_size=None, D=None):
+    """-> dz, dout_x = dout * silu(z)."""
+    batch, seqlen, nheads, headdim = x.shape
+    assert z.shape == x.shape and out_x.shape == x.shape and dout.shape == x.shape
+    c = _Call(batch, seqlen, nheads, headdim, 1, 1, chunk_size or 64, x.dtype, x.device)
+    c.set_z(z); c.set_dout(dout)
+    c.put("out_x", out_x.contiguous(), x.dtype)
+    dz = c.new("dz", x.shape, x.dtype); dout_x = c.new("dout_x", x.shape, x.dtype)
+    c.run("bimamba2_chunk_scan_bwd_dz")
+    return dz, dout_x
+
+
+def _chunk_scan_bwd_dstates(C, dA_cumsum_f, dA_cumsum_b, dout, headdim=None):
+    """-> gradient w.r.t. the states entering each chunk, both directions, float32."""
+    batch, seqlen, nheads, hd = dout.shape
+    _, _, nchunks, chunk_size = dA_cumsum_f.shape
+    _, _, ngroups, dstate = C.shape
+    c = _Call(batch, seqlen, nheads, hd, ngroups, dstate, chunk_size, dout.dtype, dout.device)
+    c.set_dout(dout); c.set_C(C)
+    c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    shape = (batch, nchunks, nheads, hd, dstate)
+    df = c.new("dstates_f", shape); db = c.new("dstates_b", shape)
+    c.run("bimamba2_chunk_scan_bwd_dstates")
+    return df, db
+
+
+def _state_passing_bwd(states_f, states_b, dA_cumsum_f, dA_cumsum_b, dstates_f, dstates_b):
+    """states_*: states entering each chunk; dstates_*: gradient w.r.t. them.
+    -> gradient w.r.t. each chunk's own state (both directions) and ddA_chunk_f/b (batch, nheads, nchunks)."""
+    batch, nchunks, nheads, headdim, dstate = states_f.shape
+    chunk_size = dA_cumsum_f.shape[-1]
+    c = _Call(batch, nchunks * chunk_size, nheads, headdim, 1, dstate, chunk_size, torch.float32, states_f.device)
+    c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    c.put("states_f", states_f, torch.float32); c.put("states_b", states_b, torch.float32)
+    gf = c.put("dstates_f", dstates_f.clone(), torch.float32); gb = c.put("dstates_b", dstates_b.clone(), torch.float32)
+    nsplit = (headdim * dstate + 1023) // 1024
+    af = c.new("ddA_chunk_f", (batch, nheads, nchunks, nsplit)); ab = c.new("ddA_chunk_b", (batch, nheads, nchunks, nsplit))
+    c.run("bimamba2_state_passing_bwd")
+    return gf, gb, af.sum(-1), ab.sum(-1)
+
+
+def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum_f, dA_cumsum_b, B, CB, dout, dstates_f, dstates_b, D=None, dx=None):
+    """-> dx, ddt_direct (batch, nheads, nchunks, chunk_size) float32, dD."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert CB.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    assert dout.shape == x.shape
+    assert dstates_f.shape == (batch, nchunks, nheads, headdim, dstate) and dstates_b.shape == dstates_f.shape
+    c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, x.dtype, x.device)
+    c.set_x(x); c.set_B(B); c.set_dout(dout); c.set_D(D)
+    c.put("CB", CB, torch.float32); c.put("dt_out", dt, torch.float32)
+    c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    c.put("dstates_f", dstates_f, torch.float32); c.put("dstates_b", dstates_b, torch.float32)
+    dx = c.put("dx", dx) if dx is not None else c.new("dx", x.shape, x.dtype)
+    ddt = c.new("ddt_direct", _bhcq(c))
+    dD = None
+    if D is not None:
+        dD = c.new("dD", tuple(D.shape))
+        c.new("red", (batch * nchunks * ((chunk_size + 63) // 64) * nheads * headdim,))
+    c.run("bimamba2_chunk_scan_bwd_dx")
+    return dx, ddt, (dD.to(D.dtype) if dD is not None else None)
+
+
+def _chunk_state_bwd_db(x, dt, dA_cumsum_f, dA_cumsum_b, dstates_f, dstates_b, B=None, ngroups=1):
+    """-> dB state part (batch, seqlen, ngroups, dstate) float32, v_f, v_b (batch, nheads, nchunks, chunk_size):
+    per-position terms whose exclusive prefix (v_f) / suffix (v_b) sums are the reference's ddA_next_f/b."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    dstate = dstates_f.shape[-1]
+    c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, x.dtype, x.device)
+    c.set_x(x); c.set_B(B)
+    c.put("dt_out", dt, torch.float32); c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    c.put("dstates_f", dstates_f, torch.float32); c.put("dstates_b", dstates_b, torch.float32)
+    dBs = torch.zeros(batch, seqlen, ngroups, dstate, device=x.device, dtype=torch.float32); c.put("dBs", dBs)
+    vf = c.new("v_f", _bhcq(c)); vb = c.new("v_b", _bhcq(c))
+    c.run("bimamba2_chunk_state_bwd_db")
+    return dBs, vf, vb
+
+
+def _chunk_scan_bwd_dC(states_f, states_b, dA_cumsum_f, dA_cumsum_b, dout, C=None, ngroups=1):
+    """-> dC state part float32, u_f, u_b: per-position terms whose inclusive suffix (u_f) / prefix (u_b) sums
+    are the reference's ddA_prev_f/b."""
+    batch, seqlen, nheads, headdim = dout.shape
+    _, _, nchunks, chunk_size = dA_cumsum_f.shape
+    dstate = states_f.shape[-1]
+    c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, dout.dtype, dout.device)
+    c.set_dout(dout); c.set_C(C)
+    c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    c.put("states_f", states_f, torch.float32); c.put("states_b", states_b, torch.float32)
+    dCs = torch.zeros(batch, seqlen, ngroups, dstate, device=dout.device, dtype=torch.float32); c.put("dCs", dCs)
+    uf = c.new("u_f", _bhcq(c)); ub = c.new("u_b", _bhcq(c))
+    c.run("bimamba2_chunk_scan_bwd_dc")
+    return dCs, uf, ub
+
+
+def _chunk_scan_bwd_dcb(x, dt, dA_cumsum_f, dA_cumsum_b, dout, CB, ngroups=1):
+    """-> dCB (batch, nchunks, ngroups, Q, Q) float32 and the within-chunk part of d(dt*A)
+    (batch, nheads, nchunks, Q) (the reference's ddA_f + ddA_b of its two "stable" kernels)."""
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, nchunks, chunk_size = dt.shape
+    c = _Call(batch, seqlen, nheads, headdim, ngroups, 1, chunk_size, x.dtype, x.device)
+    c.set_x(x); c.set_dout(dout)
+    c.put("CB", CB, torch.float32); c.put("dt_out", dt, torch.float32)
+    c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    dCB = c.new("dCB", (batch, nchunks, ngroups, chunk_size, chunk_size))
+    nqt = (chunk_size + 63) // 64
+    da = c.new("da_intra", (batch, nheads, nchunks, nqt, chunk_size))
+    c.run("bimamba2_chunk_scan_bwd_dcb")
+    return dCB, da.sum(3)
+
+
+def _bmm_chunk_bwd(B, C, dCB, dBs, dCs):
+    """dB = dBs + dCB^T.C and dC = dCs + dCB.B per chunk, in the dtype of B / C."""
+    batch, seqlen, ngroups, dstate = B.shape
+    chunk_size = dCB.shape[-1]
+    c = _Call(batch, seqlen, ngroups, 1, ngroups, dstate, chunk_size, B.dtype, B.device)
+    c.set_B(B); c.set_C(C)
+    c.put("dCB", dCB, torch.float32); c.put("dBs", dBs, torch.float32); c.put("dCs", dCs, torch.float32)
+    dB = torch.zeros(B.shape, device=B.device, dtype=B.dtype); c.put("dB", dB)
+    dC = torch.zeros(B.shape, device=B.device, dtype=B.dtype); c.put("dC", dC)
+    c.run("bimamba2_bmm_chunk_bwd")
+    return dB, dC
+
+
+# =============================================================================================================
+# combined forward / backward
+# =============================================================================================================
+def _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit):
+    batch, seqlen, nheads, headdim = x.shape
+    _, _, ngroups, dstate = B.shape
+    assert nheads % ngroups == 0
+    assert B.shape == (batch, seqlen, ngroups, dstate)
+    assert x.shape == (batch, seqlen, nheads, headdim)
+    assert dt.shape == (batch, seqlen, nheads)
+    assert A.shape == (nheads,)
+    assert C.shape == B.shape
+    _check_chunk(chunk_size)
+    if z is not None:
+        assert z.shape == x.shape
+    if D is not None:
+        assert D.shape == (nheads, headdim) or D.shape == (nheads,)
+    if dt_bias is not None:
+        assert dt_bias.shape == (nheads,)
+    _require_gpu(x, "x")
+    c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, x.dtype, x.device, dt.dtype,
+              dt_softplus, dt_limit)
+    c.set_x(x); c.set_dt(dt); c.set_A(A); c.set_B(B); c.set_C(C)
+    c.set_D(D); c.set_z(z); c.set_dt_bias(dt_bias)
+    return c
+
+
+def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
+                                   dt_limit=(0.0, _INF), return_intermediates=True):
+    """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
+    like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
+    out, out_x and the final states are materialised as tensors (the rest lives in a workspace)."""
+    c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
+    batch, seqlen, nheads, headdim = x.shape
+    dstate = B.shape[-1]
+    out = c.new("out", x.shape, x.dtype)
+    out_x = c.new("out_x", x.shape, x.dtype) if z is not None else None
+    ff = c.new("final_f", (batch, nheads, headdim, dstate)); fb = c.new("final_b", (batch, nheads, headdim, dstate))
+    dt_out = cs_f = cs_b = sf = sb = None
+    if return_intermediates:
+        dt_out = c.new("dt_out", _bhcq(c)); cs_f = c.new("cs_f", _bhcq(c)); cs_b = c.new("cs_b", _bhcq(c))
+        sshape = (batch, c.nchunks, nheads, headdim, dstate)
+        sf = c.new("states_f", sshape); sb = c.new("states_b", sshape)
+    c.workspace(False)
+    c.run("bimamba2_fwd")
+    return out, out_x, dt_out, cs_f, cs_b, sf, sb, ff, fb
+
+
+def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
+                                   dfinal_states=None, dt_softplus=False, dt_limit=(0.0, _INF),
+                                   dx=None, ddt=None, dB=None, dC=None, dz=None, recompute_output=False):
+    """Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias).  `out` must be the pre-gate output out_x when z is
+    given (it is what the autograd function saves); it is not read otherwise."""
+    assert dfinal_states is None, "final states are not supported in the backward pass"
+    assert not recompute_output, "recompute_output is not supported"
+    assert dout.shape == x.shape
+    c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
+    batch, seqlen, nheads, headdim = x.shape
+    c.set_dout(dout)
+    if z is not None:
+        assert out.shape == x.shape
+        c.put("out_x", out.contiguous() if out.dtype == x.dtype else out.to(x.dtype).contiguous())
+        dz = c.put("dz", dz) if dz is not None else c.new("dz", x.shape, x.dtype)
+    dx = c.put("dx", dx) if dx is not None else c.new("dx", x.shape, x.dtype)
+    ddt = c.put("ddt", ddt) if ddt is not None else c.new("ddt", dt.shape, dt.dtype)
+    dB = c.put("dB", dB) if dB is not None else c.new("dB", B.shape, x.dtype)
+    dC = c.put("dC", dC) if dC is not None else c.new("dC", C.shape, x.dtype)
+    dA = c.new("dA", (nheads,))
+    dD = c.new("dD", tuple(D.shape)) if D is not None else None
+    ddt_bias = c.new("ddt_bias", (nheads,)) if dt_bias is not None else None
+    c.workspace(True)
+    c.run("bimamba2_bwd")
+    return (dx, ddt, dA.to(A.dtype), dB.to(B.dtype), dC.to(C.dtype),
+            dD.to(D.dtype) if dD is not None else None, dz,
+            ddt_bias.to(dt_bias.dtype) if ddt_bias is not None else None)
+
+
+class MambaChunkScanCombinedFn(torch.autograd.Function):
+    """Same 12 positional arguments and the same 12-tuple of gradients as the reference's autograd function
+    (src/ssd/bi/ssd_combined.py:555-574)."""
+
+    @staticmethod
+    def forward(ctx, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
+                dt_limit=(0.0, _INF), return_final_states=False):
+        ctx.dt_dtype = dt.dtype
+        out, out_x, _, _, _, _, _, ff, fb = _mamba_chunk_scan_combined_fwd(
+            x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit,
+            return_intermediates=False)
+        ctx.save_for_backward(out_x if z is not None else None, x, dt, A, B, C, D, z, dt_bias)
+        ctx.dt_softplus = dt_softplus
+        ctx.chunk_size = chunk_size
+        ctx.dt_limit = dt_limit
+        ctx.return_final_states = return_final_states
+        if not return_final_states:
+            return out
+        ctx.mark_non_differentiable(ff, fb)
+        return out, ff, fb
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        out_x, x, dt, A, B, C, D, z, dt_bias = ctx.saved_tensors
+        assert not ctx.return_final_states, "final states are not currently supported in the bwd pass"
+        dx, ddt, dA, dB, dC, dD, dz, ddt_bias = _mamba_chunk_scan_combined_bwd(
+            dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
+            dt_limit=ctx.dt_limit)
+        return dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, None, None, None
+
+
+def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
+                                dt_limit=(0.0, _INF), return_final_states=False):
+    """Bidirectional SSD:  y = SS(x) + flip(SS(flip(x))) + D*x, gated by silu(z) when z is given.
+
+    Argument:
+        x: (batch, seqlen, nheads, headdim)
+        dt: (batch, seqlen, nheads)
+        A: (nheads)
+        B: (batch, seqlen, ngroups, dstate)
+        C: (batch, seqlen, ngroups, dstate)
+        chunk_size: int, 32..256
+        D: (nheads, headdim) or (nheads,)
+        z: (batch, seqlen, nheads, headdim)
+        dt_bias: (nheads,)
+        dt_softplus: whether to apply softplus to dt (+ dt_bias)
+        dt_limit: clamp range for the transformed dt
+    Return:
+        out: (batch, seqlen, nheads, headdim), or (out, final_states_f, final_states_b) with
+        return_final_states=True (final states are (batch, nheads, headdim, dstate) float32)
+    """
+    return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
+                                          return_final_states)

@@ -1,0 +1,155 @@
+/* C ABI of libbimamba2_hip.so: the bidirectional SSD operator of Bi-Mamba2 for AMD MI355X (gfx950).
+ *
+ *   y = SS(x) + flip(SS(flip(x))) + D*x   [* silu(z)]          forward and backward
+ *
+ * Every entry point takes one `const bimamba2_params*`, enqueues its kernels on `stream` and returns
+ * immediately (no host synchronisation, no device allocation, no global state).  Return value: 0 on
+ * success, a negative BIMAMBA2_E* code otherwise (bimamba2_strerror() gives the text).  All pointers are
+ * device pointers; the caller owns every buffer, including the intermediates and the workspace.
+ *
+ * Each declaration cites the function of the reference project (Hprairie/Bi-Mamba2, paths relative to its
+ * root) that it replaces.
+ *
+ * Layouts (row-major, sizes in elements; B=batch L=seqlen H=nheads P=headdim G=ngroups N=dstate
+ * Q=chunk_size nc=ceil(L/Q)):
+ *   x, z, out, out_x, dout, dx, dz   (B, L, H, P)   element type `dtype`; last-dim stride 1, the other three
+ *                                                   strides given for the inputs x, z, dout; outputs contiguous
+ *   Bm, Cm, dB, dC                   (B, L, G, N)   element type `dtype`; input strides given; outputs contiguous
+ *   dt, ddt                          (B, L, H)      element type `dt_dtype`; strides given for dt; ddt contiguous
+ *   A, D, dt_bias, dA, dD, ddt_bias  (H,) [D, dD may be (H, P)]   float32, contiguous
+ *   dt_out, cs_f, cs_b, ddt_direct, u_f, u_b, v_f, v_b   (B, H, nc, Q)   float32
+ *   CB, dCB                          (B, nc, G, Q, Q)   float32, CB[.., l, s] = C_l . B_s
+ *   states_f/b, dstates_f/b          (B, nc, H, P, N)   float32
+ *   final_f, final_b                 (B, H, P, N)       float32
+ */
+#ifndef BIMAMBA2_H
+#define BIMAMBA2_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { BIMAMBA2_F32 = 0, BIMAMBA2_BF16 = 1, BIMAMBA2_F16 = 2 };
+
+enum {
+    BIMAMBA2_OK = 0,
+    BIMAMBA2_EINVAL = -1,      /* null pointer / inconsistent dimensions */
+    BIMAMBA2_EUNSUPPORTED = -2,/* shape or dtype outside what the kernels are built for */
+    BIMAMBA2_EWORKSPACE = -3,  /* workspace missing or too small */
+    BIMAMBA2_ELAUNCH = -4      /* HIP reported a launch error */
+};
+
+/* limits of the compiled kernels */
+#define BIMAMBA2_MAX_CHUNK 256
+#define BIMAMBA2_MIN_CHUNK 32   /* same lower bound as the reference (src/ssd/bi/ssd_combined.py:306) */
+#define BIMAMBA2_MAX_HEADDIM 128
+#define BIMAMBA2_MAX_DSTATE 256
+
+typedef struct bimamba2_params {
+    /* problem */
+    int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+    int32_t dtype;          /* BIMAMBA2_* : x, z, Bm, Cm, out, out_x, dout and their gradients */
+    int32_t dt_dtype;       /* BIMAMBA2_* : dt and ddt */
+    int32_t has_D, D_has_hdim, has_z, has_dt_bias, dt_softplus;
+    float dt_min, dt_max;
+    /* element strides of the strided inputs (last dim contiguous) */
+    int64_t x_sb, x_sl, x_sh;
+    int64_t z_sb, z_sl, z_sh;
+    int64_t dout_sb, dout_sl, dout_sh;
+    int64_t B_sb, B_sl, B_sg;
+    int64_t C_sb, C_sl, C_sg;
+    int64_t dt_sb, dt_sl, dt_sh;
+    /* inputs */
+    const void *x, *dt, *Bm, *Cm, *z, *dout;
+    const float *A, *D, *dt_bias;
+    /* forward outputs */
+    void *out, *out_x;
+    float *final_f, *final_b;   /* optional */
+    /* backward outputs */
+    void *dx, *ddt, *dB, *dC, *dz;
+    float *dA, *dD, *ddt_bias;
+    /* intermediates (caller-owned; the composite entry points carve them from `workspace` when NULL) */
+    float *dt_out, *cs_f, *cs_b;
+    float *CB, *dCB;
+    float *states_f, *states_b;     /* chunk states, overwritten in place by the inter-chunk scan */
+    float *dstates_f, *dstates_b;
+    void *dout_x;                   /* dout * silu(z), element type `dtype` */
+    float *ddt_direct, *u_f, *u_b, *v_f, *v_b, *da_intra;
+    float *ddA_chunk_f, *ddA_chunk_b;   /* (B, H, nc) */
+    float *dBs, *dCs;                   /* (B, L, G, N) float32 partial gradients */
+    float *red;                         /* scratch for two-stage reductions */
+    void *workspace;
+    size_t workspace_bytes;
+    void *stream;                   /* hipStream_t */
+} bimamba2_params;
+
+/* text of an error code */
+const char *bimamba2_strerror(int code);
+/* library version (major*10000 + minor*100 + patch) */
+int bimamba2_version(void);
+/* sizeof(bimamba2_params) as compiled into the library, for bindings to check their mirror of the struct */
+size_t bimamba2_params_size(void);
+
+/* bytes of workspace the composite entry points need (is_bwd = 0: forward, 1: backward) */
+size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd);
+
+/* Whole forward; replaces _mamba_chunk_scan_combined_fwd (src/ssd/bi/ssd_combined.py:297-331).
+ * Needs: x dt A Bm Cm [D z dt_bias] out [out_x when has_z] [final_f final_b] workspace. */
+int bimamba2_fwd(const bimamba2_params *p);
+
+/* Whole backward; replaces _mamba_chunk_scan_combined_bwd (src/ssd/bi/ssd_combined.py:334-475).
+ * Needs: the forward inputs, dout, out_x (pre-gate output, when has_z), dx ddt dA dB dC [dD dz ddt_bias],
+ * workspace. */
+int bimamba2_bwd(const bimamba2_params *p);
+
+/* ---- single stages (each is also what the composites run) ------------------------------------------ */
+
+/* dt -> dt_out, cs_f, cs_b.  Replaces _chunk_cumsum_fwd (src/ssd/bi/ssd_chunk_state.py:699-724). */
+int bimamba2_chunk_cumsum_fwd(const bimamba2_params *p);
+/* Cm, Bm -> CB.  Replaces _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208). */
+int bimamba2_bmm_chunk_fwd(const bimamba2_params *p);
+/* x, Bm, dt_out, cs_f, cs_b -> states_f, states_b.  Replaces _chunk_state_fwd
+ * (src/ssd/bi/ssd_chunk_state.py:764-798). */
+int bimamba2_chunk_state_fwd(const bimamba2_params *p);
+/* states_f/b (chunk states) -> states_f/b (state entering each chunk), in place, both directions in one
+ * launch; optional final_f/final_b.  Replaces the two _state_passing_fwd calls
+ * (src/ssd/bi/ssd_state_passing.py:190-207; src/ssd/bi/ssd_combined.py:324-327). */
+int bimamba2_state_passing_fwd(const bimamba2_params *p);
+/* CB, x, z, dt_out, cs_f, cs_b, Cm, states_f/b, D -> out, out_x.  Replaces _chunk_scan_fwd
+ * (src/ssd/bi/ssd_chunk_scan.py:1638-1686). */
+int bimamba2_chunk_scan_fwd(const bimamba2_params *p);
+
+/* z, out_x, dout -> dz, dout_x.  Replaces _chunk_scan_bwd_dz (src/ssd/bi/ssd_chunk_scan.py:1741-1798);
+ * dD is produced by bimamba2_chunk_scan_bwd_dx. */
+int bimamba2_chunk_scan_bwd_dz(const bimamba2_params *p);
+/* dout (dout_x when has_z), Cm, cs_f, cs_b -> dstates_f/b.  Replaces _chunk_scan_bwd_dstates
+ * (src/ssd/bi/ssd_chunk_scan.py:1801-1826). */
+int bimamba2_chunk_scan_bwd_dstates(const bimamba2_params *p);
+/* states_f/b, dstates_f/b (in place), cs -> dstates_f/b (gradient of each chunk state), ddA_chunk_f/b.
+ * Replaces the two _state_passing_bwd calls (src/ssd/bi/ssd_state_passing.py:210-248). */
+int bimamba2_state_passing_bwd(const bimamba2_params *p);
+/* -> dx, ddt_direct, dD partials (reduced into dD).  Replaces _chunk_scan_chunk_state_bwd_dx
+ * (src/ssd/bi/ssd_combined.py:235-294). */
+int bimamba2_chunk_scan_bwd_dx(const bimamba2_params *p);
+/* x, dstates_f/b, dt_out, cs, Bm -> dBs, v_f, v_b.  Replaces _chunk_state_bwd_db
+ * (src/ssd/bi/ssd_chunk_state.py:836-894); v_* are its ddA_next terms before the scan. */
+int bimamba2_chunk_state_bwd_db(const bimamba2_params *p);
+/* dout, states_f/b, cs, Cm -> dCs, u_f, u_b.  Replaces _chunk_scan_bwd_dC
+ * (src/ssd/bi/ssd_chunk_scan.py:1829-1877); u_* are its ddA_cumsum_prev terms. */
+int bimamba2_chunk_scan_bwd_dc(const bimamba2_params *p);
+/* x, dout, dt_out, cs, CB -> dCB, da_intra.  Replaces _chunk_scan_bwd_dcb (src/ssd/bi/ssd_chunk_scan.py:1880-1909)
+ * and _chunk_scan_bwd_ddAcs_stable_fwd/_bwd (src/ssd/bi/ssd_chunk_scan.py:2036-2098) in one pass. */
+int bimamba2_chunk_scan_bwd_dcb(const bimamba2_params *p);
+/* dCB, Cm, Bm, dBs, dCs -> dB, dC.  Replaces the two _bmm_chunk_bwd calls (src/ssd/bi/ssd_bmm.py:211-262). */
+int bimamba2_bmm_chunk_bwd(const bimamba2_params *p);
+/* da_intra, u, v, ddA_chunk, ddt_direct, dt, A, dt_bias -> ddt, dA, ddt_bias.  Replaces the host-side
+ * scans (src/ssd/bi/ssd_combined.py:456-466) and _chunk_cumsum_bwd (src/ssd/bi/ssd_chunk_state.py:727-761). */
+int bimamba2_chunk_cumsum_bwd(const bimamba2_params *p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BIMAMBA2_H */

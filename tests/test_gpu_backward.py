@@ -1,0 +1,75 @@
+"""GPU parity of the backward path against torch.autograd on the float64 oracle, through the C ABI."""
+import pytest
+import torch
+
+from oracle import bimamba2_oracle as O
+from tests.helpers import assert_close, make_case, to64, to_dev
+
+pytestmark = pytest.mark.gpu
+INF = float("inf")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from bi_mamba2_amd import ops
+    return ops
+
+
+def _run_bwd(ops, inp, Q, sp, lim, seed=5):
+    d = to_dev(inp)
+    leaves = {k: (v.clone().requires_grad_(True) if v is not None else None) for k, v in d.items()}
+    out = ops.bimamba_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], Q, D=leaves["D"],
+                                          z=leaves["z"], dt_bias=leaves["dt_bias"], dt_softplus=sp, dt_limit=lim)
+    g = torch.Generator().manual_seed(seed)
+    dout = torch.randn(out.shape, generator=g).to(out.dtype)
+    out.backward(dout.to(out.device))
+    grads = {"d" + k: (v.grad if v is not None else None) for k, v in leaves.items()}
+    r = to64(inp)
+    ref = O.bimamba2_grads(dout.double(), r["x"], r["dt"], r["A"], r["B"], r["C"], D=r["D"], z=r["z"], dt_bias=r["dt_bias"],
+                           dt_softplus=sp, dt_limit=lim)
+    return out, grads, ref
+
+
+def _check(out, grads, ref, dtype):
+    assert_close(out, ref["out"], dtype, "out")
+    for k in ("dx", "dB", "dC", "dz"):
+        if ref[k] is not None:
+            assert grads[k].dtype == dtype
+            assert_close(grads[k], ref[k], dtype, k)
+    # reductions over the whole batch and sequence are float32 sums of values carrying the input rounding
+    for k in ("ddt", "dA", "dD", "ddt_bias"):
+        if ref[k] is not None:
+            assert_close(grads[k], ref[k], dtype, k)
+
+
+# the reference's own end-to-end backward grid (tests/test_bwd_scan.py:8-16 there)
+REF_BWD_GRID = [(b, L, 1, P, 1, N, 32) for b in (1, 2) for L in (32, 64, 128) for P in (1, 4) for N in (1, 4)]
+
+
+@pytest.mark.parametrize("shape", REF_BWD_GRID)
+def test_backward_reference_grid(ops, shape):
+    b, L, H, P, G, N, Q = shape
+    inp = make_case(b, L, H, P, G, N, torch.float32, with_D=False, ref_style=True)
+    out, grads, ref = _run_bwd(ops, inp, Q, True, (0.0, INF))
+    _check(out, grads, ref, torch.float32)
+
+
+E2E = [
+    # batch, seqlen, H, P, G, N, chunk, dtype, z, D, bias, softplus, limit
+    (2, 256, 4, 32, 1, 16, 64, torch.float32, False, "h", True, True, (0.0, INF)),
+    (2, 250, 4, 32, 2, 16, 64, torch.float32, True, "hp", True, True, (0.0, INF)),
+    (1, 130, 2, 64, 1, 64, 128, torch.float32, True, "h", False, False, (0.0, INF)),
+    (2, 200, 4, 16, 4, 8, 32, torch.float32, False, "none", True, True, (0.01, 0.2)),
+    (1, 100, 2, 128, 1, 128, 48, torch.float32, True, "hp", True, True, (0.0, INF)),
+    (2, 512, 8, 64, 1, 64, 256, torch.bfloat16, True, "h", True, True, (0.0, INF)),
+    (1, 700, 4, 64, 2, 128, 256, torch.bfloat16, False, "h", True, True, (0.0, INF)),
+    (2, 256, 4, 64, 4, 64, 128, torch.float16, True, "h", True, True, (0.0, INF)),
+]
+
+
+@pytest.mark.parametrize("case", E2E)
+def test_backward_end_to_end(ops, case):
+    b, L, H, P, G, N, Q, dtype, z, Dk, bias, sp, lim = case
+    inp = make_case(b, L, H, P, G, N, dtype, with_z=z, with_D=(Dk != "none"), D_has_hdim=(Dk == "hp"), with_bias=bias)
+    out, grads, ref = _run_bwd(ops, inp, Q, sp, lim)
+    _check(out, grads, ref, dtype)

@@ -1,0 +1,125 @@
+"""CPU tests that pin the oracle itself (no GPU, no kernels).
+
+The three statements of the forward (literal recurrence, quadratic closed form, chunked flip-and-sum) plus
+the staged composition are compared with each other, with the scalar C restatement, with special cases whose
+answer is textbook arithmetic, and the autograd gradients with finite differences."""
+import math
+
+import pytest
+import torch
+
+from oracle import bimamba2_oracle as O
+from oracle.seq_c import seq_forward
+from tests.helpers import make_case, to64
+
+CASES = [
+    # batch, seqlen, H, P, G, N, chunk, z, D_hdim, softplus, bias, limit
+    (2, 70, 4, 8, 2, 6, 32, True, False, True, True, (0.0, float("inf"))),
+    (1, 33, 2, 4, 1, 3, 32, False, True, False, False, (0.0, float("inf"))),
+    (2, 96, 4, 4, 4, 4, 32, False, False, True, True, (0.02, 0.3)),
+    (1, 64, 6, 5, 3, 7, 64, True, True, True, False, (0.0, float("inf"))),
+]
+
+
+def _kw(inp, softplus, limit):
+    return dict(D=inp["D"], z=inp["z"], dt_bias=inp["dt_bias"], dt_softplus=softplus, dt_limit=limit)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_forms_agree(case):
+    b, L, H, P, G, N, Q, z, dh, sp, bias, lim = case
+    inp = to64(make_case(b, L, H, P, G, N, torch.float32, with_z=z, D_has_hdim=dh, with_bias=bias))
+    args = (inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"])
+    kw = _kw(inp, sp, lim)
+    seq = O.bimamba2_sequential(*args, **kw)
+    quad = O.bimamba2_quadratic(*args, **kw)
+    naive = O.bimamba2_naive_chunked(*args, Q, **kw)
+    staged = O.bimamba2_staged(*args, Q, **kw)
+    cseq = seq_forward(*args, **kw)
+    for name, o in (("quadratic", quad), ("naive", naive), ("staged", staged), ("C", cseq)):
+        torch.testing.assert_close(o[0], seq[0], rtol=1e-11, atol=1e-11, msg=lambda m: f"{name} out: {m}")
+        torch.testing.assert_close(o[1], seq[1], rtol=1e-11, atol=1e-11, msg=lambda m: f"{name} out_x: {m}")
+    for name, o in (("naive", naive), ("staged", staged), ("C", cseq)):
+        torch.testing.assert_close(o[2], seq[2], rtol=1e-11, atol=1e-11)
+        torch.testing.assert_close(o[3], seq[3], rtol=1e-11, atol=1e-11)
+
+
+def test_A_zero_is_masked_matmul():
+    """A = 0: every decay is 1, so y_t = sum_s (C_t.B_s) dt_s x_s (1[s<=t] + 1[s>=t])."""
+    inp = to64(make_case(1, 40, 2, 3, 1, 5, with_D=False, with_bias=False))
+    inp["A"] = torch.zeros(2, dtype=torch.float64)
+    dtp = inp["dt"].abs()
+    out = O.bimamba2_sequential(inp["x"], dtp, inp["A"], inp["B"], inp["C"])[0]
+    cb = torch.einsum("btgn,bsgn->bts", inp["C"], inp["B"])
+    L = 40
+    mask = torch.tril(torch.ones(L, L, dtype=torch.float64)) + torch.triu(torch.ones(L, L, dtype=torch.float64))
+    ref = torch.einsum("bts,bsh,bshp->bthp", cb * mask, dtp, inp["x"])
+    torch.testing.assert_close(out, ref, rtol=1e-12, atol=1e-12)
+
+
+def test_constant_channel_geometric_series():
+    """x = B = C = 1, dt = d, A = a: y_t = d (sum_{k=0..t} r^k + sum_{k=0..L-1-t} r^k), r = e^{d a}."""
+    L, d, a = 17, 0.3, -0.7
+    one = torch.ones(1, L, 1, 1, dtype=torch.float64)
+    out = O.bimamba2_quadratic(one, torch.full((1, L, 1), d, dtype=torch.float64), torch.tensor([a], dtype=torch.float64),
+                               one.clone(), one.clone())[0]
+    r = math.exp(d * a)
+    ref = torch.tensor([d * ((1 - r ** (t + 1)) / (1 - r) + (1 - r ** (L - t)) / (1 - r)) for t in range(L)], dtype=torch.float64)
+    torch.testing.assert_close(out.flatten(), ref, rtol=1e-12, atol=1e-12)
+
+
+def test_flip_equivariance_and_linearity():
+    inp = to64(make_case(2, 50, 2, 4, 1, 4, with_z=False))
+    f = lambda x, dt, B, C: O.bimamba2_quadratic(x, dt, inp["A"], B, C, D=inp["D"], dt_bias=inp["dt_bias"], dt_softplus=True)[0]
+    y = f(inp["x"], inp["dt"], inp["B"], inp["C"])
+    yf = f(inp["x"].flip(1), inp["dt"].flip(1), inp["B"].flip(1), inp["C"].flip(1))
+    torch.testing.assert_close(yf.flip(1), y, rtol=1e-11, atol=1e-11)
+    y2 = f(2.5 * inp["x"], inp["dt"], inp["B"], inp["C"])
+    torch.testing.assert_close(y2, 2.5 * y, rtol=1e-11, atol=1e-11)
+
+
+def test_single_chunk_has_no_state_contribution():
+    inp = to64(make_case(1, 32, 2, 4, 1, 4))
+    dt_out, cs_f, cs_b = O.stage_chunk_cumsum(inp["dt"], inp["A"], 32, inp["dt_bias"], True)
+    S_f, S_b = O.stage_chunk_state(inp["B"], inp["x"], dt_out, cs_f, cs_b)
+    prev_f, prev_b, ff, fb = O.stage_state_passing(S_f, S_b, cs_f, cs_b)
+    assert prev_f.abs().max() == 0 and prev_b.abs().max() == 0
+    torch.testing.assert_close(ff, S_f[:, 0])
+    torch.testing.assert_close(fb, S_b[:, 0])
+
+
+def test_softplus_threshold_and_clamp():
+    dt = torch.tensor([[[-30.0], [0.0], [19.9], [20.1], [25.0]]], dtype=torch.float64)
+    out = O.dt_transform(dt, None, True, (0.0, float("inf")))
+    ref = torch.tensor([math.log1p(math.exp(-30.0)), math.log(2.0), math.log1p(math.exp(19.9)), 20.1, 25.0], dtype=torch.float64)
+    torch.testing.assert_close(out.flatten(), ref, rtol=1e-12, atol=0)
+    out = O.dt_transform(torch.tensor([[[-1.0], [0.5], [3.0]]], dtype=torch.float64), None, False, (0.1, 2.0))
+    torch.testing.assert_close(out.flatten(), torch.tensor([0.1, 0.5, 2.0], dtype=torch.float64))
+    # default limits still clamp negative dt to 0 when softplus is off
+    out = O.dt_transform(torch.tensor([[[-1.0]]], dtype=torch.float64), None, False)
+    assert out.item() == 0.0
+
+
+def test_autograd_matches_finite_differences():
+    inp = to64(make_case(1, 9, 2, 2, 1, 3, with_z=True, D_has_hdim=True))
+    leaves = [inp[k].clone().requires_grad_(True) for k in ("x", "dt", "A", "B", "C", "D", "z", "dt_bias")]
+
+    def fn(x, dt, A, B, C, D, z, bias):
+        return O.bimamba2_quadratic(x, dt, A, B, C, D=D, z=z, dt_bias=bias, dt_softplus=True, dt_limit=(0.0, 5.0))[0]
+
+    assert torch.autograd.gradcheck(fn, leaves, eps=1e-6, atol=1e-6, rtol=1e-5)
+
+    def fn_seq(x, dt, A, B, C, D, z, bias):
+        return O.bimamba2_sequential(x, dt, A, B, C, D=D, z=z, dt_bias=bias, dt_softplus=True)[0]
+
+    assert torch.autograd.gradcheck(fn_seq, leaves, eps=1e-6, atol=1e-6, rtol=1e-5)
+
+
+def test_gradients_of_forms_agree():
+    inp = to64(make_case(2, 70, 4, 4, 2, 4, with_z=True))
+    dout = torch.randn(inp["x"].shape, dtype=torch.float64, generator=torch.Generator().manual_seed(3))
+    kw = dict(D=inp["D"], z=inp["z"], dt_bias=inp["dt_bias"], dt_softplus=True)
+    a = O.bimamba2_grads(dout, inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], form="quadratic", **kw)
+    b = O.bimamba2_grads(dout, inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], form="chunked", chunk_size=32, **kw)
+    for k in a:
+        torch.testing.assert_close(a[k], b[k], rtol=1e-10, atol=1e-10, msg=lambda m: f"{k}: {m}")
