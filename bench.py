@@ -1,0 +1,252 @@
+"""Benchmark of the bidirectional SSD operator (bimamba_chunk_scan_combined, forward + backward) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one forward + backward pass through autograd on one batch of synthetic inputs that already live in
+HBM.  The workload is the forward-bench configuration of the project's baseline file (batch 4, seqlen 2048,
+32 heads x headdim 64, 1 group, dstate 64, chunk 256, bf16 x/B/C/z, float32 dt/A/D/dt_bias, z gate and D).
+Prints ONE JSON line: whole-job throughput in Mtokens/s, the roofline position of the slowest kernel (its
+duration measured here with HIP events on the launch stream) and a CPU baseline (the oracle's chunked
+flip-and-sum path in PyTorch on the host cores, on a bounded sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
+
+WORKLOAD = dict(batch=4, seqlen=2048, nheads=32, headdim=64, ngroups=1, dstate=64, chunk_size=256)
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
+# size); None until measured for the kernel in question.  Source: the summaries under profiles/.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def stage_table(w, e):
+    """Algorithmic flops and bytes per launch of every stage kernel (e = bytes per element of x/B/C/z)."""
+    B, L, H, P, G, N, Q = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate", "chunk_size"))
+    nc = (L + Q - 1) // Q
+    u, ug = B * nc * H, B * nc * G                 # (b, c, h) and (b, c, g) units
+    T4, T2, T1 = B * L * H * P, B * L * G * N, B * H * nc * Q
+    st = 4 * B * nc * H * P * N                     # one float32 state tensor
+    cb = 4 * ug * Q * Q
+    return {
+        # entry point: (flops, bytes)
+        "bimamba2_chunk_cumsum_fwd": (0, 4 * B * L * H + 3 * 4 * T1),
+        "bimamba2_bmm_chunk_fwd": (ug * 2 * Q * Q * N, 2 * e * T2 + cb),
+        "bimamba2_chunk_state_fwd": (u * 4 * P * N * Q, e * T4 + e * T2 + 3 * 4 * T1 + 2 * st),
+        "bimamba2_state_passing_fwd": (0, 4 * st),
+        "bimamba2_chunk_scan_fwd": (u * (2 * Q * Q * P + 4 * Q * P * N), 4 * e * T4 + e * T2 + 3 * 4 * T1 + 2 * st + cb),
+        "bimamba2_chunk_scan_bwd_dz": (0, 5 * e * T4),
+        "bimamba2_chunk_scan_bwd_dstates": (u * 4 * P * N * Q, e * T4 + e * T2 + 2 * 4 * T1 + 2 * st),
+        "bimamba2_state_passing_bwd": (0, 6 * st),
+        "bimamba2_chunk_scan_bwd_dx": (u * (2 * Q * Q * P + 4 * Q * P * N), 3 * e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + cb),
+        "bimamba2_chunk_state_bwd_db": (u * 4 * Q * P * N, e * T4 + e * T2 + 5 * 4 * T1 + 2 * st + 4 * T2),
+        "bimamba2_chunk_scan_bwd_dc": (u * 4 * Q * P * N, e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + 4 * T2),
+        "bimamba2_chunk_scan_bwd_dcb": (u * 2 * Q * Q * P, 2 * e * T4 + 3 * 4 * T1 + 2 * cb + 4 * B * H * nc * ((Q + 63) // 64) ** 2 * 128),
+        "bimamba2_bmm_chunk_bwd": (ug * 4 * Q * Q * N, 4 * e * T2 + cb + 2 * 4 * T2),
+        "bimamba2_chunk_cumsum_bwd": (0, 2 * 4 * B * L * H + 8 * 4 * T1),
+    }
+
+
+def whole_op_bytes(w, e, has_z):
+    B, L, H, P, G, N = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate"))
+    T4, T2, T1 = B * L * H * P, B * L * G * N, B * L * H
+    fwd = e * T4 * (2 + (2 if has_z else 0)) + 2 * e * T2 + 4 * T1
+    bwd = e * T4 * (3 + (3 if has_z else 0)) + 4 * e * T2 + 8 * T1
+    return fwd, bwd
+
+
+def cpu_baseline(w, budget_s=15.0):
+    """The oracle's naive flip-and-sum path (chunked causal SSD twice) in float32 PyTorch on the host cores,
+    forward + backward, on one batch row of the same workload, repeated for about 15 s."""
+    import torch
+    from oracle import bimamba2_oracle as O
+
+    cores = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(cores)
+    heads = w["nheads"]
+    inp = O.make_inputs(1, w["seqlen"], heads, w["headdim"], 1, w["dstate"], seed=0, dtype=torch.float32, with_z=True)
+
+    def step():
+        leaves = {k: v.clone().requires_grad_(True) for k, v in inp.items()}
+        out = O.bimamba2_naive_chunked(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], w["chunk_size"],
+                                       D=leaves["D"], z=leaves["z"], dt_bias=leaves["dt_bias"], dt_softplus=True)[0]
+        out.backward(torch.ones_like(out))
+
+    step()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 25 and (time.perf_counter() - t_start < budget_s or len(times) < 3):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    value = w["seqlen"] / med / 1e6
+    return {"value": value, "unit": "Mtokens/s", "cores": cores, "kind": "port",
+            "sample": f"batch 1 (of {w['batch']}) x seqlen {w['seqlen']} x {heads} heads, float32, fwd+bwd via autograd, "
+                      f"median of {len(times)} runs = {med * 1e3:.1f} ms"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-z", action="store_true", help="benchmark without the z gate")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this build measures the operator on ONE GPU; --gpus must be 1 "
+                         "(the path has no multi-GPU part; DESIGN.md says how it would shard).\n")
+        sys.exit(2)
+
+    import torch
+    from bi_mamba2_amd import _lib, ops
+    from oracle import bimamba2_oracle as O
+
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    w = WORKLOAD
+    dtype, e = torch.bfloat16, 2
+    has_z = not args.no_z
+    inp = O.make_inputs(w["batch"], w["seqlen"], w["nheads"], w["headdim"], w["ngroups"], w["dstate"], seed=0,
+                        dtype=dtype, with_z=has_z)
+    leaves = {k: (v.to(dev).requires_grad_(True) if v is not None else None) for k, v in inp.items()}
+    dout = torch.randn(inp["x"].shape, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
+
+    def step():
+        out = ops.bimamba_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"],
+                                              w["chunk_size"], D=leaves["D"], z=leaves["z"], dt_bias=leaves["dt_bias"],
+                                              dt_softplus=True)
+        out.backward(dout)
+        for v in leaves.values():
+            if v is not None:
+                v.grad = None
+
+    def fwd_only():
+        with torch.no_grad():
+            ops.bimamba_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"],
+                                            w["chunk_size"], D=leaves["D"], z=leaves["z"], dt_bias=leaves["dt_bias"],
+                                            dt_softplus=True)
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    for _ in range(args.warmup):
+        step()
+    t_step = timed(step, args.steps)
+    t_fwd = timed(fwd_only, args.steps)
+    tokens = w["batch"] * w["seqlen"]
+    fwd_b, bwd_b = whole_op_bytes(w, e, has_z)
+
+    # ---- per-kernel durations: HIP events on the launch stream around back-to-back launches ----
+    c = ops._problem(leaves["x"].detach(), leaves["dt"].detach(), leaves["A"].detach(), leaves["B"].detach(),
+                     leaves["C"].detach(), w["chunk_size"], leaves["D"].detach(),
+                     leaves["z"].detach() if has_z else None, leaves["dt_bias"].detach(), True, (0.0, float("inf")))
+    c.set_dout(dout)
+    c.new("out", inp["x"].shape, dtype)
+    if has_z:
+        c.new("out_x", inp["x"].shape, dtype); c.new("dz", inp["x"].shape, dtype)
+    c.new("dx", inp["x"].shape, dtype); c.new("ddt", inp["dt"].shape, torch.float32)
+    c.new("dB", inp["B"].shape, dtype); c.new("dC", inp["B"].shape, dtype)
+    c.new("dA", (w["nheads"],)); c.new("dD", (w["nheads"],)); c.new("ddt_bias", (w["nheads"],))
+    # carve all intermediates once, by running the composites on an explicit workspace, then time each stage
+    # on explicitly allocated intermediates
+    nc = c.nchunks
+    bhcq = (w["batch"], w["nheads"], nc, w["chunk_size"])
+    for f in ("dt_out", "cs_f", "cs_b", "ddt_direct", "u_f", "u_b", "v_f", "v_b"):
+        c.new(f, bhcq)
+    nqt = (w["chunk_size"] + 63) // 64
+    c.new("da_intra", bhcq[:3] + (nqt * nqt, 2, 64))
+    cbs = (w["batch"], nc, w["ngroups"], w["chunk_size"], w["chunk_size"])
+    c.new("CB", cbs); c.new("dCB", cbs)
+    sts = (w["batch"], nc, w["nheads"], w["headdim"], w["dstate"])
+    for f in ("states_f", "states_b", "dstates_f", "dstates_b"):
+        c.new(f, sts)
+    if has_z:
+        c.new("dout_x", inp["x"].shape, dtype)
+    nsplit = (w["headdim"] * w["dstate"] + 1023) // 1024
+    c.new("ddA_chunk_f", (w["batch"], w["nheads"], nc, nsplit)); c.new("ddA_chunk_b", (w["batch"], w["nheads"], nc, nsplit))
+    slices = (w["nheads"] // w["ngroups"] + 3) // 4
+    c.new("dBs", (slices,) + tuple(inp["B"].shape)); c.new("dCs", (slices,) + tuple(inp["B"].shape))
+    c.new("red", (max(w["batch"] * nc * ((w["chunk_size"] + 63) // 64) * w["nheads"] * w["headdim"], 2 * w["batch"] * nc * w["nheads"]),))
+    c.run("bimamba2_fwd")
+    c.run("bimamba2_bwd")
+    torch.cuda.synchronize()
+    table = stage_table(w, e)
+    kernels = {}
+    reps = max(10, args.steps)
+    for entry, (flops, nbytes) in table.items():
+        if entry == "bimamba2_chunk_scan_bwd_dz" and not has_z:
+            continue
+        for _ in range(3):
+            c.run(entry)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(reps):
+            c.run(entry)
+        ev1.record()
+        torch.cuda.synchronize()
+        us = ev0.elapsed_time(ev1) * 1e3 / reps
+        kernels[entry] = {"us": round(us, 2), "gflop": round(flops / 1e9, 3), "mbytes": round(nbytes / 1e6, 2),
+                          "tflops": round(flops / us / 1e6, 2), "gbs": round(nbytes / us / 1e3, 1)}
+    dom = max(kernels, key=lambda k: kernels[k]["us"])
+    flops, nbytes = table[dom]
+    t_mfma = flops / (MFMA_PEAK_TFLOPS["bf16"] * 1e12)
+    t_hbm = nbytes / (HBM_PEAK_GBS * 1e9)
+    if t_mfma > t_hbm:
+        roof = {"kernel": dom, "bound": "mfma", "achieved": flops / kernels[dom]["us"] / 1e6, "peak": MFMA_PEAK_TFLOPS["bf16"],
+                "unit": "TFLOP/s"}
+    else:
+        roof = {"kernel": dom, "bound": "hbm", "achieved": nbytes / kernels[dom]["us"] / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(dom)
+    roof["launch_us"] = kernels[dom]["us"]
+
+    result = {
+        "metric": "fwd+bwd Mtokens/s of bimamba_chunk_scan_combined; % HBM/MFMA roofline",
+        "value": tokens / t_step / 1e6,
+        "unit": "Mtokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": t_step * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "bimamba_chunk_scan_combined fwd+bwd, batch 4 x seqlen 2048 x 32 heads x headdim 64, "
+                               "ngroups 1, dstate 64, chunk 256, bf16 x/B/C/z + fp32 dt/A/D/dt_bias, "
+                               + ("z gate, " if has_z else "no z, ") + "D (nheads,), dt_bias + softplus",
+                   **w, "has_z": has_z},
+        "roofline": roof,
+        "whole_op": {"fwd_ms": t_fwd * 1e3, "fwd_Mtokens_s": tokens / t_fwd / 1e6,
+                     "fwd_bwd_alg_MB": (fwd_b + bwd_b) / 1e6,
+                     "fwd_bwd_hbm_frac": (fwd_b + bwd_b) / t_step / (HBM_PEAK_GBS * 1e9),
+                     "fwd_hbm_frac": fwd_b / t_fwd / (HBM_PEAK_GBS * 1e9),
+                     "sum_kernel_us": round(sum(k["us"] for k in kernels.values()), 1)},
+        "kernels": kernels,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

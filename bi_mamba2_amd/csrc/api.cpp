@@ -79,10 +79,11 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
         need_f(q->u_b, bhcq);
         need_f(q->v_f, bhcq);
         need_f(q->v_b, bhcq);
-        need_f(q->da_intra, bhcq * nqt);
+        need_f(q->da_intra, (size_t)q->batch * q->nheads * nc * nqt * nqt * 128);
         need_f(q->ddA_chunk_f, (size_t)q->batch * q->nheads * nc * sp_nsplit(q));
         need_f(q->ddA_chunk_b, (size_t)q->batch * q->nheads * nc * sp_nsplit(q));
-        const size_t bn = (size_t)q->batch * q->seqlen * q->ngroups * q->dstate;
+        const size_t slices = (q->nheads / q->ngroups + 3) / 4;   // head slices of the dB / dC partial sums
+        const size_t bn = slices * q->batch * q->seqlen * q->ngroups * q->dstate;
         need_f(q->dBs, bn);
         need_f(q->dCs, bn);
         const size_t red = std::max((size_t)q->batch * nc * rt * q->nheads * q->headdim, (size_t)2 * q->batch * nc * q->nheads);

@@ -55,16 +55,18 @@ template <> struct Mma<f16_t> {
 // acc[j] += A(16 rows at As) * B(16 cols at Bs + 16*j rows)^T over one BK-wide LDS tile.
 // As points at the first of the wave's 16 rows ([row][k], leading dimension LD); Bs at the first of NJ*16
 // columns stored [col][k].
-template <typename T, int NJ>
+// KW is the K extent of the LDS tiles (multiple of BK); their leading dimension is KW + (LD - BK).
+template <typename T, int NJ, int KW = BK>
 __device__ __forceinline__ void mma_tile(f32x4 (&acc)[NJ], const T *As, const T *Bs, int lane) {
     typedef Mma<T> M;
+    constexpr int LD = M::LD - BK + KW;
     const int r = lane & 15, kq = (lane >> 4) * M::KPL;
 #pragma unroll
-    for (int k0 = 0; k0 < BK; k0 += M::KSTEP) {
-        typename M::Frag a = M::load(As + r * M::LD + k0 + kq);
+    for (int k0 = 0; k0 < KW; k0 += M::KSTEP) {
+        typename M::Frag a = M::load(As + r * LD + k0 + kq);
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            typename M::Frag b = M::load(Bs + (16 * j + r) * M::LD + k0 + kq);
+            typename M::Frag b = M::load(Bs + (16 * j + r) * LD + k0 + kq);
             acc[j] = M::mma(a, b, acc[j]);
         }
     }
@@ -80,11 +82,11 @@ template <typename S> __device__ __forceinline__ bool aligned16(const S *p, int6
     return ((reinterpret_cast<uintptr_t>(p) | static_cast<uintptr_t>(stride_elems * sizeof(S))) & 15) == 0;
 }
 
-// dst[r][k] = f(r, k, src[r*rs + k]) for r < ROWS, k < BK; elements with r >= rvalid or k >= kvalid are 0
+// dst[r][k] = f(r, k, src[r*rs + k]) for r < ROWS, k < KW; elements with r >= rvalid or k >= kvalid are 0
 // (f is still applied to the 0).  Source is contiguous along k.
-template <typename T, typename S, int ROWS, class F>
+template <typename T, typename S, int ROWS, int KW = BK, class F>
 __device__ __forceinline__ void tile_load_kcontig(T *dst, const S *src, int64_t rs, int rvalid, int kvalid, F f) {
-    constexpr int VS = 16 / sizeof(S), KV = BK / VS, LD = Mma<T>::LD;
+    constexpr int VS = 16 / sizeof(S), KV = KW / VS, LD = Mma<T>::LD - BK + KW;
     const bool vec = aligned16(src, rs);
     for (int idx = threadIdx.x; idx < ROWS * KV; idx += NTHREADS) {
         const int r = idx / KV, k0 = (idx % KV) * VS;
@@ -160,10 +162,15 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
     return v;
 }
-// sum over the 16 lanes that share l/16 (one row group of an MFMA output tile)
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// sum over the 16 lanes that share l/16 (one row group of an MFMA output tile); every lane gets the sum
 __device__ __forceinline__ float row16_sum(float v) {
-#pragma unroll
-    for (int d = 8; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+    v += dpp_mov<0x128>(v);  // row_ror:8
+    v += dpp_mov<0x124>(v);  // row_ror:4
+    v += dpp_mov<0x122>(v);  // row_ror:2
+    v += dpp_mov<0x121>(v);  // row_ror:1
     return v;
 }
 // inclusive prefix / suffix sums over the 64 lanes

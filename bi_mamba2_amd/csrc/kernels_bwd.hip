@@ -179,6 +179,9 @@ int launch_state_passing_bwd(const bimamba2_params *p) {
 //   tmp_f = x_h[r,:] . dS_f[h],  dBs[r,n] += dt[r] (e^{cs_f[Q-1]-cs_f[r]} tmp_f + e^{cs_b[0]-cs_b[r]} tmp_b)
 //   v_f[h,r] = dt[r] e^{cs_f[Q-1]-cs_f[r]} sum_n tmp_f[r,n] B[r,n]
 // =========================================================================================================
+constexpr int DBDC_HEADS = 4;
+static inline int dbdc_slices(const bimamba2_params *p) { return (p->nheads / p->ngroups + DBDC_HEADS - 1) / DBDC_HEADS; }
+
 template <typename T, int NT, bool IS_DB>
 __global__ __launch_bounds__(NTHREADS) void bwd_dbdc_kernel(const bimamba2_params p, int nc) {
     constexpr int LD = Mma<T>::LD;
@@ -208,7 +211,10 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dbdc_kernel(const bimamba2_param
                 creg[nt][j][i] = (r0 + rl < limit && n < N) ? to_f(cbp[(int64_t)rl * cbs + n]) : 0.f;
             }
     f32x4 tot[NT][4] = {};
-    for (int hh = 0; hh < hpg; ++hh) {
+    // blockIdx.z selects a slice of DBDC_HEADS heads of the group; its partial sum goes to slice blockIdx.z of the
+    // output, and bmm_chunk_bwd adds the slices up
+    const int hh_end = min(hpg, ((int)blockIdx.z + 1) * DBDC_HEADS);
+    for (int hh = blockIdx.z * DBDC_HEADS; hh < hh_end; ++hh) {
         const int h = g * hpg + hh;
         const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
         __syncthreads();
@@ -276,7 +282,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dbdc_kernel(const bimamba2_param
             }
         }
     }
-    float *out = (IS_DB ? p.dBs : p.dCs);
+    float *out = (IS_DB ? p.dBs : p.dCs) + (int64_t)blockIdx.z * p.batch * p.seqlen * p.ngroups * N;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -292,7 +298,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dbdc_kernel(const bimamba2_param
 template <typename T, bool IS_DB>
 static int launch_dbdc_t(const bimamba2_params *p) {
     const int nc = nchunks(p);
-    dim3 grid((p->chunk_size + 63) / 64, p->batch * nc * p->ngroups);
+    dim3 grid((p->chunk_size + 63) / 64, p->batch * nc * p->ngroups, dbdc_slices(p));
     const int nt = (p->dstate + 63) / 64;
     if (nt == 1) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 1, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
     else if (nt == 2) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 2, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
@@ -311,183 +317,183 @@ int launch_bwd_dbdc(const bimamba2_params *p, bool is_db) {
 }
 
 // =========================================================================================================
-// G[t,s] = dy_h[t,:] . x_h[s,:]  (K = headdim) for a 64-row tile of t and all s of the chunk, per head:
+// One workgroup owns one 64x64 tile (tt, st) of the chunk's (t, s) plane for one (b, c, g) and loops over the
+// heads of the group.  Per head, G[t,s] = dy_h[t,:] . x_h[s,:] (K = headdim), then
 //   f[t,s] = 1[s<=t] G dt[s] e^{cs_f[t]-cs_f[s]},  b[t,s] = 1[s>=t] G dt[s] e^{cs_b[t]-cs_b[s]}
-//   dCB[t,s] = sum_{h in group} (f + b)
-//   da_intra[h, i] = sum_{t>=i} sum_{s<i} f[t,s] CB[t,s]  +  sum_{t<=i} sum_{s>i} b[t,s] CB[t,s]
-// The row prefix (resp. suffix) over s runs across the 16 lanes of an MFMA row group with DPP adds and is
-// carried from column tile to column tile, ascending s for the forward direction, descending for the reverse.
-// Output da_intra[b, h, c, tt, Q] holds this row tile's share; the consumer sums over tt.
+//   dCB[t,s] = sum_{h in group} (f + b)                       (kept in registers across the head loop)
+//   W_f = 1[s<t] f CB,  W_b = 1[s>t] b CB                     (what the within-chunk gradient of dt*A is made of)
+// The within-chunk gradient  da[i] = sum_{t>=i>s} W_f[t,s] + sum_{t<=i<s} W_b[t,s]  is assembled by the consumer
+// (chunk_cumsum_bwd) from per-tile vectors written here to da_intra[b, h, c, tile, 2, 64]:
+//   off-diagonal tile: [0] = column sums cw[s] = sum_t W,  [1] = row sums rw[t] = sum_s W
+//   diagonal tile    : [0] = the tile's complete contribution to da[i] (row prefix / suffix with DPP), [1] = 0
 // =========================================================================================================
-template <typename T, int QT>
-__global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params p, int nc) {
-    constexpr int LD = Mma<T>::LD;
+template <typename T>
+__global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params p, int nc, int nqt) {
+    constexpr int KW = 64, LD = Mma<T>::LD - BK + KW;
     __shared__ __attribute__((aligned(16))) T As[64 * LD];
     __shared__ __attribute__((aligned(16))) T Bs[64 * LD];
-    __shared__ float csf[BIMAMBA2_MAX_CHUNK], csb[BIMAMBA2_MAX_CHUNK], dts[BIMAMBA2_MAX_CHUNK];
-    __shared__ float red[4][QT * 64];
+    __shared__ float csf_t[64], csb_t[64], csf_s[64], csb_s[64], dt_s[64];
+    __shared__ float red[4][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int tt = blockIdx.x;
+    const int tt = blockIdx.x / nqt, st = blockIdx.x % nqt;
     const int g = blockIdx.y % p.ngroups, bc = blockIdx.y / p.ngroups, c = bc % nc, b = bc / nc;
     const int Q = p.chunk_size, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
     const int limit = min(Q, p.seqlen - c * Q);
-    const int t0 = tt * 64;
-    const int nqt = (Q + 63) / 64;
+    const int t0 = tt * 64, s0 = st * 64;
+    const bool live = t0 < limit && s0 < limit;
     const float *cbg = p.CB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
-    int trow[4];
+    int tl[4];     // local row of this lane's accumulator elements
 #pragma unroll
-    for (int i = 0; i < 4; ++i) trow[i] = t0 + wave * 16 + (lane >> 4) * 4 + i;
-    f32x4 cbr[QT][4], dcb[QT][4] = {};
+    for (int i = 0; i < 4; ++i) tl[i] = wave * 16 + (lane >> 4) * 4 + i;
+    f32x4 cbr[4], dcb[4] = {};
 #pragma unroll
-    for (int st = 0; st < QT; ++st)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int s = st * 64 + j * 16 + (lane & 15);
-                cbr[st][j][i] = (trow[i] < Q && s < Q) ? cbg[(int64_t)trow[i] * Q + s] : 0.f;
-            }
+        for (int i = 0; i < 4; ++i) {
+            const int t = t0 + tl[i], s = s0 + j * 16 + (lane & 15);
+            cbr[j][i] = (t < Q && s < Q) ? cbg[(int64_t)t * Q + s] : 0.f;
+        }
     for (int hh = 0; hh < hpg; ++hh) {
         const int h = g * hpg + hh;
         const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
+        float *tv = p.da_intra + ((o / Q) * nqt * nqt + blockIdx.x) * 128;
+        if (!live) {
+            if (threadIdx.x < 128) tv[threadIdx.x] = 0.f;
+            continue;
+        }
         __syncthreads();
-        for (int q = threadIdx.x; q < Q; q += NTHREADS) {
-            csf[q] = p.cs_f[o + q];
-            csb[q] = p.cs_b[o + q];
-            dts[q] = p.dt_out[o + q];
+        if (threadIdx.x < 64) {
+            const int t = min(t0 + (int)threadIdx.x, Q - 1);
+            csf_t[threadIdx.x] = p.cs_f[o + t];
+            csb_t[threadIdx.x] = p.cs_b[o + t];
+        } else if (threadIdx.x < 128) {
+            const int sl = threadIdx.x - 64, s = min(s0 + sl, Q - 1);
+            csf_s[sl] = p.cs_f[o + s];
+            csb_s[sl] = p.cs_b[o + s];
+            dt_s[sl] = p.dt_out[o + s];
         }
         const T *yp;
         int64_t ys;
-        if (p.has_z) { ys = (int64_t)H * P; yp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * ys + (int64_t)h * P; }
-        else { ys = p.dout_sl; yp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * ys + h * p.dout_sh; }
-        const T *xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh;
-        float col[QT][4];
+        if (p.has_z) { ys = (int64_t)H * P; yp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q + t0) * ys + (int64_t)h * P; }
+        else { ys = p.dout_sl; yp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + ((int64_t)c * Q + t0) * ys + h * p.dout_sh; }
+        const T *xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + ((int64_t)c * Q + s0) * p.x_sl + h * p.x_sh;
+        f32x4 acc[4] = {};
+        for (int k0 = 0; k0 < P; k0 += KW) {
+            if (k0) __syncthreads();
+            tile_load_kcontig<T, T, 64, KW>(As, yp + k0, ys, limit - t0, P - k0, Ident());
+            tile_load_kcontig<T, T, 64, KW>(Bs, xp + k0, p.x_sl, limit - s0, P - k0, Ident());
+            __syncthreads();
+            mma_tile<T, 4, KW>(acc, As + wave * 16 * LD, Bs, lane);
+        }
+        float cft[4], cbt[4];
 #pragma unroll
-        for (int st = 0; st < QT; ++st)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) col[st][j] = 0.f;
-
-        auto gtile = [&](int st, f32x4(&acc)[4]) {
-            for (int k0 = 0; k0 < P; k0 += BK) {
-                __syncthreads();
-                tile_load_kcontig<T, T, 64>(As, yp + (int64_t)t0 * ys + k0, ys, limit - t0, P - k0, Ident());
-                tile_load_kcontig<T, T, 64>(Bs, xp + (int64_t)st * 64 * p.x_sl + k0, p.x_sl, limit - st * 64, P - k0, Ident());
-                __syncthreads();
-                mma_tile<T, 4>(acc, As + wave * 16 * LD, Bs, lane);
-            }
-        };
-        float csft[4], csbt[4];
-        // (cs vectors were written before the first barrier inside gtile; read them after it)
-        // ---- ascending pass: forward direction, column tiles st <= tt ----
-        float carry[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int st = 0; st < QT; ++st) {
-            if (st > tt || st * 64 >= limit) continue;
-            f32x4 acc[4] = {};
-            gtile(st, acc);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { csft[i] = csf[min(trow[i], Q - 1)]; csbt[i] = csb[min(trow[i], Q - 1)]; }
+        for (int i = 0; i < 4; ++i) { cft[i] = csf_t[tl[i]]; cbt[i] = csb_t[tl[i]]; }
+        if (st != tt) {
+            // one direction only: forward below the diagonal, reverse above it
+            float rw[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int s = st * 64 + j * 16 + (lane & 15);
-                const int sc = min(s, Q - 1);
-                const float dtv = dts[sc], cfs = csf[sc], cbs_ = csb[sc];
+                const int sl = j * 16 + (lane & 15);
+                const float dtv = dt_s[sl], cs = st < tt ? csf_s[sl] : csb_s[sl];
+                float cw = 0.f;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const int t = trow[i];
+                    const float v = acc[j][i] * dtv * __expf((st < tt ? cft[i] : cbt[i]) - cs);
+                    dcb[j][i] += v;
+                    const float w = v * cbr[j][i];
+                    cw += w;
+                    rw[i] += w;
+                }
+                cw += __shfl_xor(cw, 16, 64);
+                cw += __shfl_xor(cw, 32, 64);
+                if (lane < 16) red[wave][j * 16 + lane] = cw;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float r = row16_sum(rw[i]);
+                if ((lane & 15) == 0) tv[64 + tl[i]] = r;
+            }
+        } else {
+            float col[4] = {0.f, 0.f, 0.f, 0.f};
+            float wf[4][4], wb[4][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int sl = j * 16 + (lane & 15);
+                const float dtv = dt_s[sl], cfs = csf_s[sl], cbs = csb_s[sl];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
                     const float gv = acc[j][i] * dtv;
-                    const float f = (s <= t) ? gv * __expf(csft[i] - cfs) : 0.f;
-                    float both = f;
-                    if (st == tt) both += (s >= t) ? gv * __expf(csbt[i] - cbs_) : 0.f;
-                    dcb[st][j][i] += both;
-                    const float w = (s < t) ? f * cbr[st][j][i] : 0.f;
-                    const float incl = row16_incl_prefix(w);
-                    const float excl = carry[i] + incl - w;
-                    if (t >= s) col[st][j] += excl;
+                    const float f = (sl <= tl[i]) ? gv * __expf(cft[i] - cfs) : 0.f;
+                    const float r = (sl >= tl[i]) ? gv * __expf(cbt[i] - cbs) : 0.f;
+                    dcb[j][i] += f + r;
+                    wf[j][i] = (sl < tl[i]) ? f * cbr[j][i] : 0.f;
+                    wb[j][i] = (sl > tl[i]) ? r * cbr[j][i] : 0.f;
+                }
+            }
+            float carry[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int sl = j * 16 + (lane & 15);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float w = wf[j][i];
+                    const float excl = carry[i] + row16_incl_prefix(w) - w;   // sum over s' < s of this row
+                    if (tl[i] >= sl) col[j] += excl;
                     carry[i] += row16_sum(w);
                 }
             }
-        }
-        // ---- descending pass: reverse direction, column tiles st >= tt ----
 #pragma unroll
-        for (int i = 0; i < 4; ++i) carry[i] = 0.f;
-#pragma unroll
-        for (int st = QT - 1; st >= 0; --st) {
-            if (st < tt || st * 64 >= limit) continue;
-            f32x4 acc[4] = {};
-            gtile(st, acc);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) csbt[i] = csb[min(trow[i], Q - 1)];
+            for (int i = 0; i < 4; ++i) carry[i] = 0.f;
 #pragma unroll
             for (int j = 3; j >= 0; --j) {
-                const int s = st * 64 + j * 16 + (lane & 15);
-                const int sc = min(s, Q - 1);
-                const float dtv = dts[sc], cbs_ = csb[sc];
+                const int sl = j * 16 + (lane & 15);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const int t = trow[i];
-                    const float gv = acc[j][i] * dtv;
-                    const float bv = (s >= t) ? gv * __expf(csbt[i] - cbs_) : 0.f;
-                    if (st != tt) dcb[st][j][i] += bv;
-                    const float w = (s > t) ? bv * cbr[st][j][i] : 0.f;
-                    const float incl = row16_incl_suffix(w);
-                    const float excl = carry[i] + incl - w;
-                    if (t <= s) col[st][j] += excl;
+                    const float w = wb[j][i];
+                    const float excl = carry[i] + row16_incl_suffix(w) - w;   // sum over s' > s of this row
+                    if (tl[i] <= sl) col[j] += excl;
                     carry[i] += row16_sum(w);
                 }
             }
-        }
-        // ---- column sums over the 64 rows of this tile ----
-#pragma unroll
-        for (int st = 0; st < QT; ++st)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                float v = col[st][j];
+                float v = col[j];
                 v += __shfl_xor(v, 16, 64);
                 v += __shfl_xor(v, 32, 64);
-                if (lane < 16) red[wave][st * 64 + j * 16 + lane] = v;
+                if (lane < 16) red[wave][j * 16 + lane] = v;
             }
+            if (threadIdx.x < 64) tv[64 + threadIdx.x] = 0.f;
+        }
         __syncthreads();
-        for (int q = threadIdx.x; q < Q; q += NTHREADS)
-            p.da_intra[(o * nqt) + (int64_t)tt * Q + q] = red[0][q] + red[1][q] + red[2][q] + red[3][q];
+        if (threadIdx.x < 64) tv[threadIdx.x] = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
     }
     float *out = p.dCB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
 #pragma unroll
-    for (int st = 0; st < QT; ++st)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int s = st * 64 + j * 16 + (lane & 15);
-                if (trow[i] < Q && s < Q) out[(int64_t)trow[i] * Q + s] = dcb[st][j][i];
-            }
-}
-
-template <typename T>
-static int launch_dcb_t(const bimamba2_params *p) {
-    const int nc = nchunks(p), qt = (p->chunk_size + 63) / 64;
-    dim3 grid(qt, p->batch * nc * p->ngroups);
-    if (qt == 1) hipLaunchKernelGGL((bwd_dcb_kernel<T, 1>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
-    else if (qt == 2) hipLaunchKernelGGL((bwd_dcb_kernel<T, 2>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
-    else if (qt <= 4) hipLaunchKernelGGL((bwd_dcb_kernel<T, 4>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
-    else return BIMAMBA2_EUNSUPPORTED;
-    return check_launch();
+        for (int i = 0; i < 4; ++i) {
+            const int t = t0 + tl[i], s = s0 + j * 16 + (lane & 15);
+            if (t < Q && s < Q) out[(int64_t)t * Q + s] = dcb[j][i];
+        }
 }
 
 int launch_bwd_dcb(const bimamba2_params *p) {
+    const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
+    dim3 grid(nqt * nqt, p->batch * nc * p->ngroups);
     switch (p->dtype) {
-        case BIMAMBA2_F32: return launch_dcb_t<float>(p);
-        case BIMAMBA2_BF16: return launch_dcb_t<bf16_t>(p);
-        case BIMAMBA2_F16: return launch_dcb_t<f16_t>(p);
+        case BIMAMBA2_F32: hipLaunchKernelGGL(bwd_dcb_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL(bwd_dcb_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL(bwd_dcb_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt); break;
         default: return BIMAMBA2_EUNSUPPORTED;
     }
+    return check_launch();
 }
 
 // =========================================================================================================
 // which = 0 : dB[s,n] = dBs[s,n] + sum_t dCB[t,s] C[t,n]      which = 1 : dC[t,n] = dCs[t,n] + sum_s dCB[t,s] B[s,n]
 // =========================================================================================================
 template <typename T>
-__global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_params p, int nc) {
+__global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_params p, int nc, int nslices) {
     constexpr int LD = Mma<T>::LD;
     __shared__ __attribute__((aligned(16))) T As[64 * LD];
     __shared__ __attribute__((aligned(16))) T Bs[64 * LD];
@@ -521,7 +527,9 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
             const int r = r0 + wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
             if (r < limit && n < N) {
                 const int64_t a = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n;
-                out[a] = from_f<T>(acc[j][i] + res[a]);
+                float v = acc[j][i];
+                for (int sl = 0; sl < nslices; ++sl) v += res[a + (int64_t)sl * p.batch * p.seqlen * p.ngroups * N];
+                out[a] = from_f<T>(v);
             }
         }
 }
@@ -530,9 +538,9 @@ int launch_bmm_chunk_bwd(const bimamba2_params *p) {
     const int nc = nchunks(p);
     dim3 grid((p->dstate + 63) / 64, (p->chunk_size + 63) / 64, p->batch * nc * p->ngroups * 2);
     switch (p->dtype) {
-        case BIMAMBA2_F32: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
-        case BIMAMBA2_BF16: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
-        case BIMAMBA2_F16: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc); break;
+        case BIMAMBA2_F32: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p)); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p)); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p)); break;
         default: return BIMAMBA2_EUNSUPPORTED;
     }
     return check_launch();
@@ -540,7 +548,7 @@ int launch_bmm_chunk_bwd(const bimamba2_params *p) {
 
 // =========================================================================================================
 // one wave per (b, c, h); lane i owns positions 4i..4i+3.
-//   da[q] = sum_tt da_intra[tt][q] + sum_{s<q} v_f[s] + sum_{s>q} v_b[s] + sum_{t>=q} u_f[t] + sum_{t<=q} u_b[t]
+//   da[q] = (within-chunk part from the tile vectors in da_intra) + sum_{s<q} v_f[s] + sum_{s>q} v_b[s] + sum_{t>=q} u_f[t] + sum_{t<=q} u_b[t]
 //           + ddA_chunk_f + ddA_chunk_b
 //   ddt' = da*A + ddt_direct ; through clamp and softplus -> ddt ; dA += sum da*dt' ; ddt_bias += sum ddt
 // Partials per (b, c) go to red[(b*nc + c)*H + h] (dA) and red[B*nc*H + ...] (ddt_bias).
@@ -562,9 +570,54 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
         vb[e] = ok ? p.v_b[o + q] : 0.f;
         uf[e] = ok ? p.u_f[o + q] : 0.f;
         ub[e] = ok ? p.u_b[o + q] : 0.f;
-        float s = 0.f;
-        if (ok) for (int t = 0; t < nqt; ++t) s += p.da_intra[o * nqt + (int64_t)t * Q + q];
-        di[e] = s;
+        di[e] = 0.f;
+    }
+    // within-chunk part from the per-tile vectors of bwd_dcb_kernel; tile I = lane / 16 holds this lane's positions
+    {
+        const int I = lane >> 4, i0 = (lane & 15) * 4;
+        if (I < nqt) {
+            const float *tv = p.da_intra + (o / Q) * nqt * nqt * 128;
+            auto vec = [&](int tile, int which, float (&r)[4], bool add) {
+                const float4 v = *reinterpret_cast<const float4 *>(tv + (tile * 2 + which) * 64 + i0);
+                if (add) { r[0] += v.x; r[1] += v.y; r[2] += v.z; r[3] += v.w; }
+                else { r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w; }
+            };
+            float d[4];
+            vec(I * nqt + I, 0, d, false);
+            float cwf[4] = {0.f, 0.f, 0.f, 0.f}, rwf[4] = {0.f, 0.f, 0.f, 0.f};
+            float cwb[4] = {0.f, 0.f, 0.f, 0.f}, rwb[4] = {0.f, 0.f, 0.f, 0.f};
+            float between = 0.f;
+            for (int a = 0; a < nqt; ++a) {
+                if (a > I) { vec(a * nqt + I, 0, cwf, true); vec(I * nqt + a, 1, rwb, true); }
+                if (a < I) { vec(I * nqt + a, 1, rwf, true); vec(a * nqt + I, 0, cwb, true); }
+            }
+            // tiles with this tile strictly between their row tile and column tile add their total
+            for (int a = 0; a < nqt; ++a)
+                for (int bq = 0; bq < nqt; ++bq)
+                    if ((bq < I && I < a) || (a < I && I < bq)) {
+                        float t4[4];
+                        vec(a * nqt + bq, 0, t4, false);
+                        between += t4[0] + t4[1] + t4[2] + t4[3];
+                    }
+            between = row16_sum(between);
+            // forward: exclusive prefix of cwf + inclusive suffix of rwf; reverse: inclusive prefix of rwb + exclusive suffix of cwb
+            const float t_cwf = cwf[0] + cwf[1] + cwf[2] + cwf[3], t_rwb = rwb[0] + rwb[1] + rwb[2] + rwb[3];
+            const float t_rwf = rwf[0] + rwf[1] + rwf[2] + rwf[3], t_cwb = cwb[0] + cwb[1] + cwb[2] + cwb[3];
+            float ex = row16_incl_prefix(t_cwf) - t_cwf, in = row16_incl_prefix(t_rwb) - t_rwb;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                in += rwb[e];
+                di[e] = d[e] + between + ex + in;
+                ex += cwf[e];
+            }
+            float exs = row16_incl_suffix(t_cwb) - t_cwb, ins = row16_incl_suffix(t_rwf) - t_rwf;
+#pragma unroll
+            for (int e = 3; e >= 0; --e) {
+                ins += rwf[e];
+                di[e] += exs + ins;
+                exs += cwb[e];
+            }
+        }
     }
     float chunk_term = 0.f;
     for (int s = 0; s < nsplit; ++s)

@@ -143,6 +143,11 @@ def _check_chunk(chunk_size):
     assert chunk_size >= 32, "chunk_size must be at least 32 (as in the reference) and at most 256"
 
 
+def _slices(nheads, ngroups):
+    """Number of head slices whose partial dB / dC sums the kernels keep apart (4 heads per slice)."""
+    return (nheads // ngroups + 3) // 4
+
+
 def _bhcq(c):
     return (c.p.batch, c.p.nheads, c.nchunks, c.p.chunk_size)
 
@@ -309,7 +314,8 @@ def _chunk_state_bwd_db(x, dt, dA_cumsum_f, dA_cumsum_b, dstates_f, dstates_b, B
     c.set_x(x); c.set_B(B)
     c.put("dt_out", dt, torch.float32); c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     c.put("dstates_f", dstates_f, torch.float32); c.put("dstates_b", dstates_b, torch.float32)
-    dBs = torch.zeros(batch, seqlen, ngroups, dstate, device=x.device, dtype=torch.float32); c.put("dBs", dBs)
+    dBs = torch.zeros(_slices(nheads, ngroups), batch, seqlen, ngroups, dstate, device=x.device, dtype=torch.float32)
+    c.put("dBs", dBs)
     vf = c.new("v_f", _bhcq(c)); vb = c.new("v_b", _bhcq(c))
     c.run("bimamba2_chunk_state_bwd_db")
     return dBs, vf, vb
@@ -325,15 +331,17 @@ def _chunk_scan_bwd_dC(states_f, states_b, dA_cumsum_f, dA_cumsum_b, dout, C=Non
     c.set_dout(dout); c.set_C(C)
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     c.put("states_f", states_f, torch.float32); c.put("states_b", states_b, torch.float32)
-    dCs = torch.zeros(batch, seqlen, ngroups, dstate, device=dout.device, dtype=torch.float32); c.put("dCs", dCs)
+    dCs = torch.zeros(_slices(nheads, ngroups), batch, seqlen, ngroups, dstate, device=dout.device, dtype=torch.float32)
+    c.put("dCs", dCs)
     uf = c.new("u_f", _bhcq(c)); ub = c.new("u_b", _bhcq(c))
     c.run("bimamba2_chunk_scan_bwd_dc")
     return dCs, uf, ub
 
 
 def _chunk_scan_bwd_dcb(x, dt, dA_cumsum_f, dA_cumsum_b, dout, CB, ngroups=1):
-    """-> dCB (batch, nchunks, ngroups, Q, Q) float32 and the within-chunk part of d(dt*A)
-    (batch, nheads, nchunks, Q) (the reference's ddA_f + ddA_b of its two "stable" kernels)."""
+    """-> dCB (batch, nchunks, ngroups, Q, Q) float32 and the per-tile vectors (batch, nheads, nchunks, tiles, 2, 64)
+    from which chunk_cumsum_bwd assembles the within-chunk part of d(dt*A) (the reference's ddA_f + ddA_b of
+    its two "stable" kernels): column / row sums of off-diagonal 64x64 tiles, full contribution of diagonal ones."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape
     c = _Call(batch, seqlen, nheads, headdim, ngroups, 1, chunk_size, x.dtype, x.device)
@@ -342,16 +350,18 @@ def _chunk_scan_bwd_dcb(x, dt, dA_cumsum_f, dA_cumsum_b, dout, CB, ngroups=1):
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     dCB = c.new("dCB", (batch, nchunks, ngroups, chunk_size, chunk_size))
     nqt = (chunk_size + 63) // 64
-    da = c.new("da_intra", (batch, nheads, nchunks, nqt, chunk_size))
+    da = c.new("da_intra", (batch, nheads, nchunks, nqt * nqt, 2, 64))
     c.run("bimamba2_chunk_scan_bwd_dcb")
-    return dCB, da.sum(3)
+    return dCB, da
 
 
 def _bmm_chunk_bwd(B, C, dCB, dBs, dCs):
-    """dB = dBs + dCB^T.C and dC = dCs + dCB.B per chunk, in the dtype of B / C."""
+    """dB = sum(dBs) + dCB^T.C and dC = sum(dCs) + dCB.B per chunk, in the dtype of B / C; dBs, dCs are the
+    (slices, batch, seqlen, ngroups, dstate) partial sums of _chunk_state_bwd_db / _chunk_scan_bwd_dC."""
     batch, seqlen, ngroups, dstate = B.shape
     chunk_size = dCB.shape[-1]
-    c = _Call(batch, seqlen, ngroups, 1, ngroups, dstate, chunk_size, B.dtype, B.device)
+    # nheads is only used to tell the kernel how many slices to add up
+    c = _Call(batch, seqlen, ngroups * 4 * dBs.shape[0], 1, ngroups, dstate, chunk_size, B.dtype, B.device)
     c.set_B(B); c.set_C(C)
     c.put("dCB", dCB, torch.float32); c.put("dBs", dBs, torch.float32); c.put("dCs", dCs, torch.float32)
     dB = torch.zeros(B.shape, device=B.device, dtype=B.dtype); c.put("dB", dB)

@@ -77,9 +77,10 @@ typedef struct bimamba2_params {
     float *states_f, *states_b;     /* chunk states, overwritten in place by the inter-chunk scan */
     float *dstates_f, *dstates_b;
     void *dout_x;                   /* dout * silu(z), element type `dtype` */
-    float *ddt_direct, *u_f, *u_b, *v_f, *v_b, *da_intra;
-    float *ddA_chunk_f, *ddA_chunk_b;   /* (B, H, nc) */
-    float *dBs, *dCs;                   /* (B, L, G, N) float32 partial gradients */
+    float *ddt_direct, *u_f, *u_b, *v_f, *v_b;
+    float *da_intra;                    /* (B, H, nc, T*T, 2, 64), T = ceil(Q/64): per-tile column / row sums */
+    float *ddA_chunk_f, *ddA_chunk_b;   /* (B, H, nc, ceil(P*N/1024)) partial sums */
+    float *dBs, *dCs;                   /* (S, B, L, G, N) float32 partial gradients, S = ceil(H/G/4) head slices */
     float *red;                         /* scratch for two-stage reductions */
     void *workspace;
     size_t workspace_bytes;
