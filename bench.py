@@ -174,7 +174,7 @@ def main():
     nqt = (w["chunk_size"] + 63) // 64
     c.new("da_intra", bhcq[:3] + (nqt * nqt, 2, 64))
     cbs = (w["batch"], nc, w["ngroups"], w["chunk_size"], w["chunk_size"])
-    c.new("CB", cbs); c.new("dCB", cbs)
+    c.new("CB", cbs); c.new("dCB", cbs); c.new("CBT", cbs)
     sts = (w["batch"], nc, w["nheads"], w["headdim"], w["dstate"])
     for f in ("states_f", "states_b", "dstates_f", "dstates_b"):
         c.new(f, sts)
@@ -184,7 +184,7 @@ def main():
     c.new("ddA_chunk_f", (w["batch"], w["nheads"], nc, nsplit)); c.new("ddA_chunk_b", (w["batch"], w["nheads"], nc, nsplit))
     slices = (w["nheads"] // w["ngroups"] + 3) // 4
     c.new("dBs", (slices,) + tuple(inp["B"].shape)); c.new("dCs", (slices,) + tuple(inp["B"].shape))
-    c.new("red", (max(w["batch"] * nc * ((w["chunk_size"] + 63) // 64) * w["nheads"] * w["headdim"], 2 * w["batch"] * nc * w["nheads"]),))
+    c.new("red", (max(w["batch"] * nc * w["nheads"] * w["headdim"], 2 * w["batch"] * nc * w["nheads"]),))
     c.run("bimamba2_fwd")
     c.run("bimamba2_bwd")
     torch.cuda.synchronize()

@@ -7,7 +7,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libbimamba2_hip.so")
+# BIMAMBA2_LIB lets a caller point at another build of the same library (e.g. an instrumented one)
+LIB_PATH = os.environ.get("BIMAMBA2_LIB") or os.path.join(_HERE, "libbimamba2_hip.so")
 
 F32, BF16, F16 = 0, 1, 2
 
@@ -25,7 +26,7 @@ class Params(ctypes.Structure):
         + [(n, _vp) for n in ("x", "dt", "Bm", "Cm", "z", "dout", "A", "D", "dt_bias",
                               "out", "out_x", "final_f", "final_b",
                               "dx", "ddt", "dB", "dC", "dz", "dA", "dD", "ddt_bias",
-                              "dt_out", "cs_f", "cs_b", "CB", "dCB", "states_f", "states_b",
+                              "dt_out", "cs_f", "cs_b", "CB", "dCB", "CBT", "states_f", "states_b",
                               "dstates_f", "dstates_b", "dout_x",
                               "ddt_direct", "u_f", "u_b", "v_f", "v_b", "da_intra",
                               "ddA_chunk_f", "ddA_chunk_b", "dBs", "dCs", "red", "workspace")]

@@ -68,8 +68,9 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     need_f(q->states_f, stn);
     need_f(q->states_b, stn);
     if (is_bwd) {
-        const size_t nqt = (Q + 63) / 64, rt = nqt;
+        const size_t nqt = (Q + 63) / 64;
         need_f(q->dCB, cbn);
+        need_f(q->CBT, cbn);
         need_f(q->dstates_f, stn);
         need_f(q->dstates_b, stn);
         if (q->has_z && !q->dout_x)
@@ -86,7 +87,7 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
         const size_t bn = slices * q->batch * q->seqlen * q->ngroups * q->dstate;
         need_f(q->dBs, bn);
         need_f(q->dCs, bn);
-        const size_t red = std::max((size_t)q->batch * nc * rt * q->nheads * q->headdim, (size_t)2 * q->batch * nc * q->nheads);
+        const size_t red = std::max((size_t)q->batch * nc * q->nheads * q->headdim, (size_t)2 * q->batch * nc * q->nheads);
         need_f(q->red, red);
     }
     return (cv.off + 255) & ~size_t(255);
@@ -175,18 +176,17 @@ int bimamba2_state_passing_bwd(const bimamba2_params *p) {
 
 int bimamba2_chunk_scan_bwd_dx(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->CB); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->CBT); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
     REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->dx); REQUIRE(p->ddt_direct);
     if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
     if (p->has_D) { REQUIRE(p->D); REQUIRE(p->dD); REQUIRE(p->red); }
     const int nc = nchunks(p);
-    if (p->headdim > 64)   // several headdim tiles add their row sums atomically
+    if (p->headdim > (p->dtype == BIMAMBA2_F32 ? 32 : 64))   // several headdim tiles add their row sums atomically
         TRY(launch_fill(p->ddt_direct, (size_t)p->batch * p->nheads * nc * p->chunk_size, 0.f, stream_of(p)));
     TRY(launch_chunk_scan(p, true));
     if (p->has_D) {
-        const int rt = (p->chunk_size + 63) / 64;
-        if (p->D_has_hdim) return launch_reduce(p->red, p->dD, p->batch * nc * rt, p->nheads * p->headdim, 1, stream_of(p));
-        return launch_reduce(p->red, p->dD, p->batch * nc * rt, p->nheads, p->headdim, stream_of(p));
+        if (p->D_has_hdim) return launch_reduce(p->red, p->dD, p->batch * nc, p->nheads * p->headdim, 1, stream_of(p));
+        return launch_reduce(p->red, p->dD, p->batch * nc, p->nheads, p->headdim, stream_of(p));
     }
     return BIMAMBA2_OK;
 }
@@ -231,6 +231,7 @@ int bimamba2_chunk_cumsum_bwd(const bimamba2_params *p) {
 int bimamba2_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     bimamba2_params q = *p;
+    q.CBT = nullptr;
     const size_t need = carve(&q, 0, p->workspace);
     if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
     TRY(bimamba2_chunk_cumsum_fwd(&q));

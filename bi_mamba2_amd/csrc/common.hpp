@@ -31,6 +31,7 @@ template <> struct Mma<float> {
     static constexpr int KPL = 1, KSTEP = 4, LD = BK + 4;
     typedef float Frag;
     static __device__ __forceinline__ Frag load(const float *p) { return *p; }
+    static __device__ __forceinline__ Frag pack(const float *a) { return a[0]; }
     static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
     }
@@ -39,6 +40,12 @@ template <> struct Mma<bf16_t> {
     static constexpr int KPL = 8, KSTEP = 32, LD = BK + 8;
     typedef bf16x8 Frag;
     static __device__ __forceinline__ Frag load(const bf16_t *p) { return *reinterpret_cast<const bf16x8 *>(p); }
+    static __device__ __forceinline__ Frag pack(const float *a) {
+        Frag f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = static_cast<bf16_t>(a[i]);
+        return f;
+    }
     static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
@@ -47,6 +54,12 @@ template <> struct Mma<f16_t> {
     static constexpr int KPL = 8, KSTEP = 32, LD = BK + 8;
     typedef f16x8 Frag;
     static __device__ __forceinline__ Frag load(const f16_t *p) { return *reinterpret_cast<const f16x8 *>(p); }
+    static __device__ __forceinline__ Frag pack(const float *a) {
+        Frag f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = static_cast<f16_t>(a[i]);
+        return f;
+    }
     static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
@@ -88,7 +101,7 @@ template <typename T, typename S, int ROWS, int KW = BK, class F>
 __device__ __forceinline__ void tile_load_kcontig(T *dst, const S *src, int64_t rs, int rvalid, int kvalid, F f) {
     constexpr int VS = 16 / sizeof(S), KV = KW / VS, LD = Mma<T>::LD - BK + KW;
     const bool vec = aligned16(src, rs);
-    for (int idx = threadIdx.x; idx < ROWS * KV; idx += NTHREADS) {
+    for (int idx = threadIdx.x; idx < ROWS * KV; idx += blockDim.x) {
         const int r = idx / KV, k0 = (idx % KV) * VS;
         float v[VS];
         if (vec && r < rvalid && k0 + VS <= kvalid) {
@@ -111,7 +124,7 @@ template <typename T, typename S, int ROWS, class F>
 __device__ __forceinline__ void tile_load_rcontig(T *dst, const S *src, int64_t ks, int rvalid, int kvalid, F f) {
     constexpr int VS = 16 / sizeof(S), RV = ROWS / VS, LD = Mma<T>::LD;
     const bool vec = aligned16(src, ks);
-    for (int idx = threadIdx.x; idx < BK * RV; idx += NTHREADS) {
+    for (int idx = threadIdx.x; idx < BK * RV; idx += blockDim.x) {
         const int k = idx / RV, r0 = (idx % RV) * VS;
         float v[VS];
         if (vec && k < kvalid && r0 + VS <= rvalid) {
@@ -133,7 +146,7 @@ __device__ __forceinline__ void tile_load_rcontig2(T *dst1, T *dst2, const S *sr
                                                    int kvalid, F1 f1, F2 f2) {
     constexpr int VS = 16 / sizeof(S), RV = ROWS / VS, LD = Mma<T>::LD;
     const bool vec = aligned16(src, ks);
-    for (int idx = threadIdx.x; idx < BK * RV; idx += NTHREADS) {
+    for (int idx = threadIdx.x; idx < BK * RV; idx += blockDim.x) {
         const int k = idx / RV, r0 = (idx % RV) * VS;
         float v[VS];
         if (vec && k < kvalid && r0 + VS <= rvalid) {
@@ -211,8 +224,9 @@ __device__ __forceinline__ float row16_incl_suffix(float v) {
     return v;
 }
 
-__device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
-__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + __expf(-z)); }
+// reciprocal by the hardware approximation (1 ulp) instead of a full division sequence
+__device__ __forceinline__ float sigmoid_f(float z) { return __builtin_amdgcn_rcpf(1.f + __expf(-z)); }
+__device__ __forceinline__ float silu_f(float z) { return z * sigmoid_f(z); }
 
 // chunk bookkeeping shared by all kernels
 struct ChunkIdx {

@@ -4,8 +4,7 @@
 //   chunk_state        per chunk and head: x^T . (B * decay * dt) for both directions (also used, with other
 //                      operands and weights, for the gradient of the chunk-entry states)
 //   state_passing_fwd  forward and reverse inter-chunk recurrences in one launch, in place
-//   chunk_scan         y = C.prev_f e^{cs_f} + C.prev_b e^{cs_b} + (CB * decay * dt) . x + D x, z gate
-//                      (its mirrored form computes dx in the backward pass)
+// (the chunk-scan kernel itself lives in kernels_scan.hip)
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -82,12 +81,16 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_fwd_kernel(const bimamba2_
         mma_tile<T, 4>(acc, As + wave * 16 * LD, Bs, lane);
     }
     float *out = p.CB + (int64_t)blockIdx.z * Q * Q;
+    float *outT = p.CBT ? p.CBT + (int64_t)blockIdx.z * Q * Q : nullptr;   // CBT[s, t] = CB[t, s], read by the dx kernel
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int t = tt * 64 + wave * 16 + (lane >> 4) * 4 + i, s = st * 64 + j * 16 + (lane & 15);
-            if (t < Q && s < Q) out[(int64_t)t * Q + s] = acc[j][i];
+            if (t < Q && s < Q) {
+                out[(int64_t)t * Q + s] = acc[j][i];
+                if (outT) outT[(int64_t)s * Q + t] = acc[j][i];
+            }
         }
 }
 
@@ -221,181 +224,6 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_kernel(const bimam
 }
 
 // =========================================================================================================
-// chunk scan (BWD = false), rows r = output positions t:
-//   acc[r,p] = e^{cs_f[r]} C_r.prev_f[p,:] + e^{cs_b[r]} C_r.prev_b[p,:]
-//            + sum_k CB[r,k] (1[k<=r] e^{cs_f[r]-cs_f[k]} + 1[k>=r] e^{cs_b[r]-cs_b[k]}) dt[k] x[k,p]
-//   out_x = acc + D x[r,p];  out = out_x * silu(z)
-// its mirror (BWD = true), rows r = input positions s:
-//   acc[r,p] = e^{cs_f[Q-1]-cs_f[r]} B_r.dS_f[p,:] + e^{cs_b[0]-cs_b[r]} B_r.dS_b[p,:]
-//            + sum_k CB[k,r] (1[k>=r] e^{cs_f[k]-cs_f[r]} + 1[k<=r] e^{cs_b[k]-cs_b[r]}) dy[k,p]
-//   dx = acc dt[r] + D dy[r,p];  ddt_direct[r] = sum_p acc x[r,p];  dD partial = sum_r dy x
-// =========================================================================================================
-template <typename T, bool BWD>
-__global__ __launch_bounds__(NTHREADS) void chunk_scan_kernel(const bimamba2_params p, int nc) {
-    constexpr int LD = Mma<T>::LD;
-    __shared__ __attribute__((aligned(16))) T As[64 * LD];
-    __shared__ __attribute__((aligned(16))) T B1[64 * LD];
-    __shared__ __attribute__((aligned(16))) T B2[64 * LD];
-    __shared__ float csf[BIMAMBA2_MAX_CHUNK], csb[BIMAMBA2_MAX_CHUNK], dts[BIMAMBA2_MAX_CHUNK];
-    __shared__ float red[4][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int pt = blockIdx.x, rt = blockIdx.y;
-    const int h = blockIdx.z % p.nheads, bc = blockIdx.z / p.nheads, c = bc % nc, b = bc / nc;
-    const int g = h / (p.nheads / p.ngroups);
-    const int Q = p.chunk_size, N = p.dstate, P = p.headdim;
-    const int limit = min(Q, p.seqlen - c * Q);
-    const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
-    for (int q = threadIdx.x; q < Q; q += NTHREADS) {
-        csf[q] = p.cs_f[o + q];
-        csb[q] = p.cs_b[o + q];
-        dts[q] = p.dt_out[o + q];
-    }
-    // ---- part 1: contribution of the states, K = dstate ----
-    const T *ap;
-    int64_t as;
-    if (BWD) { as = p.B_sl; ap = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + ((int64_t)c * Q + rt * 64) * as + g * p.B_sg; }
-    else { as = p.C_sl; ap = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + ((int64_t)c * Q + rt * 64) * as + g * p.C_sg; }
-    const float *s1 = (BWD ? p.dstates_f : p.states_f) + (int64_t)blockIdx.z * P * N + (int64_t)pt * 64 * N;
-    const float *s2 = (BWD ? p.dstates_b : p.states_b) + (int64_t)blockIdx.z * P * N + (int64_t)pt * 64 * N;
-    f32x4 acc[4] = {};
-    {
-        f32x4 accf[4] = {}, accb[4] = {};
-        for (int k0 = 0; k0 < N; k0 += BK) {
-            __syncthreads();
-            tile_load_kcontig<T, T, 64>(As, ap + k0, as, limit - rt * 64, N - k0, Ident());
-            tile_load_kcontig<T, float, 64>(B1, s1 + k0, N, P - pt * 64, N - k0, Ident());
-            tile_load_kcontig<T, float, 64>(B2, s2 + k0, N, P - pt * 64, N - k0, Ident());
-            __syncthreads();
-            mma_tile<T, 4>(accf, As + wave * 16 * LD, B1, lane);
-            mma_tile<T, 4>(accb, As + wave * 16 * LD, B2, lane);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = rt * 64 + wave * 16 + (lane >> 4) * 4 + i;
-            float sf = 0.f, sb = 0.f;
-            if (r < limit) {
-                sf = BWD ? __expf(csf[Q - 1] - csf[r]) : __expf(csf[r]);
-                sb = BWD ? __expf(csb[0] - csb[r]) : __expf(csb[r]);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j][i] = accf[j][i] * sf + accb[j][i] * sb;
-        }
-    }
-    // ---- part 2: inside the chunk, K = chunk positions ----
-    const float *cb = p.CB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
-    const T *kp;
-    int64_t ks;
-    if (!BWD) { ks = p.x_sl; kp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * ks + h * p.x_sh; }
-    else if (p.has_z) { ks = (int64_t)p.nheads * P; kp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * ks + (int64_t)h * P; }
-    else { ks = p.dout_sl; kp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * ks + h * p.dout_sh; }
-    const T *kp_tile = kp + pt * 64;
-    const int r0 = rt * 64;
-    for (int k0 = 0; k0 < limit; k0 += BK) {
-        __syncthreads();
-        if (!BWD) {
-            tile_load_kcontig<T, float, 64>(As, cb + (int64_t)r0 * Q + k0, Q, Q - r0, Q - k0, [&](int rl, int kl, float v) {
-                const int r = r0 + rl, k = k0 + kl;
-                if (r >= limit || k >= limit) return 0.f;
-                float m = 0.f;
-                if (k <= r) m += __expf(csf[r] - csf[k]);
-                if (k >= r) m += __expf(csb[r] - csb[k]);
-                return v * m * dts[k];
-            });
-        } else {
-            tile_load_rcontig<T, float, 64>(As, cb + (int64_t)k0 * Q + r0, Q, Q - r0, Q - k0, [&](int rl, int kl, float v) {
-                const int r = r0 + rl, k = k0 + kl;
-                if (r >= limit || k >= limit) return 0.f;
-                float m = 0.f;
-                if (k >= r) m += __expf(csf[k] - csf[r]);
-                if (k <= r) m += __expf(csb[k] - csb[r]);
-                return v * m;
-            });
-        }
-        tile_load_rcontig<T, T, 64>(B1, kp_tile + k0 * ks, ks, P - pt * 64, limit - k0, Ident());
-        __syncthreads();
-        mma_tile<T, 4>(acc, As + wave * 16 * LD, B1, lane);
-    }
-    // ---- epilogue ----
-    const int col0 = pt * 64 + (lane & 15);
-    if (!BWD) {
-        T *outp = reinterpret_cast<T *>(p.out);
-        T *outx = reinterpret_cast<T *>(p.out_x);
-        const T *xrow = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh;
-        const T *zrow = p.has_z ? reinterpret_cast<const T *>(p.z) + b * p.z_sb + (int64_t)c * Q * p.z_sl + h * p.z_sh : nullptr;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = r0 + wave * 16 + (lane >> 4) * 4 + i;
-            if (r >= limit) continue;
-            const int64_t orow = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.nheads + h) * P;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int col = col0 + j * 16;
-                if (col >= P) continue;
-                float v = acc[j][i];
-                if (p.has_D) v += (p.D_has_hdim ? p.D[h * P + col] : p.D[h]) * to_f(xrow[(int64_t)r * p.x_sl + col]);
-                if (p.has_z) {
-                    if (outx) outx[orow + col] = from_f<T>(v);
-                    v *= silu_f(to_f(zrow[(int64_t)r * p.z_sl + col]));
-                }
-                outp[orow + col] = from_f<T>(v);
-            }
-        }
-    } else {
-        T *dxp = reinterpret_cast<T *>(p.dx);
-        const T *xrow = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh;
-        float dsum[4] = {0.f, 0.f, 0.f, 0.f};   // per column tile j: sum over this lane's rows of dy*x
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = r0 + wave * 16 + (lane >> 4) * 4 + i;
-            const bool rok = r < limit;
-            const float dtr = rok ? dts[r] : 0.f;
-            const int64_t orow = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.nheads + h) * P;
-            float rs = 0.f;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int col = col0 + j * 16;
-                if (rok && col < P) {
-                    const float xv = to_f(xrow[(int64_t)r * p.x_sl + col]);
-                    const float a = acc[j][i];
-                    rs += a * xv;
-                    float v = a * dtr;
-                    if (p.has_D) {
-                        const float dy = to_f(kp[(int64_t)r * ks + col]);
-                        v += (p.D_has_hdim ? p.D[h * P + col] : p.D[h]) * dy;
-                        dsum[j] += dy * xv;
-                    }
-                    dxp[orow + col] = from_f<T>(v);
-                }
-            }
-            rs = row16_sum(rs);
-            if (rok && (lane & 15) == 0) {
-                // with more than one headdim tile the partial row sums are added atomically
-                if (gridDim.x == 1) p.ddt_direct[o + r] = rs;
-                else atomicAdd(p.ddt_direct + o + r, rs);
-            }
-        }
-        if (p.has_D) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float v = dsum[j];
-                v += __shfl_xor(v, 16, 64);
-                v += __shfl_xor(v, 32, 64);
-                if (lane < 16) red[wave][j * 16 + lane] = v;
-            }
-            __syncthreads();
-            if (threadIdx.x < 64) {
-                const int col = pt * 64 + threadIdx.x;
-                if (col < P) {
-                    const float v = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
-                    // partials: [(b*nc + c)*RT + rt][h][P]
-                    p.red[(((int64_t)(b * nc + c) * gridDim.y + rt) * p.nheads + h) * P + col] = v;
-                }
-            }
-        }
-    }
-}
-
-// =========================================================================================================
 // launchers
 // =========================================================================================================
 static inline int nchunks(const bimamba2_params *p) { return (p->seqlen + p->chunk_size - 1) / p->chunk_size; }
@@ -445,14 +273,6 @@ int launch_state_passing_fwd(const bimamba2_params *p) {
     const int nc = nchunks(p), PN = p->headdim * p->dstate;
     dim3 grid((PN + NTHREADS - 1) / NTHREADS, p->nheads, p->batch);
     hipLaunchKernelGGL(state_passing_fwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
-    return check_launch();
-}
-
-int launch_chunk_scan(const bimamba2_params *p, bool bwd) {
-    const int nc = nchunks(p);
-    dim3 grid((p->headdim + 63) / 64, (p->chunk_size + 63) / 64, p->batch * nc * p->nheads);
-    if (bwd) { BM2_DISPATCH_T(p, chunk_scan_kernel, grid, true) }
-    else { BM2_DISPATCH_T(p, chunk_scan_kernel, grid, false) }
     return check_launch();
 }
 

@@ -1,0 +1,500 @@
+// The chunk-scan kernel (forward output) and its mirror (dx in the backward pass) for gfx950.
+//
+// One workgroup (8 waves) owns one (batch, chunk, head) and a tile of up to 64 headdim columns; wave w owns the
+// rows [w*16*QT, (w+1)*16*QT) of the chunk.  The K operand of the big product (x * dt, resp. dy) is staged ONCE,
+// transposed, into LDS; the A operand (CB times the decay factors) is built directly in registers in the MFMA
+// operand layout from float32 CB rows, so the main loop has no barrier and no LDS round trip for A.
+//
+//   forward (BWD = false), rows r = output positions t, k = source positions s:
+//     acc[r,p] = e^{cs_f[r]} C_r.prev_f[p,:] + e^{cs_b[r]} C_r.prev_b[p,:]
+//              + sum_k CB[r,k] m(r,k) dt[k] x[k,p],    m = e^{cs_f[r]-cs_f[k]} (k<r), e^{cs_b[r]-cs_b[k]} (k>r), 2 (k=r)
+//     out_x = acc + D x[r,p];  out = out_x * silu(z)
+//   mirror (BWD = true), rows r = input positions s, k = output positions t, CBT[r,k] = CB[k,r]:
+//     acc[r,p] = e^{cs_f[Q-1]-cs_f[r]} B_r.dS_f[p,:] + e^{cs_b[0]-cs_b[r]} B_r.dS_b[p,:]
+//              + sum_k CBT[r,k] m'(r,k) dy[k,p],       m' = e^{cs_f[k]-cs_f[r]} (k>r), e^{cs_b[k]-cs_b[r]} (k<r), 2 (k=r)
+//     dx = acc dt[r] + D dy[r,p];  ddt_direct[r] = sum_p acc x[r,p];  dD partial = sum_r dy x
+#include <type_traits>
+
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace bm2 {
+
+static inline int nchunks(const bimamba2_params *p) { return (p->seqlen + p->chunk_size - 1) / p->chunk_size; }
+static inline hipStream_t stream_of(const bimamba2_params *p) { return reinterpret_cast<hipStream_t>(p->stream); }
+
+constexpr float LOG2E = 1.4426950408889634f;
+
+// LDS image of the K operand: element (r, k) of a [R][KTOT] matrix lives at r*LDX + (16-byte chunk of k, XORed
+// with (r/VS)&7) so that neither the staging writes (rows VS apart) nor the fragment reads (consecutive rows)
+// pile up on the same banks.
+template <typename T, int LDX>
+__device__ __forceinline__ int xt_index(int r, int k) {
+    constexpr int VS = 16 / sizeof(T);
+    const int chunk = (k / VS) ^ ((r / VS) & 7);
+    return r * LDX + chunk * VS + (k % VS);
+}
+
+// Stage src[k][r] (r contiguous, row stride ks) for k < KTOT, r < RTOT into dst as (r, k), scaled by scale(k);
+// rows k >= kvalid and columns r >= rvalid read as 0.  Each thread moves VS x VS blocks: VS 16-byte reads along r,
+// transposed in registers, VS 16-byte LDS writes along k.
+// FAST: every 16-byte read is known to be aligned and inside the column range; rows past kvalid are read from the
+// last valid row and zeroed by scale().
+template <typename T, int KTOT, int RTOT, int LDX, bool FAST, class F>
+__device__ __forceinline__ void stage_transposed(T *dst, const T *src, int64_t ks, int kvalid, int rvalid, F scale) {
+    constexpr int VS = 16 / sizeof(T), RB = RTOT / VS, NB = (KTOT / VS) * RB;
+    const bool vec = FAST || aligned16(src, ks);
+    for (int blk = threadIdx.x; blk < NB; blk += blockDim.x) {
+        const int rb = blk % RB, kb = blk / RB;
+        float v[VS][VS];
+#pragma unroll
+        for (int kk = 0; kk < VS; ++kk) {
+            const int k = kb * VS + kk;
+            const T *row = src + (int64_t)(FAST ? min(k, kvalid - 1) : k) * ks + rb * VS;
+            if (FAST || (vec && k < kvalid && rb * VS + VS <= rvalid)) {
+                Vec16<T> raw = *reinterpret_cast<const Vec16<T> *>(row);
+#pragma unroll
+                for (int i = 0; i < VS; ++i) v[kk][i] = to_f(raw.v[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < VS; ++i) v[kk][i] = (k < kvalid && rb * VS + i < rvalid) ? to_f(row[i]) : 0.f;
+            }
+            const float sc = scale(k);
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[kk][i] *= sc;
+        }
+#pragma unroll
+        for (int rr = 0; rr < VS; ++rr) {
+            Vec16<T> o;
+#pragma unroll
+            for (int kk = 0; kk < VS; ++kk) o.v[kk] = from_f<T>(v[kk][rr]);
+            *reinterpret_cast<Vec16<T> *>(dst + xt_index<T, LDX>(rb * VS + rr, kb * VS)) = o;
+        }
+    }
+}
+
+constexpr int SCAN_WAVES = 8, SCAN_THREADS = 64 * SCAN_WAVES;
+
+// FAST = true is chosen by the launcher when chunk_size % 32 == 0, headdim is a multiple of the column tile,
+// dstate % 64 == 0 and every operand is 16-byte aligned with strides that keep rows aligned: all guarded scalar
+// fallbacks compile away and loads become unconditional (rows past the end of the sequence are read from a valid
+// row and never stored).
+template <typename T, int QT, int NJ, bool BWD, bool FAST>
+__global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimamba2_params p, int nc, int npt) {
+    typedef Mma<T> M;
+    constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
+    constexpr int VS = 16 / (int)sizeof(T);
+    constexpr int QP = SCAN_WAVES * 16 * QT;      // rows the workgroup covers (>= chunk_size); QT row tiles per wave
+    constexpr int PW = 16 * NJ;                   // headdim columns the workgroup covers
+    constexpr int LDX = QP + VS;
+    constexpr int NW = 64;                        // dstate columns of the state tiles held in LDS at a time
+    constexpr int LDS_ = M::LD - BK + NW;         // their leading dimension
+    constexpr int SLD = PW + 4;                   // float32 row of the epilogue staging patches
+    constexpr int XT_BYTES = PW * LDX * (int)sizeof(T), ST_BYTES = 2 * PW * LDS_ * (int)sizeof(T);
+    constexpr int STG_BYTES = SCAN_WAVES * 16 * SLD * 4;
+    // the operand images (xT and the two state tiles) and the per-wave epilogue staging patches are never live together
+    __shared__ __attribute__((aligned(16))) char shared_u[XT_BYTES + ST_BYTES > STG_BYTES ? XT_BYTES + ST_BYTES : STG_BYTES];
+    __shared__ float lo[QP], up[QP];              // decay exponents (times log2 e), see below
+    __shared__ float red[SCAN_WAVES][PW];
+    T *xT = reinterpret_cast<T *>(shared_u);
+    T *sF = reinterpret_cast<T *>(shared_u + XT_BYTES), *sB = sF + PW * LDS_;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
+    // linear block id -> (pt, h, bc) with bc fastest: all heads of one (batch, chunk) share CB and C, and
+    // consecutive ids are dealt round-robin to the 8 XCDs, so equal bc % 8 keeps them on one XCD's L2
+    const int nbc = p.batch * nc;
+    const int bc = blockIdx.x % nbc, hp = blockIdx.x / nbc, pt = hp % npt, h = hp / npt;
+    const int c = bc % nc, b = bc / nc;
+    const int g = h / (p.nheads / p.ngroups);
+    const int Q = p.chunk_size, N = p.dstate, P = p.headdim, H = p.nheads;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int p0 = pt * PW;
+    const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
+    const float *csf = p.cs_f + o, *csb = p.cs_b + o, *dto = p.dt_out + o;
+
+#ifdef BM2_DBG_TIME
+    long long *tlog = reinterpret_cast<long long *>(p.workspace) + ((int64_t)blockIdx.x * SCAN_WAVES + wave) * 8;
+#define TSTAMP(i) if (lane == 0) tlog[i] = wall_clock64();
+#else
+#define TSTAMP(i)
+#endif
+    TSTAMP(0)
+    int rowi[QT];                                  // this lane's A-operand row in each row tile
+#pragma unroll
+    for (int rt = 0; rt < QT; ++rt) rowi[rt] = (wave * QT + rt) * 16 + lr;
+
+    // A operand of part 1: C rows (forward) or B rows (mirror), straight from global memory in operand layout
+    const T *ap;
+    int64_t as;
+    if (BWD) { as = p.B_sl; ap = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * as + g * p.B_sg; }
+    else { as = p.C_sl; ap = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * as + g * p.C_sg; }
+    const bool avec = aligned16(ap, as) && (N % VS == 0);
+    float arow[QT][NW / KSTEP][KPL];               // rows of the first NW dstate columns, requested up front
+    auto load_arows = [&](int n0) {
+#pragma unroll
+        for (int rt = 0; rt < QT; ++rt)
+#pragma unroll
+            for (int s = 0; s < NW / KSTEP; ++s) {
+                const int r = rowi[rt], kb = n0 + s * KSTEP + lg * KPL;
+                if (FAST && KPL == 1) {
+                    arow[rt][s][0] = to_f(ap[(int64_t)min(r, limit - 1) * as + kb]);
+                } else if (KPL > 1 && (FAST || (r < limit && avec && kb + KPL <= N))) {
+                    Vec16<T> raw = *reinterpret_cast<const Vec16<T> *>(ap + (int64_t)(FAST ? min(r, limit - 1) : r) * as + kb);
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) arow[rt][s][i] = to_f(raw.v[i % Vec16<T>::N]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) arow[rt][s][i] = (r < limit && kb + i < N) ? to_f(ap[(int64_t)r * as + kb + i]) : 0.f;
+                }
+            }
+    };
+
+    // forward: k<r uses lo[r]-lo[k] with lo = cs_f, k>r uses up[r]-up[k] with up = cs_b
+    // mirror : k<r uses e^{cs_b[k]-cs_b[r]} -> lo = -cs_b;  k>r uses e^{cs_f[k]-cs_f[r]} -> up = -cs_f
+    for (int q = threadIdx.x; q < QP; q += SCAN_THREADS) {
+        const int qq = min(q, Q - 1);
+        const float f = csf[qq] * LOG2E, r = csb[qq] * LOG2E;
+        lo[q] = BWD ? -r : f;
+        up[q] = BWD ? -f : r;
+    }
+    // K operand of part 2, transposed into LDS
+    const T *kp;
+    int64_t ks;
+    if (!BWD) { ks = p.x_sl; kp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * ks + h * p.x_sh; }
+    else if (p.has_z) { ks = (int64_t)H * P; kp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * ks + (int64_t)h * P; }
+    else { ks = p.dout_sl; kp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * ks + h * p.dout_sh; }
+    if (BWD) stage_transposed<T, QP, PW, LDX, FAST>(xT, kp + p0, ks, limit, P - p0, [&](int k) { return k < limit ? 1.f : 0.f; });
+    else stage_transposed<T, QP, PW, LDX, FAST>(xT, kp + p0, ks, limit, P - p0, [&](int k) { return k < limit ? dto[k] : 0.f; });
+
+    load_arows(0);
+    f32x4 acc[QT][NJ] = {};
+    TSTAMP(1)
+
+    // ---- part 1: states.  A = (C or B rows) * row scale, K = dstate; B operand = state tiles [p][n] in LDS ----
+    {
+        const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * N + (int64_t)p0 * N;
+        const float *stf = (BWD ? p.dstates_f : p.states_f) + so, *stb = (BWD ? p.dstates_b : p.states_b) + so;
+        float rsf[QT], rsb[QT];
+#pragma unroll
+        for (int rt = 0; rt < QT; ++rt) {
+            const int r = rowi[rt];
+            float ef = 0.f, eb = 0.f;
+            if (r < limit) {
+                ef = BWD ? __expf(csf[Q - 1] - csf[r]) : __expf(csf[r]);
+                eb = BWD ? __expf(csb[0] - csb[r]) : __expf(csb[r]);
+            }
+            rsf[rt] = ef;
+            rsb[rt] = eb;
+        }
+        for (int n0 = 0; n0 < N; n0 += NW) {
+            if (n0) {
+                __syncthreads();
+                load_arows(n0);
+            }
+            tile_load_kcontig<T, float, PW, NW>(sF, stf + n0, N, P - p0, N - n0, Ident());
+            tile_load_kcontig<T, float, PW, NW>(sB, stb + n0, N, P - p0, N - n0, Ident());
+            __syncthreads();
+            TSTAMP(2)
+#pragma unroll
+            for (int s = 0; s < NW / KSTEP; ++s) {
+                if (n0 + s * KSTEP >= N) break;
+                const int kq = s * KSTEP + lg * KPL;
+                typename M::Frag bff[NJ], bfb[NJ];
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    bff[j] = M::load(sF + (j * 16 + lr) * LDS_ + kq);
+                    bfb[j] = M::load(sB + (j * 16 + lr) * LDS_ + kq);
+                }
+#pragma unroll
+                for (int rt = 0; rt < QT; ++rt) {
+                    float vf[KPL], vb[KPL];
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) { vf[i] = arow[rt][s][i] * rsf[rt]; vb[i] = arow[rt][s][i] * rsb[rt]; }
+                    const typename M::Frag aff = M::pack(vf), afb = M::pack(vb);
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        acc[rt][j] = M::mma(aff, bff[j], acc[rt][j]);
+                        acc[rt][j] = M::mma(afb, bfb[j], acc[rt][j]);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- epilogue operands (x and z, resp. x and dy) are requested one row tile ahead of their use ----
+    constexpr int CPR = PW / VS;                   // 16-byte chunks per row
+    constexpr int NPASS = (16 * CPR + 63) / 64;    // chunks per lane and row tile
+    const T *xrow = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh;
+    const T *zrow = (!BWD && p.has_z) ? reinterpret_cast<const T *>(p.z) + b * p.z_sb + (int64_t)c * Q * p.z_sl + h * p.z_sh : nullptr;
+    const bool need2 = BWD ? (bool)p.has_D : (bool)p.has_z;      // second operand: dy (for D) resp. z
+    const T *row2 = BWD ? kp : zrow;
+    const int64_t s2 = BWD ? ks : p.z_sl;
+    const bool xvec = aligned16(xrow + p0, p.x_sl) && (P % VS == 0);
+    const bool vec2 = need2 && aligned16(row2 + p0, s2) && (P % VS == 0);
+    const bool ovec = (P % VS == 0);
+    float ex[1][NPASS][VS], e2[1][NPASS][VS];
+    auto load_vec = [&](const T *ptr, bool vec, int ncol, float (&v)[VS]) {
+        if (FAST || (vec && ncol >= VS)) {
+            Vec16<T> raw = *reinterpret_cast<const Vec16<T> *>(ptr);
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = to_f(raw.v[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = i < ncol ? to_f(ptr[i]) : 0.f;
+        }
+    };
+    auto store_vec = [&](T *ptr, bool vec, int ncol, const float (&v)[VS]) {
+        if (FAST || (vec && ncol >= VS)) {
+            Vec16<T> ov;
+#pragma unroll
+            for (int i = 0; i < VS; ++i) ov.v[i] = from_f<T>(v[i]);
+            *reinterpret_cast<Vec16<T> *>(ptr) = ov;
+        } else {
+#pragma unroll
+            for (int i = 0; i < VS; ++i)
+                if (i < ncol) ptr[i] = from_f<T>(v[i]);
+        }
+    };
+    auto epi_issue = [&](auto BUF, int rt) {
+        constexpr int B_ = decltype(BUF)::value;
+        const int r0 = (wave * QT + rt) * 16;
+#pragma unroll
+        for (int ps = 0; ps < NPASS; ++ps) {
+            const int id = lane + ps * 64;
+            const int r = r0 + id / CPR, col = p0 + (id % CPR) * VS;
+            const int ncol = (id < 16 * CPR && r < limit) ? P - col : 0;
+            if (FAST && id >= 16 * CPR) continue;
+            const int rc = min(r, limit - 1);
+            load_vec(xrow + (int64_t)rc * p.x_sl + col, xvec, ncol, ex[B_][ps]);
+            if (need2) load_vec(row2 + (int64_t)rc * s2 + col, vec2, ncol, e2[B_][ps]);
+        }
+    };
+    typedef std::integral_constant<int, 0> B0;
+    typedef std::integral_constant<int, 1> B1;
+
+    TSTAMP(3)
+#ifndef BM2_DBG_SKIP2
+    // ---- part 2: inside the chunk.  A built in registers from CB (forward) or CB^T (mirror); the CB rows of
+    // the next K step are requested before the current step is consumed (two register buffers) ----
+    {
+        const float *cb = (BWD ? p.CBT : p.CB) + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+        const bool cvec = (Q % 4 == 0);
+        float lor[QT], upr[QT];
+        const float *rowp[QT];
+#pragma unroll
+        for (int rt = 0; rt < QT; ++rt) {
+            lor[rt] = lo[rowi[rt]];
+            upr[rt] = up[rowi[rt]];
+            rowp[rt] = cb + (int64_t)min(rowi[rt], Q - 1) * Q;
+        }
+        float cbv[1][QT][KPL];
+        auto issue = [&](auto BUF, int k0) {
+            constexpr int B_ = decltype(BUF)::value;
+            const int kb = k0 + lg * KPL;
+#pragma unroll
+            for (int rt = 0; rt < QT; ++rt) {
+                if (FAST || (cvec && kb + KPL <= Q)) {
+                    if (KPL >= 4) {
+#pragma unroll
+                        for (int i = 0; i < KPL; i += 4) {
+                            const float4 t4 = *reinterpret_cast<const float4 *>(rowp[rt] + kb + i);
+                            cbv[B_][rt][i] = t4.x; cbv[B_][rt][(i + 1) % KPL] = t4.y;
+                            cbv[B_][rt][(i + 2) % KPL] = t4.z; cbv[B_][rt][(i + 3) % KPL] = t4.w;
+                        }
+                    } else {
+                        cbv[B_][rt][0] = rowp[rt][kb];
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) cbv[B_][rt][i] = (kb + i < Q) ? rowp[rt][kb + i] : 0.f;
+                }
+            }
+        };
+        auto process = [&](auto BUF, int k0) {
+            constexpr int B_ = decltype(BUF)::value;
+            const int kb = k0 + lg * KPL;
+            typename M::Frag bf[NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) bf[j] = M::load(xT + xt_index<T, LDX>(j * 16 + lr, kb));
+            float lok[KPL], upk[KPL];
+#pragma unroll
+            for (int i = 0; i < KPL; ++i) { lok[i] = lo[kb + i]; upk[i] = up[kb + i]; }
+#pragma unroll
+            for (int rt = 0; rt < QT; ++rt) {
+                const int r = rowi[rt], r0 = (wave * QT + rt) * 16;
+                float v[KPL];
+                if (k0 + KSTEP - 1 < r0) {            // every k of this step is below every row of the tile
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) v[i] = cbv[B_][rt][i] * __builtin_amdgcn_exp2f(lor[rt] - lok[i]);
+                } else if (k0 > r0 + 15) {            // every k above every row
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) v[i] = cbv[B_][rt][i] * __builtin_amdgcn_exp2f(upr[rt] - upk[i]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) {
+                        const int k = kb + i;
+                        const float e = k < r ? lor[rt] - lok[i] : upr[rt] - upk[i];
+                        v[i] = cbv[B_][rt][i] * ((k == r) ? 2.f : __builtin_amdgcn_exp2f(e));
+                    }
+                }
+                const typename M::Frag af = M::pack(v);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) acc[rt][j] = M::mma(af, bf[j], acc[rt][j]);
+            }
+        };
+        for (int k0 = 0; k0 < limit; k0 += KSTEP) {
+            issue(B0(), k0);
+            process(B0(), k0);
+        }
+    }
+#endif
+
+    // ---- epilogue.  Each wave passes its 16-row accumulator tiles through a private LDS patch so that out, out_x,
+    // dx are written (and x, z, dy were read) as 16-byte vectors along headdim ----
+    TSTAMP(4)
+    __syncthreads();   // every wave is done with xT: the operand images become the staging area
+    TSTAMP(5)
+    float *stg = reinterpret_cast<float *>(shared_u) + wave * 16 * SLD;
+    float dsum[VS];
+#pragma unroll
+    for (int i = 0; i < VS; ++i) dsum[i] = 0.f;
+    auto epi_consume = [&](auto BUF, int rt) {
+        constexpr int B_ = decltype(BUF)::value;
+        const int r0 = (wave * QT + rt) * 16;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) stg[(lg * 4 + i) * SLD + j * 16 + lr] = acc[rt][j][i];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int ps = 0; ps < NPASS; ++ps) {
+            const int id = lane + ps * 64;
+            const int rl = id / CPR, cc = (id % CPR) * VS;
+            const int r = r0 + rl, col = p0 + cc;
+            const int ncol = P - col;              // valid columns from col on
+            const bool ok = id < 16 * CPR && r < limit && ncol > 0;
+            float a[VS];
+#pragma unroll
+            for (int i = 0; i < VS; i += 4) {
+                const float4 t4 = *reinterpret_cast<const float4 *>(stg + (rl & 15) * SLD + cc + i);
+                a[i] = t4.x; a[i + 1] = t4.y; a[i + 2] = t4.z; a[i + 3] = t4.w;
+            }
+            const int64_t orow = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * H + h) * P + col;
+            float rsum = 0.f;
+            if (ok) {
+                if (!BWD) {
+                    if (p.has_D) {
+#pragma unroll
+                        for (int i = 0; i < VS; ++i)
+                            a[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : p.D[h]) * ex[B_][ps][i];
+                    }
+                    if (p.has_z) {
+                        if (p.out_x) store_vec(reinterpret_cast<T *>(p.out_x) + orow, ovec, ncol, a);
+#pragma unroll
+                        for (int i = 0; i < VS; ++i) a[i] *= silu_f(e2[B_][ps][i]);
+                    }
+                    store_vec(reinterpret_cast<T *>(p.out) + orow, ovec, ncol, a);
+                } else {
+                    const float dtr = dto[r];
+                    float dxv[VS];
+#pragma unroll
+                    for (int i = 0; i < VS; ++i) { rsum += a[i] * ex[B_][ps][i]; dxv[i] = a[i] * dtr; }
+                    if (p.has_D) {
+#pragma unroll
+                        for (int i = 0; i < VS; ++i) {
+                            dxv[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : p.D[h]) * e2[B_][ps][i];
+                            dsum[i] += e2[B_][ps][i] * ex[B_][ps][i];
+                        }
+                    }
+                    store_vec(reinterpret_cast<T *>(p.dx) + orow, ovec, ncol, dxv);
+                }
+            }
+            if (BWD) {
+                // the CPR lanes of a row sit next to each other: butterfly over them
+#pragma unroll
+                for (int d = 1; d < CPR; d <<= 1) rsum += __shfl_xor(rsum, d, 64);
+                if (id < 16 * CPR && r < limit && (id % CPR) == 0) {
+                    if (npt == 1) p.ddt_direct[o + r] = rsum;
+                    else atomicAdd(p.ddt_direct + o + r, rsum);   // several headdim tiles share a row
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+#pragma unroll
+    for (int rt = 0; rt < QT; ++rt) {
+        if ((wave * QT + rt) * 16 < limit) {
+            epi_issue(B0(), rt);
+            epi_consume(B0(), rt);
+        }
+    }
+    TSTAMP(6)
+    if (BWD && p.has_D) {
+        // dsum[i]: this lane's share of column (lane % CPR)*VS + i; add the lanes that hold other rows
+#pragma unroll
+        for (int i = 0; i < VS; ++i) {
+            float v = dsum[i];
+#pragma unroll
+            for (int d = CPR; d < 64; d <<= 1) v += __shfl_xor(v, d, 64);
+            dsum[i] = v;
+        }
+        if (lane < CPR) {
+#pragma unroll
+            for (int i = 0; i < VS; ++i) red[wave][lane * VS + i] = dsum[i];
+        }
+        __syncthreads();
+        if (threadIdx.x < PW && p0 + (int)threadIdx.x < P) {
+            float v = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < SCAN_WAVES; ++wv) v += red[wv][threadIdx.x];
+            p.red[((int64_t)(b * nc + c) * H + h) * P + p0 + threadIdx.x] = v;   // partials [(b, c)][h][P]
+        }
+    }
+}
+
+static inline bool al16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+
+template <typename T, int NJMAX, bool BWD>
+static int launch_scan_t(const bimamba2_params *p) {
+    const int nc = nchunks(p);
+    const int P = p->headdim, Q = p->chunk_size, N = p->dstate;
+    constexpr int VS = 16 / (int)sizeof(T);
+    // headdim tile: the widest the LDS image allows (64 columns for 16-bit types, 32 for float32)
+    const int pw = P <= 16 ? 16 : (P <= 32 || NJMAX == 2) ? 32 : 64;
+    const int npt = (P + pw - 1) / pw;
+    dim3 grid(p->batch * nc * p->nheads * npt);
+    hipStream_t s = reinterpret_cast<hipStream_t>(p->stream);
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % VS == 0 && b % VS == 0 && c % VS == 0; };
+    bool fast = Q % 32 == 0 && P % pw == 0 && N % 64 == 0 && al16(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
+    if (BWD) {
+        fast = fast && al16(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al16(p->dx);
+        fast = fast && (p->has_z ? al16(p->dout_x) : (al16(p->dout) && mult(p->dout_sb, p->dout_sl, p->dout_sh)));
+    } else {
+        fast = fast && al16(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg) && al16(p->out);
+        if (p->has_z) fast = fast && al16(p->z) && mult(p->z_sb, p->z_sl, p->z_sh) && (!p->out_x || al16(p->out_x));
+    }
+#define BM2_SCAN(QTV, NJV)                                                                                                     \
+    do {                                                                                                                       \
+        if (fast) hipLaunchKernelGGL((chunk_scan_kernel<T, QTV, NJV, BWD, true>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt); \
+        else hipLaunchKernelGGL((chunk_scan_kernel<T, QTV, NJV, BWD, false>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);     \
+    } while (0)
+    const int qt = Q <= 128 ? 1 : 2;             // 16-row tiles per wave (8 waves)
+    if (pw == 16) { if (qt == 1) BM2_SCAN(1, 1); else BM2_SCAN(2, 1); }
+    else if (pw == 32) { if (qt == 1) BM2_SCAN(1, 2); else BM2_SCAN(2, 2); }
+    else { if (qt == 1) BM2_SCAN(1, NJMAX); else BM2_SCAN(2, NJMAX); }
+#undef BM2_SCAN
+    return check_launch();
+}
+
+int launch_chunk_scan(const bimamba2_params *p, bool bwd) {
+    switch (p->dtype) {
+        case BIMAMBA2_F32: return bwd ? launch_scan_t<float, 2, true>(p) : launch_scan_t<float, 2, false>(p);
+        case BIMAMBA2_BF16: return bwd ? launch_scan_t<bf16_t, 4, true>(p) : launch_scan_t<bf16_t, 4, false>(p);
+        case BIMAMBA2_F16: return bwd ? launch_scan_t<f16_t, 4, true>(p) : launch_scan_t<f16_t, 4, false>(p);
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+}
+
+}  // namespace bm2

@@ -168,14 +168,19 @@ def _chunk_cumsum_fwd(dt, A, chunk_size, dt_bias=None, dt_softplus=False, dt_lim
     return cs_f, cs_b, dt_out
 
 
-def _bmm_chunk_fwd(C, B, chunk_size, output_dtype=torch.float32):
-    """CB (batch, nchunks, ngroups, chunk_size, chunk_size); kept in float32 (the reference's choice too)."""
+def _bmm_chunk_fwd(C, B, chunk_size, output_dtype=torch.float32, with_transpose=False):
+    """CB (batch, nchunks, ngroups, chunk_size, chunk_size); kept in float32 (the reference's choice too).
+    with_transpose=True also returns CBT = CB.transpose(-1, -2) as a second contiguous tensor (the dx kernel
+    reads CB by columns)."""
     batch, seqlen, ngroups, dstate = B.shape
     assert C.shape == B.shape
     c = _Call(batch, seqlen, ngroups, 1, ngroups, dstate, chunk_size, C.dtype, C.device)
     c.set_B(B); c.set_C(C)
     CB = c.new("CB", (batch, c.nchunks, ngroups, chunk_size, chunk_size))
+    CBT = c.new("CBT", CB.shape) if with_transpose else None
     c.run("bimamba2_bmm_chunk_fwd")
+    if with_transpose:
+        return CB, CBT
     return CB if output_dtype in (None, torch.float32) else CB.to(output_dtype)
 
 
@@ -291,7 +296,7 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum_f, dA_cumsum_b, B, CB, dout,
     assert dstates_f.shape == (batch, nchunks, nheads, headdim, dstate) and dstates_b.shape == dstates_f.shape
     c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, x.dtype, x.device)
     c.set_x(x); c.set_B(B); c.set_dout(dout); c.set_D(D)
-    c.put("CB", CB, torch.float32); c.put("dt_out", dt, torch.float32)
+    c.put("CBT", CB.transpose(-1, -2).contiguous(), torch.float32); c.put("dt_out", dt, torch.float32)
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     c.put("dstates_f", dstates_f, torch.float32); c.put("dstates_b", dstates_b, torch.float32)
     dx = c.put("dx", dx) if dx is not None else c.new("dx", x.shape, x.dtype)
@@ -299,7 +304,7 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum_f, dA_cumsum_b, B, CB, dout,
     dD = None
     if D is not None:
         dD = c.new("dD", tuple(D.shape))
-        c.new("red", (batch * nchunks * ((chunk_size + 63) // 64) * nheads * headdim,))
+        c.new("red", (batch * nchunks * nheads * headdim,))
     c.run("bimamba2_chunk_scan_bwd_dx")
     return dx, ddt, (dD.to(D.dtype) if dD is not None else None)
 

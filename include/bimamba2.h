@@ -18,7 +18,7 @@
  *   dt, ddt                          (B, L, H)      element type `dt_dtype`; strides given for dt; ddt contiguous
  *   A, D, dt_bias, dA, dD, ddt_bias  (H,) [D, dD may be (H, P)]   float32, contiguous
  *   dt_out, cs_f, cs_b, ddt_direct, u_f, u_b, v_f, v_b   (B, H, nc, Q)   float32
- *   CB, dCB                          (B, nc, G, Q, Q)   float32, CB[.., l, s] = C_l . B_s
+ *   CB, CBT, dCB                     (B, nc, G, Q, Q)   float32, CB[.., l, s] = C_l . B_s, CBT its transpose
  *   states_f/b, dstates_f/b          (B, nc, H, P, N)   float32
  *   final_f, final_b                 (B, H, P, N)       float32
  */
@@ -74,6 +74,7 @@ typedef struct bimamba2_params {
     /* intermediates (caller-owned; the composite entry points carve them from `workspace` when NULL) */
     float *dt_out, *cs_f, *cs_b;
     float *CB, *dCB;
+    float *CBT;                     /* optional: CB transposed per chunk, CBT[.., s, l] = CB[.., l, s] */
     float *states_f, *states_b;     /* chunk states, overwritten in place by the inter-chunk scan */
     float *dstates_f, *dstates_b;
     void *dout_x;                   /* dout * silu(z), element type `dtype` */
@@ -110,7 +111,7 @@ int bimamba2_bwd(const bimamba2_params *p);
 
 /* dt -> dt_out, cs_f, cs_b.  Replaces _chunk_cumsum_fwd (src/ssd/bi/ssd_chunk_state.py:699-724). */
 int bimamba2_chunk_cumsum_fwd(const bimamba2_params *p);
-/* Cm, Bm -> CB.  Replaces _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208). */
+/* Cm, Bm -> CB (and CBT when that pointer is set).  Replaces _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208). */
 int bimamba2_bmm_chunk_fwd(const bimamba2_params *p);
 /* x, Bm, dt_out, cs_f, cs_b -> states_f, states_b.  Replaces _chunk_state_fwd
  * (src/ssd/bi/ssd_chunk_state.py:764-798). */
