@@ -6,6 +6,8 @@
 //   bwd_dcb            G = dy.x^T once per head -> dCB (summed over heads) and the within-chunk decay gradient
 //   bmm_chunk_bwd      dB = dBs + dCB^T.C ; dC = dCs + dCB.B
 //   chunk_cumsum_bwd   assembles d(dt*A) from its pieces with wavefront scans; ddt, dA, ddt_bias
+#include <type_traits>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -318,23 +320,35 @@ int launch_bwd_dbdc(const bimamba2_params *p, bool is_db) {
 
 // =========================================================================================================
 // One workgroup owns one 64x64 tile (tt, st) of the chunk's (t, s) plane for one (b, c, g) and loops over the
-// heads of the group.  Per head, G[t,s] = dy_h[t,:] . x_h[s,:] (K = headdim), then
+// heads of the group; wave w owns rows 16w..16w+15 of the tile.  Per head, G[t,s] = dy_h[t,:] . x_h[s,:]
+// (K = headdim; both operands are read from global memory straight into MFMA operand registers, the next
+// K chunk being requested while the current one is multiplied), then
 //   f[t,s] = 1[s<=t] G dt[s] e^{cs_f[t]-cs_f[s]},  b[t,s] = 1[s>=t] G dt[s] e^{cs_b[t]-cs_b[s]}
 //   dCB[t,s] = sum_{h in group} (f + b)                       (kept in registers across the head loop)
 //   W_f = 1[s<t] f CB,  W_b = 1[s>t] b CB                     (what the within-chunk gradient of dt*A is made of)
 // The within-chunk gradient  da[i] = sum_{t>=i>s} W_f[t,s] + sum_{t<=i<s} W_b[t,s]  is assembled by the consumer
 // (chunk_cumsum_bwd) from per-tile vectors written here to da_intra[b, h, c, tile, 2, 64]:
 //   off-diagonal tile: [0] = column sums cw[s] = sum_t W,  [1] = row sums rw[t] = sum_s W
-//   diagonal tile    : [0] = the tile's complete contribution to da[i] (row prefix / suffix with DPP), [1] = 0
+//   diagonal tile    : [0] = cw_f - rw_f, [1] = cw_b - rw_b of the tile's own W_f, W_b; the tile's contribution
+//                      to da[i] is the exclusive prefix sum of [0] plus the exclusive suffix sum of [1]
+//                      (da[i+1] - da[i] = cw_f[i] - rw_f[i] inside a tile; at most 64 terms, so the cancellation
+//                      stays at float32 rounding level)
+// One barrier per head (to combine the four waves' column sums); the decay vectors of up to DCB_HEADS heads are
+// put into LDS beforehand.
 // =========================================================================================================
-template <typename T>
+constexpr int DCB_HEADS = 32;
+constexpr int DCB_VEC = 2 * 64;      // floats per tile and head in da_intra
+
+template <typename T, bool FAST>
 __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params p, int nc, int nqt) {
-    constexpr int KW = 64, LD = Mma<T>::LD - BK + KW;
-    __shared__ __attribute__((aligned(16))) T As[64 * LD];
-    __shared__ __attribute__((aligned(16))) T Bs[64 * LD];
-    __shared__ float csf_t[64], csb_t[64], csf_s[64], csb_s[64], dt_s[64];
-    __shared__ float red[4][64];
+    typedef Mma<T> M;
+    constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
+    constexpr int KC = sizeof(T) == 2 ? 64 : 16;          // K chunk held in registers
+    constexpr int NKS = KC / KSTEP;
+    __shared__ float cst[DCB_HEADS][5][64];               // cs_f[t], cs_b[t], cs_f[s], cs_b[s], dt[s] per head
+    __shared__ float part[2][10][64];                     // per-wave column sums (f: 0-3, b: 4-7), row sums (f: 8, b: 9)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
     const int tt = blockIdx.x / nqt, st = blockIdx.x % nqt;
     const int g = blockIdx.y % p.ngroups, bc = blockIdx.y / p.ngroups, c = bc % nc, b = bc / nc;
     const int Q = p.chunk_size, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
@@ -344,149 +358,224 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
     const float *cbg = p.CB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
     int tl[4];     // local row of this lane's accumulator elements
 #pragma unroll
-    for (int i = 0; i < 4; ++i) tl[i] = wave * 16 + (lane >> 4) * 4 + i;
+    for (int i = 0; i < 4; ++i) tl[i] = wave * 16 + lg * 4 + i;
     f32x4 cbr[4], dcb[4] = {};
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int t = t0 + tl[i], s = s0 + j * 16 + (lane & 15);
-            cbr[j][i] = (t < Q && s < Q) ? cbg[(int64_t)t * Q + s] : 0.f;
+            const int t = t0 + tl[i], s = s0 + j * 16 + lr;
+            cbr[j][i] = (t < limit && s < limit) ? cbg[(int64_t)t * Q + s] : 0.f;   // 0 also masks rows / columns past the end
         }
-    for (int hh = 0; hh < hpg; ++hh) {
-        const int h = g * hpg + hh;
-        const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
-        float *tv = p.da_intra + ((o / Q) * nqt * nqt + blockIdx.x) * 128;
-        if (!live) {
-            if (threadIdx.x < 128) tv[threadIdx.x] = 0.f;
-            continue;
+    // operand rows of this lane: A = dy row t0 + 16 wave + lr; B = x rows s0 + 16 j + lr
+    const int arow = min(t0 + wave * 16 + lr, limit - 1);
+    int brow[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) brow[j] = min(s0 + j * 16 + lr, limit - 1);
+    const int nkc = (P + KC - 1) / KC;
+
+    for (int hbase = 0; hbase < hpg; hbase += DCB_HEADS) {
+        const int nh = min(DCB_HEADS, hpg - hbase);
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nh * 5 * 64; idx += NTHREADS) {
+            const int hh = idx / 320, which = (idx % 320) / 64, q = idx % 64;
+            const int64_t o = (((int64_t)b * H + g * hpg + hbase + hh) * nc + c) * Q;
+            const int pos = min((which < 2 ? t0 : s0) + q, Q - 1);
+            const float *src = which == 0 || which == 2 ? p.cs_f : (which == 4 ? p.dt_out : p.cs_b);
+            cst[hh][which][q] = src[o + pos];
         }
         __syncthreads();
-        if (threadIdx.x < 64) {
-            const int t = min(t0 + (int)threadIdx.x, Q - 1);
-            csf_t[threadIdx.x] = p.cs_f[o + t];
-            csb_t[threadIdx.x] = p.cs_b[o + t];
-        } else if (threadIdx.x < 128) {
-            const int sl = threadIdx.x - 64, s = min(s0 + sl, Q - 1);
-            csf_s[sl] = p.cs_f[o + s];
-            csb_s[sl] = p.cs_b[o + s];
-            dt_s[sl] = p.dt_out[o + s];
+        if (!live) {
+            for (int hh = 0; hh < nh; ++hh) {
+                const int64_t o = (((int64_t)b * H + g * hpg + hbase + hh) * nc + c);
+                float *tv = p.da_intra + (o * nqt * nqt + blockIdx.x) * DCB_VEC;
+                for (int i = threadIdx.x; i < DCB_VEC; i += NTHREADS) tv[i] = 0.f;
+            }
+            continue;
         }
-        const T *yp;
-        int64_t ys;
-        if (p.has_z) { ys = (int64_t)H * P; yp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q + t0) * ys + (int64_t)h * P; }
-        else { ys = p.dout_sl; yp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + ((int64_t)c * Q + t0) * ys + h * p.dout_sh; }
-        const T *xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + ((int64_t)c * Q + s0) * p.x_sl + h * p.x_sh;
-        f32x4 acc[4] = {};
-        for (int k0 = 0; k0 < P; k0 += KW) {
-            if (k0) __syncthreads();
-            tile_load_kcontig<T, T, 64, KW>(As, yp + k0, ys, limit - t0, P - k0, Ident());
-            tile_load_kcontig<T, T, 64, KW>(Bs, xp + k0, p.x_sl, limit - s0, P - k0, Ident());
-            __syncthreads();
-            mma_tile<T, 4, KW>(acc, As + wave * 16 * LD, Bs, lane);
-        }
-        float cft[4], cbt[4];
+        // flattened loop over (head, K chunk) with two operand buffers
+        typename M::Frag af[1][NKS], bf[1][4][NKS];        // operands in flight (next step)
+        typename M::Frag afc[NKS], bfc[4][NKS];            // operands being multiplied
+        const int nit = nh * nkc;
+        auto issue = [&](int it) __attribute__((always_inline)) {
+            constexpr int B_ = 0;
+            const int hh = it / nkc, k0 = (it % nkc) * KC;
+            const int h = g * hpg + hbase + hh;
+            const T *yp;
+            int64_t ys;
+            if (p.has_z) { ys = (int64_t)H * P; yp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * ys + (int64_t)h * P; }
+            else { ys = p.dout_sl; yp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * ys + h * p.dout_sh; }
+            const T *xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh;
+            const T *ar = yp + (int64_t)arow * ys;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { cft[i] = csf_t[tl[i]]; cbt[i] = csb_t[tl[i]]; }
-        if (st != tt) {
-            // one direction only: forward below the diagonal, reverse above it
-            float rw[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int ks = 0; ks < NKS; ++ks) {
+                const int kb = k0 + ks * KSTEP + lg * KPL;
+                if (FAST || ((reinterpret_cast<uintptr_t>(ar + kb) & 15) == 0 && kb + KPL <= P)) af[B_][ks] = M::load(ar + kb);
+                else {
+                    float v[KPL];
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) v[i] = kb + i < P ? to_f(ar[kb + i]) : 0.f;
+                    af[B_][ks] = M::pack(v);
+                }
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int sl = j * 16 + (lane & 15);
-                const float dtv = dt_s[sl], cs = st < tt ? csf_s[sl] : csb_s[sl];
-                float cw = 0.f;
+                const T *br = xp + (int64_t)brow[j] * p.x_sl;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float v = acc[j][i] * dtv * __expf((st < tt ? cft[i] : cbt[i]) - cs);
-                    dcb[j][i] += v;
-                    const float w = v * cbr[j][i];
-                    cw += w;
-                    rw[i] += w;
+                for (int ks = 0; ks < NKS; ++ks) {
+                    const int kb = k0 + ks * KSTEP + lg * KPL;
+                    if (FAST || ((reinterpret_cast<uintptr_t>(br + kb) & 15) == 0 && kb + KPL <= P)) bf[B_][j][ks] = M::load(br + kb);
+                    else {
+                        float v[KPL];
+#pragma unroll
+                        for (int i = 0; i < KPL; ++i) v[i] = kb + i < P ? to_f(br[kb + i]) : 0.f;
+                        bf[B_][j][ks] = M::pack(v);
+                    }
                 }
-                cw += __shfl_xor(cw, 16, 64);
-                cw += __shfl_xor(cw, 32, 64);
-                if (lane < 16) red[wave][j * 16 + lane] = cw;
+            }
+        };
+        f32x4 acc[4] = {};
+        auto finish_head = [&](int hh) __attribute__((always_inline)) {
+            const float(*cs)[64] = cst[hh];
+            float cft[4], cbt[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { cft[i] = cs[0][tl[i]]; cbt[i] = cs[1][tl[i]]; }
+            // column sums (this wave's 16 rows) and row sums of W; on the diagonal tile one pair per direction
+            float cwa[4], cwb[4], rwa[4] = {0.f, 0.f, 0.f, 0.f}, rwb[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int sl = j * 16 + lr;
+                const float dtv = cs[4][sl];
+                float ca = 0.f, cb2 = 0.f;
+                if (st != tt) {
+                    // one direction only: forward below the diagonal, reverse above it
+                    const float csv = st < tt ? cs[2][sl] : cs[3][sl];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float v = acc[j][i] * dtv * __expf((st < tt ? cft[i] : cbt[i]) - csv);
+                        dcb[j][i] += v;
+                        const float w = v * cbr[j][i];
+                        ca += w;
+                        rwa[i] += w;
+                    }
+                } else {
+                    const float cfs = cs[2][sl], cbs = cs[3][sl];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float gv = acc[j][i] * dtv;
+                        const float f = (sl <= tl[i]) ? gv * __expf(cft[i] - cfs) : 0.f;
+                        const float r = (sl >= tl[i]) ? gv * __expf(cbt[i] - cbs) : 0.f;
+                        dcb[j][i] += f + r;
+                        const float wf = (sl < tl[i]) ? f * cbr[j][i] : 0.f;
+                        const float wb = (sl > tl[i]) ? r * cbr[j][i] : 0.f;
+                        ca += wf; rwa[i] += wf;
+                        cb2 += wb; rwb[i] += wb;
+                    }
+                }
+                cwa[j] = ca;
+                cwb[j] = cb2;
+            }
+            // hand the sums to the other waves through LDS (double-buffered by head parity)
+            float(*pb)[64] = part[hh & 1];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v = cwa[j];
+                v += __shfl_xor(v, 16, 64);
+                v += __shfl_xor(v, 32, 64);
+                if (lane < 16) pb[wave][j * 16 + lane] = v;
+                if (st == tt) {
+                    float u = cwb[j];
+                    u += __shfl_xor(u, 16, 64);
+                    u += __shfl_xor(u, 32, 64);
+                    if (lane < 16) pb[4 + wave][j * 16 + lane] = u;
+                }
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float r = row16_sum(rw[i]);
-                if ((lane & 15) == 0) tv[64 + tl[i]] = r;
-            }
-        } else {
-            float col[4] = {0.f, 0.f, 0.f, 0.f};
-            float wf[4][4], wb[4][4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int sl = j * 16 + (lane & 15);
-                const float dtv = dt_s[sl], cfs = csf_s[sl], cbs = csb_s[sl];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float gv = acc[j][i] * dtv;
-                    const float f = (sl <= tl[i]) ? gv * __expf(cft[i] - cfs) : 0.f;
-                    const float r = (sl >= tl[i]) ? gv * __expf(cbt[i] - cbs) : 0.f;
-                    dcb[j][i] += f + r;
-                    wf[j][i] = (sl < tl[i]) ? f * cbr[j][i] : 0.f;
-                    wb[j][i] = (sl > tl[i]) ? r * cbr[j][i] : 0.f;
+                const float r = row16_sum(rwa[i]);
+                if (lr == 0) pb[8][tl[i]] = r;
+                if (st == tt) {
+                    const float u = row16_sum(rwb[i]);
+                    if (lr == 0) pb[9][tl[i]] = u;
                 }
             }
-            float carry[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int sl = j * 16 + (lane & 15);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float w = wf[j][i];
-                    const float excl = carry[i] + row16_incl_prefix(w) - w;   // sum over s' < s of this row
-                    if (tl[i] >= sl) col[j] += excl;
-                    carry[i] += row16_sum(w);
-                }
+            __syncthreads();
+            // off-diagonal: [0] = column sums, [1] = row sums.  diagonal: [0] = cw_f - rw_f, [1] = cw_b - rw_b
+            // (the consumer turns them into the tile's own contribution with a prefix resp. suffix sum)
+            if (threadIdx.x < 128) {
+                const int h = g * hpg + hbase + hh;
+                const int64_t o = (((int64_t)b * H + h) * nc + c);
+                float *tv = p.da_intra + (o * nqt * nqt + blockIdx.x) * DCB_VEC;
+                const int q = threadIdx.x & 63, which = threadIdx.x >> 6;
+                float v;
+                if (st != tt) v = which == 0 ? pb[0][q] + pb[1][q] + pb[2][q] + pb[3][q] : pb[8][q];
+                else if (which == 0) v = pb[0][q] + pb[1][q] + pb[2][q] + pb[3][q] - pb[8][q];
+                else v = pb[4][q] + pb[5][q] + pb[6][q] + pb[7][q] - pb[9][q];
+                tv[which * 64 + q] = v;
             }
+        };
+        issue(0);
+        for (int it = 0; it < nit; ++it) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) carry[i] = 0.f;
+            for (int ks = 0; ks < NKS; ++ks) {
+                afc[ks] = af[0][ks];
 #pragma unroll
-            for (int j = 3; j >= 0; --j) {
-                const int sl = j * 16 + (lane & 15);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float w = wb[j][i];
-                    const float excl = carry[i] + row16_incl_suffix(w) - w;   // sum over s' > s of this row
-                    if (tl[i] <= sl) col[j] += excl;
-                    carry[i] += row16_sum(w);
-                }
+                for (int j = 0; j < 4; ++j) bfc[j][ks] = bf[0][j][ks];
             }
+            if (it + 1 < nit) issue(it + 1);                // requested now, needed in the next iteration
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float v = col[j];
-                v += __shfl_xor(v, 16, 64);
-                v += __shfl_xor(v, 32, 64);
-                if (lane < 16) red[wave][j * 16 + lane] = v;
+            for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = M::mma(afc[ks], bfc[j][ks], acc[j]);
+            if (it % nkc == nkc - 1) {
+                // rows past the end of the sequence were read from a valid row: drop them
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (t0 + tl[i] >= limit) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) acc[j][i] = 0.f;
+                    }
+#ifndef BM2_DBG_SKIPFIN
+                finish_head(it / nkc);
+#else
+#pragma unroll
+                for (int j = 0; j < 4; ++j) dcb[j] += acc[j];
+#endif
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
-            if (threadIdx.x < 64) tv[64 + threadIdx.x] = 0.f;
         }
-        __syncthreads();
-        if (threadIdx.x < 64) tv[threadIdx.x] = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
     }
     float *out = p.dCB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int t = t0 + tl[i], s = s0 + j * 16 + (lane & 15);
+            const int t = t0 + tl[i], s = s0 + j * 16 + lr;
             if (t < Q && s < Q) out[(int64_t)t * Q + s] = dcb[j][i];
         }
 }
 
-int launch_bwd_dcb(const bimamba2_params *p) {
+template <typename T>
+static int launch_dcb_t(const bimamba2_params *p) {
     const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
     dim3 grid(nqt * nqt, p->batch * nc * p->ngroups);
+    constexpr int VS = 16 / (int)sizeof(T);
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    bool fast = p->headdim % (sizeof(T) == 2 ? 64 : 16) == 0 && al(p->x) && p->x_sb % VS == 0 && p->x_sl % VS == 0 && p->x_sh % VS == 0;
+    fast = fast && (p->has_z ? al(p->dout_x) : (al(p->dout) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && p->dout_sh % VS == 0));
+    if (fast) hipLaunchKernelGGL((bwd_dcb_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
+    else hipLaunchKernelGGL((bwd_dcb_kernel<T, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
+    return check_launch();
+}
+
+int launch_bwd_dcb(const bimamba2_params *p) {
     switch (p->dtype) {
-        case BIMAMBA2_F32: hipLaunchKernelGGL(bwd_dcb_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt); break;
-        case BIMAMBA2_BF16: hipLaunchKernelGGL(bwd_dcb_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt); break;
-        case BIMAMBA2_F16: hipLaunchKernelGGL(bwd_dcb_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt); break;
+        case BIMAMBA2_F32: return launch_dcb_t<float>(p);
+        case BIMAMBA2_BF16: return launch_dcb_t<bf16_t>(p);
+        case BIMAMBA2_F16: return launch_dcb_t<f16_t>(p);
         default: return BIMAMBA2_EUNSUPPORTED;
     }
-    return check_launch();
 }
 
 // =========================================================================================================
@@ -576,16 +665,16 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
     {
         const int I = lane >> 4, i0 = (lane & 15) * 4;
         if (I < nqt) {
-            const float *tv = p.da_intra + (o / Q) * nqt * nqt * 128;
+            const float *tv = p.da_intra + (o / Q) * nqt * nqt * DCB_VEC;
             auto vec = [&](int tile, int which, float (&r)[4], bool add) {
-                const float4 v = *reinterpret_cast<const float4 *>(tv + (tile * 2 + which) * 64 + i0);
+                const float4 v = *reinterpret_cast<const float4 *>(tv + tile * DCB_VEC + which * 64 + i0);
                 if (add) { r[0] += v.x; r[1] += v.y; r[2] += v.z; r[3] += v.w; }
                 else { r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w; }
             };
-            float d[4];
-            vec(I * nqt + I, 0, d, false);
-            float cwf[4] = {0.f, 0.f, 0.f, 0.f}, rwf[4] = {0.f, 0.f, 0.f, 0.f};
-            float cwb[4] = {0.f, 0.f, 0.f, 0.f}, rwb[4] = {0.f, 0.f, 0.f, 0.f};
+            // the diagonal tile's difference vectors join the exclusive scans: cwf gets cw_f - rw_f, cwb gets cw_b - rw_b
+            float cwf[4], cwb[4], rwf[4] = {0.f, 0.f, 0.f, 0.f}, rwb[4] = {0.f, 0.f, 0.f, 0.f};
+            vec(I * nqt + I, 0, cwf, false);
+            vec(I * nqt + I, 1, cwb, false);
             float between = 0.f;
             for (int a = 0; a < nqt; ++a) {
                 if (a > I) { vec(a * nqt + I, 0, cwf, true); vec(I * nqt + a, 1, rwb, true); }
@@ -607,7 +696,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 in += rwb[e];
-                di[e] = d[e] + between + ex + in;
+                di[e] = between + ex + in;
                 ex += cwf[e];
             }
             float exs = row16_incl_suffix(t_cwb) - t_cwb, ins = row16_incl_suffix(t_rwf) - t_rwf;
