@@ -231,7 +231,6 @@ int bimamba2_chunk_cumsum_bwd(const bimamba2_params *p) {
 int bimamba2_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     bimamba2_params q = *p;
-    q.CBT = nullptr;
     const size_t need = carve(&q, 0, p->workspace);
     if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
     TRY(bimamba2_chunk_cumsum_fwd(&q));
@@ -248,11 +247,16 @@ int bimamba2_bwd(const bimamba2_params *p) {
     q.final_f = q.final_b = nullptr;
     const size_t need = carve(&q, 1, p->workspace);
     if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
-    // recompute the forward intermediates (the reference does the same, src/ssd/bi/ssd_combined.py:373-380)
-    TRY(bimamba2_chunk_cumsum_fwd(&q));
-    TRY(bimamba2_bmm_chunk_fwd(&q));
-    TRY(bimamba2_chunk_state_fwd(&q));
-    TRY(bimamba2_state_passing_fwd(&q));
+    if (p->fwd_saved) {
+        REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->CB); REQUIRE(p->CBT);
+        REQUIRE(p->states_f); REQUIRE(p->states_b);
+    } else {
+        // recompute the forward intermediates (the reference does the same, src/ssd/bi/ssd_combined.py:373-380)
+        TRY(bimamba2_chunk_cumsum_fwd(&q));
+        TRY(bimamba2_bmm_chunk_fwd(&q));
+        TRY(bimamba2_chunk_state_fwd(&q));
+        TRY(bimamba2_state_passing_fwd(&q));
+    }
     if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
     TRY(bimamba2_chunk_scan_bwd_dstates(&q));
     TRY(bimamba2_state_passing_bwd(&q));

@@ -403,37 +403,49 @@ def _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit):
 
 
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
-                                   dt_limit=(0.0, _INF), return_intermediates=True):
+                                   dt_limit=(0.0, _INF), return_intermediates=True, keep_for_bwd=False):
     """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
     like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
-    out, out_x and the final states are materialised as tensors (the rest lives in a workspace)."""
+    out, out_x and the final states are materialised as tensors (the rest lives in a workspace).
+    keep_for_bwd=True appends a tenth element: the tuple (dt_out, cs_f, cs_b, CB, CBT, states_f, states_b) that
+    _mamba_chunk_scan_combined_bwd accepts as `saved` to skip its recomputation."""
     c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
     batch, seqlen, nheads, headdim = x.shape
-    dstate = B.shape[-1]
+    ngroups, dstate = B.shape[2], B.shape[3]
     out = c.new("out", x.shape, x.dtype)
     out_x = c.new("out_x", x.shape, x.dtype) if z is not None else None
     ff = c.new("final_f", (batch, nheads, headdim, dstate)); fb = c.new("final_b", (batch, nheads, headdim, dstate))
     dt_out = cs_f = cs_b = sf = sb = None
-    if return_intermediates:
+    saved = None
+    if return_intermediates or keep_for_bwd:
         dt_out = c.new("dt_out", _bhcq(c)); cs_f = c.new("cs_f", _bhcq(c)); cs_b = c.new("cs_b", _bhcq(c))
         sshape = (batch, c.nchunks, nheads, headdim, dstate)
         sf = c.new("states_f", sshape); sb = c.new("states_b", sshape)
+    if keep_for_bwd:
+        cbshape = (batch, c.nchunks, ngroups, chunk_size, chunk_size)
+        saved = (dt_out, cs_f, cs_b, c.new("CB", cbshape), c.new("CBT", cbshape), sf, sb)
     c.workspace(False)
     c.run("bimamba2_fwd")
-    return out, out_x, dt_out, cs_f, cs_b, sf, sb, ff, fb
+    res = (out, out_x, dt_out, cs_f, cs_b, sf, sb, ff, fb)
+    return res + (saved,) if keep_for_bwd else res
 
 
 def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
                                    dfinal_states=None, dt_softplus=False, dt_limit=(0.0, _INF),
-                                   dx=None, ddt=None, dB=None, dC=None, dz=None, recompute_output=False):
+                                   dx=None, ddt=None, dB=None, dC=None, dz=None, recompute_output=False, saved=None):
     """Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias).  `out` must be the pre-gate output out_x when z is
-    given (it is what the autograd function saves); it is not read otherwise."""
+    given (it is what the autograd function saves); it is not read otherwise.  `saved` is the tuple the forward
+    returns with keep_for_bwd=True; without it the forward intermediates are recomputed, as in the reference."""
     assert dfinal_states is None, "final states are not supported in the backward pass"
     assert not recompute_output, "recompute_output is not supported"
     assert dout.shape == x.shape
     c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
     batch, seqlen, nheads, headdim = x.shape
     c.set_dout(dout)
+    if saved is not None:
+        for name, t in zip(("dt_out", "cs_f", "cs_b", "CB", "CBT", "states_f", "states_b"), saved):
+            c.put(name, t, torch.float32)
+        c.p.fwd_saved = 1
     if z is not None:
         assert out.shape == x.shape
         c.put("out_x", out.contiguous() if out.dtype == x.dtype else out.to(x.dtype).contiguous())
@@ -452,6 +464,11 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
             ddt_bias.to(dt_bias.dtype) if ddt_bias is not None else None)
 
 
+# True: the autograd function keeps the forward's small and state intermediates for the backward pass (about
+# 2 * batch * nchunks * nheads * headdim * dstate * 4 bytes); False: recompute them as the reference does.
+KEEP_FORWARD_INTERMEDIATES = True
+
+
 class MambaChunkScanCombinedFn(torch.autograd.Function):
     """Same 12 positional arguments and the same 12-tuple of gradients as the reference's autograd function
     (src/ssd/bi/ssd_combined.py:555-574)."""
@@ -460,10 +477,15 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
     def forward(ctx, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
                 dt_limit=(0.0, _INF), return_final_states=False):
         ctx.dt_dtype = dt.dtype
-        out, out_x, _, _, _, _, _, ff, fb = _mamba_chunk_scan_combined_fwd(
+        keep = KEEP_FORWARD_INTERMEDIATES and any(
+            t is not None and t.requires_grad for t in (x, dt, A, B, C, D, z, dt_bias))
+        res = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit,
-            return_intermediates=False)
-        ctx.save_for_backward(out_x if z is not None else None, x, dt, A, B, C, D, z, dt_bias)
+            return_intermediates=False, keep_for_bwd=keep)
+        out, out_x, ff, fb = res[0], res[1], res[7], res[8]
+        saved = res[9] if keep else ()
+        ctx.n_saved = len(saved)
+        ctx.save_for_backward(out_x if z is not None else None, x, dt, A, B, C, D, z, dt_bias, *saved)
         ctx.dt_softplus = dt_softplus
         ctx.chunk_size = chunk_size
         ctx.dt_limit = dt_limit
@@ -475,11 +497,12 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *args):
-        out_x, x, dt, A, B, C, D, z, dt_bias = ctx.saved_tensors
+        out_x, x, dt, A, B, C, D, z, dt_bias = ctx.saved_tensors[:9]
+        saved = ctx.saved_tensors[9:] if ctx.n_saved else None
         assert not ctx.return_final_states, "final states are not currently supported in the bwd pass"
         dx, ddt, dA, dB, dC, dD, dz, ddt_bias = _mamba_chunk_scan_combined_bwd(
             dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
-            dt_limit=ctx.dt_limit)
+            dt_limit=ctx.dt_limit, saved=saved)
         return dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, None, None, None
 
 

@@ -54,6 +54,9 @@ typedef struct bimamba2_params {
     int32_t dtype;          /* BIMAMBA2_* : x, z, Bm, Cm, out, out_x, dout and their gradients */
     int32_t dt_dtype;       /* BIMAMBA2_* : dt and ddt */
     int32_t has_D, D_has_hdim, has_z, has_dt_bias, dt_softplus;
+    int32_t fwd_saved;      /* bimamba2_bwd only: dt_out, cs_f, cs_b, CB, CBT, states_f, states_b hold what bimamba2_fwd
+                               left in them, so the backward pass does not recompute them */
+    int32_t reserved0;
     float dt_min, dt_max;
     /* element strides of the strided inputs (last dim contiguous) */
     int64_t x_sb, x_sl, x_sh;
@@ -99,12 +102,15 @@ size_t bimamba2_params_size(void);
 size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd);
 
 /* Whole forward; replaces _mamba_chunk_scan_combined_fwd (src/ssd/bi/ssd_combined.py:297-331).
- * Needs: x dt A Bm Cm [D z dt_bias] out [out_x when has_z] [final_f final_b] workspace. */
+ * Needs: x dt A Bm Cm [D z dt_bias] out [out_x when has_z] [final_f final_b] workspace.  Intermediates given as
+ * non-NULL pointers (dt_out cs_f cs_b CB CBT states_f states_b) are filled in place of workspace memory, so a
+ * caller can keep them for the backward pass. */
 int bimamba2_fwd(const bimamba2_params *p);
 
 /* Whole backward; replaces _mamba_chunk_scan_combined_bwd (src/ssd/bi/ssd_combined.py:334-475).
  * Needs: the forward inputs, dout, out_x (pre-gate output, when has_z), dx ddt dA dB dC [dD dz ddt_bias],
- * workspace. */
+ * workspace.  With fwd_saved = 0 it recomputes the forward intermediates as the reference does; with
+ * fwd_saved = 1 it reads them from the seven pointers named at that flag. */
 int bimamba2_bwd(const bimamba2_params *p);
 
 /* ---- single stages (each is also what the composites run) ------------------------------------------ */

@@ -73,3 +73,14 @@ def test_backward_end_to_end(ops, case):
     inp = make_case(b, L, H, P, G, N, dtype, with_z=z, with_D=(Dk != "none"), D_has_hdim=(Dk == "hp"), with_bias=bias)
     out, grads, ref = _run_bwd(ops, inp, Q, sp, lim)
     _check(out, grads, ref, dtype)
+
+
+@pytest.mark.parametrize("case", [E2E[1], E2E[5]])
+def test_backward_with_recomputation(ops, case, monkeypatch):
+    """The backward pass recomputes the forward intermediates (as the reference does) instead of reading the
+    ones the forward kept."""
+    monkeypatch.setattr(ops, "KEEP_FORWARD_INTERMEDIATES", False)
+    b, L, H, P, G, N, Q, dtype, z, Dk, bias, sp, lim = case
+    inp = make_case(b, L, H, P, G, N, dtype, with_z=z, with_D=(Dk != "none"), D_has_hdim=(Dk == "hp"), with_bias=bias)
+    out, grads, ref = _run_bwd(ops, inp, Q, sp, lim)
+    _check(out, grads, ref, dtype)
