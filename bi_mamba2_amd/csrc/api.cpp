@@ -69,7 +69,7 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     need_f(q->states_b, stn);
     if (is_bwd) {
         const size_t nqt = (Q + 63) / 64;
-        need_f(q->dCB, cbn);
+        need_f(q->dCB, cbn * dcb_slices(q));
         need_f(q->CBT, cbn);
         need_f(q->dstates_f, stn);
         need_f(q->dstates_b, stn);

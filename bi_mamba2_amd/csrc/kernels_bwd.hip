@@ -337,6 +337,7 @@ int launch_bwd_dbdc(const bimamba2_params *p, bool is_db) {
 // put into LDS beforehand.
 // =========================================================================================================
 constexpr int DCB_HEADS = 32;
+constexpr int DCB_SLICES_MAX = 4;
 constexpr int DCB_VEC = 2 * 64;      // floats per tile and head in da_intra
 
 template <typename T, bool FAST>
@@ -374,8 +375,11 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
     for (int j = 0; j < 4; ++j) brow[j] = min(s0 + j * 16 + lr, limit - 1);
     const int nkc = (P + KC - 1) / KC;
 
-    for (int hbase = 0; hbase < hpg; hbase += DCB_HEADS) {
-        const int nh = min(DCB_HEADS, hpg - hbase);
+    // blockIdx.z selects a slice of the group's heads; its dCB partial sum goes to slice blockIdx.z of the output
+    const int hps = (hpg + gridDim.z - 1) / gridDim.z;
+    const int h_begin = blockIdx.z * hps, h_end = min(hpg, h_begin + hps);
+    for (int hbase = h_begin; hbase < h_end; hbase += DCB_HEADS) {
+        const int nh = min(DCB_HEADS, h_end - hbase);
         __syncthreads();
         for (int idx = threadIdx.x; idx < nh * 5 * 64; idx += NTHREADS) {
             const int hh = idx / 320, which = (idx % 320) / 64, q = idx % 64;
@@ -546,7 +550,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
             }
         }
     }
-    float *out = p.dCB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    float *out = p.dCB + ((int64_t)blockIdx.z * gridDim.y + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -556,16 +560,43 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
         }
 }
 
+// dst[i] += sum_{s=1..nslices-1} dst[s*n + i]
+__global__ __launch_bounds__(NTHREADS) void sum_slices_kernel(float *dst, size_t n4, int nslices) {
+    float4 *d = reinterpret_cast<float4 *>(dst);
+    for (size_t i = blockIdx.x * (size_t)NTHREADS + threadIdx.x; i < n4; i += (size_t)gridDim.x * NTHREADS) {
+        float4 v = d[i];
+        for (int s = 1; s < nslices; ++s) {
+            const float4 u = d[s * n4 + i];
+            v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
+        }
+        d[i] = v;
+    }
+}
+
+// head slices of the dCB kernel: one per 32 heads of a group (more slices only cost traffic: measured)
+int dcb_slices(const bimamba2_params *p) {
+    const int hpg = p->nheads / p->ngroups;
+    return std::max(1, std::min(DCB_SLICES_MAX, hpg / 32));
+}
+
 template <typename T>
 static int launch_dcb_t(const bimamba2_params *p) {
     const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
-    dim3 grid(nqt * nqt, p->batch * nc * p->ngroups);
+    const int slices = dcb_slices(p);
+    dim3 grid(nqt * nqt, p->batch * nc * p->ngroups, slices);
     constexpr int VS = 16 / (int)sizeof(T);
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     bool fast = p->headdim % (sizeof(T) == 2 ? 64 : 16) == 0 && al(p->x) && p->x_sb % VS == 0 && p->x_sl % VS == 0 && p->x_sh % VS == 0;
     fast = fast && (p->has_z ? al(p->dout_x) : (al(p->dout) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && p->dout_sh % VS == 0));
     if (fast) hipLaunchKernelGGL((bwd_dcb_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
     else hipLaunchKernelGGL((bwd_dcb_kernel<T, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
+    if (slices > 1) {
+        // (Q*Q is a multiple of 4 only when Q is even; odd chunk sizes are rejected by the 16-byte requirement below)
+        const size_t n = (size_t)p->batch * nc * p->ngroups * p->chunk_size * p->chunk_size;
+        if (n % 4) return BIMAMBA2_EUNSUPPORTED;
+        const int blocks = (int)std::min<size_t>((n / 4 + NTHREADS - 1) / NTHREADS, 4096);
+        hipLaunchKernelGGL(sum_slices_kernel, dim3(blocks), dim3(NTHREADS), 0, stream_of(p), p->dCB, n / 4, slices);
+    }
     return check_launch();
 }
 

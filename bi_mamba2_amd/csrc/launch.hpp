@@ -18,6 +18,7 @@ int launch_bwd_dz(const bimamba2_params *p);
 int launch_state_passing_bwd(const bimamba2_params *p);
 int launch_bwd_dbdc(const bimamba2_params *p, bool is_db);
 int launch_bwd_dcb(const bimamba2_params *p);
+int dcb_slices(const bimamba2_params *p);   // head slices whose dCB partial sums the kernel keeps apart
 int launch_bmm_chunk_bwd(const bimamba2_params *p);
 int launch_chunk_cumsum_bwd(const bimamba2_params *p);
 int launch_fill(float *ptr, size_t n, float value, hipStream_t stream);

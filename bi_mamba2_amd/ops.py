@@ -353,7 +353,8 @@ def _chunk_scan_bwd_dcb(x, dt, dA_cumsum_f, dA_cumsum_b, dout, CB, ngroups=1):
     c.set_x(x); c.set_dout(dout)
     c.put("CB", CB, torch.float32); c.put("dt_out", dt, torch.float32)
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
-    dCB = c.new("dCB", (batch, nchunks, ngroups, chunk_size, chunk_size))
+    nsl = max(1, min(4, nheads // ngroups // 32))      # head slices, added up in place by the kernel launcher
+    dCB = c.new("dCB", (nsl, batch, nchunks, ngroups, chunk_size, chunk_size))[0]
     nqt = (chunk_size + 63) // 64
     da = c.new("da_intra", (batch, nheads, nchunks, nqt * nqt, 2, 64))
     c.run("bimamba2_chunk_scan_bwd_dcb")

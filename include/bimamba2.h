@@ -76,7 +76,8 @@ typedef struct bimamba2_params {
     float *dA, *dD, *ddt_bias;
     /* intermediates (caller-owned; the composite entry points carve them from `workspace` when NULL) */
     float *dt_out, *cs_f, *cs_b;
-    float *CB, *dCB;
+    float *CB;
+    float *dCB;                     /* room for min(4, max(1, H/G/32)) copies: head-slice partial sums, added up in place */
     float *CBT;                     /* optional: CB transposed per chunk, CBT[.., s, l] = CB[.., l, s] */
     float *states_f, *states_b;     /* chunk states, overwritten in place by the inter-chunk scan */
     float *dstates_f, *dstates_b;
