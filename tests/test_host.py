@@ -1,0 +1,122 @@
+"""CPU-only tests of the host side: the C-ABI library loads and exports what include/bimamba2.h declares, argument
+checks answer with error codes before anything is launched, and the Python mirror of the reference interface
+refuses what the reference refuses.  No kernel runs here."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from bi_mamba2_amd import _lib, ops
+from bi_mamba2_amd.modules import BiMamba2
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "bimamba2.h")).read()
+    declared = set(re.findall(r"\b(bimamba2_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(_lib.ALL_SYMBOLS), declared ^ set(_lib.ALL_SYMBOLS)
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.bimamba2_version() >= 100
+    assert lib.bimamba2_params_size() == ctypes.sizeof(_lib.Params)
+
+
+def _params(**kw):
+    p = _lib.Params()
+    base = dict(batch=2, seqlen=100, nheads=4, headdim=32, ngroups=2, dstate=16, chunk_size=64, dtype=_lib.BF16,
+                dt_dtype=_lib.F32, dt_max=float("inf"))
+    base.update(kw)
+    for k, v in base.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_argument_checks_return_error_codes():
+    lib = _lib.load()
+    assert lib.bimamba2_fwd(None) == -1
+    assert lib.bimamba2_fwd(ctypes.byref(_params())) == -3                      # no workspace
+    assert lib.bimamba2_chunk_cumsum_fwd(ctypes.byref(_params())) == -1         # null pointers
+    assert lib.bimamba2_fwd(ctypes.byref(_params(chunk_size=512))) == -2        # chunk too large
+    assert lib.bimamba2_fwd(ctypes.byref(_params(chunk_size=16))) == -2         # chunk too small (reference: >= 32)
+    assert lib.bimamba2_fwd(ctypes.byref(_params(headdim=256))) == -2
+    assert lib.bimamba2_fwd(ctypes.byref(_params(nheads=3))) == -1              # heads not divisible by groups
+    assert lib.bimamba2_fwd(ctypes.byref(_params(dtype=7))) == -2
+    assert lib.bimamba2_bwd(ctypes.byref(_params(fwd_saved=1, workspace=1, workspace_bytes=1 << 40))) == -1
+    for code in (0, -1, -2, -3, -4, -99):
+        assert lib.bimamba2_strerror(code)
+    with pytest.raises(ValueError):
+        _lib.call("bimamba2_chunk_cumsum_fwd", _params())
+
+
+def test_workspace_sizes():
+    lib = _lib.load()
+    p = _params()
+    fwd, bwd = lib.bimamba2_workspace_bytes(ctypes.byref(p), 0), lib.bimamba2_workspace_bytes(ctypes.byref(p), 1)
+    nc = 2
+    states = 2 * 2 * nc * 4 * 32 * 16 * 4
+    assert fwd >= states and bwd > 2 * fwd - 4096
+    assert lib.bimamba2_workspace_bytes(ctypes.byref(_params(chunk_size=8)), 0) == 0
+
+
+def _cpu_inputs(b=1, L=64, H=2, P=4, G=1, N=4):
+    return (torch.randn(b, L, H, P), torch.randn(b, L, H), -torch.rand(H), torch.randn(b, L, G, N), torch.randn(b, L, G, N))
+
+
+def test_no_cpu_fallback():
+    x, dt, A, B, C = _cpu_inputs()
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.bimamba_chunk_scan_combined(x, dt, A, B, C, 32)
+
+
+def test_shape_checks_match_the_reference():
+    x, dt, A, B, C = _cpu_inputs()
+    with pytest.raises(AssertionError):
+        ops.bimamba_chunk_scan_combined(x, dt, A, B, C, 16)                       # chunk_size >= 32
+    with pytest.raises(AssertionError):
+        ops.bimamba_chunk_scan_combined(x, dt[:, :-1], A, B, C, 32)
+    with pytest.raises(AssertionError):
+        ops.bimamba_chunk_scan_combined(x, dt, A, B, C[..., :-1], 32)
+    with pytest.raises(AssertionError):
+        ops.bimamba_chunk_scan_combined(x, dt, A, B, C, 32, D=torch.randn(3))
+    with pytest.raises(AssertionError):
+        ops.bimamba_chunk_scan_combined(x, dt, A, B, C, 32, z=torch.randn(1, 64, 2, 5))
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    code = ("import os; os.environ['BIMAMBA2_LIB'] = %r\n"
+            "from bi_mamba2_amd import _lib\n"
+            "try:\n    _lib.load()\nexcept RuntimeError as e:\n    print('RAISED', 'no CPU or PyTorch fallback' in str(e))\n") % str(tmp_path / "absent.so")
+    out = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True)
+    assert "RAISED True" in out.stdout, out.stdout + out.stderr
+
+
+def test_bench_refuses_more_than_one_gpu():
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert out.returncode != 0 and "ONE GPU" in out.stderr
+
+
+def test_bimamba2_layer_parameters():
+    """Same parameter names and shapes as the reference layer (src/ssd/modules.py:65-116 there)."""
+    m = BiMamba2(d_model=64, d_state=16, headdim=16, ngroups=2, learnable_init_states=True)
+    shapes = {k: tuple(v.shape) for k, v in m.state_dict().items()}
+    d_inner, nheads, bc = 128, 8, 2 * 2 * 16
+    assert shapes == {
+        "in_proj.weight": (2 * d_inner + bc + nheads, 64), "conv1d.weight": (d_inner + bc, 1, 7), "conv1d.bias": (d_inner + bc,),
+        "init_states": (nheads, 16, 16), "dt_bias": (nheads,), "A_log": (nheads,), "D": (nheads,),
+        "fc_D.weight": (nheads, d_inner), "norm.weight": (d_inner,), "out_proj.weight": (64, d_inner)}
+    assert torch.all(m.A_log == 0) and torch.all(m.D == 1)
+    dt0 = torch.nn.functional.softplus(m.dt_bias)
+    assert dt0.min() >= 1e-4 and dt0.max() <= 0.1 + 1e-6
+
+
+def test_import_aliases():
+    from ssd.bi.ssd_combined import bimamba_chunk_scan_combined, MambaChunkScanCombinedFn
+    from ssd.modules import BiMamba2 as Alias
+    assert bimamba_chunk_scan_combined is ops.bimamba_chunk_scan_combined
+    assert MambaChunkScanCombinedFn is ops.MambaChunkScanCombinedFn and Alias is BiMamba2
