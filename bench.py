@@ -26,7 +26,12 @@ WORKLOAD = dict(batch=4, seqlen=2048, nheads=32, headdim=64, ngroups=1, dstate=6
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
 # size); None until measured for the kernel in question.  Source: the summaries under profiles/.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    "bimamba2_chunk_scan_bwd_dcb": 264.5e6, "bimamba2_chunk_scan_bwd_dc": 203.1e6, "bimamba2_chunk_state_bwd_db": 202.1e6,
+    "bimamba2_chunk_scan_fwd": 235.7e6, "bimamba2_chunk_scan_bwd_dx": 191.4e6, "bimamba2_chunk_scan_bwd_dz": 167.9e6,
+    "bimamba2_state_passing_bwd": 101.9e6, "bimamba2_bmm_chunk_bwd": 63.7e6, "bimamba2_chunk_state_fwd": 78.4e6,
+    "bimamba2_chunk_scan_bwd_dstates": 78.4e6, "bimamba2_state_passing_fwd": 70.6e6,
+}
 
 
 def stage_table(w, e):
@@ -204,6 +209,17 @@ def main():
         us = ev0.elapsed_time(ev1) * 1e3 / reps
         kernels[entry] = {"us": round(us, 2), "gflop": round(flops / 1e9, 3), "mbytes": round(nbytes / 1e6, 2),
                           "tflops": round(flops / us / 1e6, 2), "gbs": round(nbytes / us / 1e3, 1)}
+    # one plain device copy of known size: the unit against which the FETCH_SIZE / WRITE_SIZE counters are scaled
+    cal_src = torch.empty(64 << 20, device=dev, dtype=torch.float32)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(10):
+        cal_dst.copy_(cal_src)
+    ev1.record()
+    torch.cuda.synchronize()
+    copy_gbs = 2 * cal_src.numel() * 4 * 10 / (ev0.elapsed_time(ev1) * 1e-3) / 1e9
     dom = max(kernels, key=lambda k: kernels[k]["us"])
     flops, nbytes = table[dom]
     t_mfma = flops / (MFMA_PEAK_TFLOPS["bf16"] * 1e12)
@@ -239,7 +255,8 @@ def main():
                      "fwd_bwd_alg_MB": (fwd_b + bwd_b) / 1e6,
                      "fwd_bwd_hbm_frac": (fwd_b + bwd_b) / t_step / (HBM_PEAK_GBS * 1e9),
                      "fwd_hbm_frac": fwd_b / t_fwd / (HBM_PEAK_GBS * 1e9),
-                     "sum_kernel_us": round(sum(k["us"] for k in kernels.values()), 1)},
+                     "sum_kernel_us": round(sum(k["us"] for k in kernels.values()), 1),
+                     "measured_copy_GBs": round(copy_gbs, 1)},
         "kernels": kernels,
     }
     if not args.no_cpu:
