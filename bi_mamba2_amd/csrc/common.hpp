@@ -165,6 +165,94 @@ __device__ __forceinline__ void tile_load_rcontig2(T *dst1, T *dst2, const S *sr
     }
 }
 
+// ---- transposing stage: global [k][r] -> LDS image addressed by (r, k) ----------------------------------
+// LDS image of the K operand: element (r, k) of a [R][KTOT] matrix lives at r*LDX + (16-byte chunk of k, XORed
+// with (r/VS)&7) so that neither the staging writes (rows VS apart) nor the fragment reads (consecutive rows)
+// pile up on the same banks.
+template <typename T, int LDX>
+__device__ __forceinline__ int xt_index(int r, int k) {
+    constexpr int VS = 16 / sizeof(T);
+    const int chunk = (k / VS) ^ ((r / VS) & 7);
+    return r * LDX + chunk * VS + (k % VS);
+}
+
+// Stage src[k][r] (r contiguous, row stride ks) for k < KTOT, r < RTOT into dst as (r, k), scaled by scale(k);
+// rows k >= kvalid and columns r >= rvalid read as 0.  Each thread moves VS x VS blocks: VS 16-byte reads along r,
+// transposed in registers, VS 16-byte LDS writes along k.
+// FAST: every 16-byte read is known to be aligned and inside the column range; rows past kvalid are read from the
+// last valid row and zeroed by scale().
+// The source element type S may differ from T (float32 states staged as 16-bit operands): a thread moves a block of
+// VK = 16/sizeof(T) rows (k) by VR = 16/sizeof(S) columns (r).
+template <typename T, int KTOT, int RTOT, int LDX, bool FAST, typename S, class F>
+__device__ __forceinline__ void stage_transposed(T *dst, const S *src, int64_t ks, int kvalid, int rvalid, F scale) {
+    constexpr int VK = 16 / sizeof(T), VR = 16 / sizeof(S), RB = RTOT / VR, NB = (KTOT / VK) * RB;
+    const bool vec = FAST || aligned16(src, ks);
+    for (int blk = threadIdx.x; blk < NB; blk += blockDim.x) {
+        const int rb = blk % RB, kb = blk / RB;
+        float v[VK][VR];
+#pragma unroll
+        for (int kk = 0; kk < VK; ++kk) {
+            const int k = kb * VK + kk;
+            const S *row = src + (int64_t)(FAST ? min(k, kvalid - 1) : k) * ks + rb * VR;
+            if (FAST || (vec && k < kvalid && rb * VR + VR <= rvalid)) {
+                Vec16<S> raw = *reinterpret_cast<const Vec16<S> *>(row);
+#pragma unroll
+                for (int i = 0; i < VR; ++i) v[kk][i] = to_f(raw.v[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < VR; ++i) v[kk][i] = (k < kvalid && rb * VR + i < rvalid) ? to_f(row[i]) : 0.f;
+            }
+            const float sc = scale(k);
+#pragma unroll
+            for (int i = 0; i < VR; ++i) v[kk][i] *= sc;
+        }
+#pragma unroll
+        for (int rr = 0; rr < VR; ++rr) {
+            Vec16<T> o;
+#pragma unroll
+            for (int kk = 0; kk < VK; ++kk) o.v[kk] = from_f<T>(v[kk][rr]);
+            *reinterpret_cast<Vec16<T> *>(dst + xt_index<T, LDX>(rb * VR + rr, kb * VK)) = o;
+        }
+    }
+}
+
+// same read of the source, two scaled images (used where both directions weight one operand differently)
+template <typename T, int KTOT, int RTOT, int LDX, bool FAST, typename S, class F1, class F2>
+__device__ __forceinline__ void stage_transposed2(T *dst1, T *dst2, const S *src, int64_t ks, int kvalid, int rvalid,
+                                                  F1 scale1, F2 scale2) {
+    constexpr int VK = 16 / sizeof(T), VR = 16 / sizeof(S), RB = RTOT / VR, NB = (KTOT / VK) * RB;
+    const bool vec = FAST || aligned16(src, ks);
+    for (int blk = threadIdx.x; blk < NB; blk += blockDim.x) {
+        const int rb = blk % RB, kb = blk / RB;
+        float v[VK][VR], s1[VK], s2[VK];
+#pragma unroll
+        for (int kk = 0; kk < VK; ++kk) {
+            const int k = kb * VK + kk;
+            const S *row = src + (int64_t)(FAST ? min(k, kvalid - 1) : k) * ks + rb * VR;
+            if (FAST || (vec && k < kvalid && rb * VR + VR <= rvalid)) {
+                Vec16<S> raw = *reinterpret_cast<const Vec16<S> *>(row);
+#pragma unroll
+                for (int i = 0; i < VR; ++i) v[kk][i] = to_f(raw.v[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < VR; ++i) v[kk][i] = (k < kvalid && rb * VR + i < rvalid) ? to_f(row[i]) : 0.f;
+            }
+            s1[kk] = scale1(k);
+            s2[kk] = scale2(k);
+        }
+#pragma unroll
+        for (int rr = 0; rr < VR; ++rr) {
+            Vec16<T> o1, o2;
+#pragma unroll
+            for (int kk = 0; kk < VK; ++kk) { o1.v[kk] = from_f<T>(v[kk][rr] * s1[kk]); o2.v[kk] = from_f<T>(v[kk][rr] * s2[kk]); }
+            const int at = xt_index<T, LDX>(rb * VR + rr, kb * VK);
+            *reinterpret_cast<Vec16<T> *>(dst1 + at) = o1;
+            *reinterpret_cast<Vec16<T> *>(dst2 + at) = o2;
+        }
+    }
+}
+
+
 struct Ident {
     __device__ __forceinline__ float operator()(int, int, float v) const { return v; }
 };

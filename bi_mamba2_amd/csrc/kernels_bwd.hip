@@ -192,8 +192,10 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dbdc_kernel(const bimamba2_param
     __shared__ __attribute__((aligned(16))) T Bb[64 * LD];
     __shared__ float sfs[64], sbs[64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int rt = blockIdx.x;
-    const int g = blockIdx.y % p.ngroups, bc = blockIdx.y / p.ngroups, c = bc % nc, b = bc / nc;
+    // blockIdx.x = (b, c, g) varies fastest: consecutive workgroups are dealt round-robin to the 8 XCDs, so the row
+    // tiles of one (b, c, g), which read the same states, land on the same XCD and share its L2
+    const int rt = blockIdx.y;
+    const int g = blockIdx.x % p.ngroups, bc = blockIdx.x / p.ngroups, c = bc % nc, b = bc / nc;
     const int Q = p.chunk_size, N = p.dstate, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
     const int limit = min(Q, p.seqlen - c * Q);
     const int r0 = rt * 64;
@@ -300,7 +302,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dbdc_kernel(const bimamba2_param
 template <typename T, bool IS_DB>
 static int launch_dbdc_t(const bimamba2_params *p) {
     const int nc = nchunks(p);
-    dim3 grid((p->chunk_size + 63) / 64, p->batch * nc * p->ngroups, dbdc_slices(p));
+    dim3 grid(p->batch * nc * p->ngroups, (p->chunk_size + 63) / 64, dbdc_slices(p));
     const int nt = (p->dstate + 63) / 64;
     if (nt == 1) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 1, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
     else if (nt == 2) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 2, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
@@ -350,8 +352,11 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
     __shared__ float part[2][10][64];                     // per-wave column sums (f: 0-3, b: 4-7), row sums (f: 8, b: 9)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lr = lane & 15, lg = lane >> 4;
-    const int tt = blockIdx.x / nqt, st = blockIdx.x % nqt;
-    const int g = blockIdx.y % p.ngroups, bc = blockIdx.y / p.ngroups, c = bc % nc, b = bc / nc;
+    // blockIdx.x = (b, c, g) varies fastest so that the tiles of one (b, c, g), which share x and dout rows, run on
+    // the same XCD (workgroups are dealt round-robin to the 8 XCDs) and hit its L2
+    const int tile = blockIdx.y;
+    const int tt = tile / nqt, st = tile % nqt;
+    const int g = blockIdx.x % p.ngroups, bc = blockIdx.x / p.ngroups, c = bc % nc, b = bc / nc;
     const int Q = p.chunk_size, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
     const int limit = min(Q, p.seqlen - c * Q);
     const int t0 = tt * 64, s0 = st * 64;
@@ -392,7 +397,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
         if (!live) {
             for (int hh = 0; hh < nh; ++hh) {
                 const int64_t o = (((int64_t)b * H + g * hpg + hbase + hh) * nc + c);
-                float *tv = p.da_intra + (o * nqt * nqt + blockIdx.x) * DCB_VEC;
+                float *tv = p.da_intra + (o * nqt * nqt + tile) * DCB_VEC;
                 for (int i = threadIdx.x; i < DCB_VEC; i += NTHREADS) tv[i] = 0.f;
             }
             continue;
@@ -509,7 +514,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
             if (threadIdx.x < 128) {
                 const int h = g * hpg + hbase + hh;
                 const int64_t o = (((int64_t)b * H + h) * nc + c);
-                float *tv = p.da_intra + (o * nqt * nqt + blockIdx.x) * DCB_VEC;
+                float *tv = p.da_intra + (o * nqt * nqt + tile) * DCB_VEC;
                 const int q = threadIdx.x & 63, which = threadIdx.x >> 6;
                 float v;
                 if (st != tt) v = which == 0 ? pb[0][q] + pb[1][q] + pb[2][q] + pb[3][q] : pb[8][q];
@@ -550,7 +555,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
             }
         }
     }
-    float *out = p.dCB + ((int64_t)blockIdx.z * gridDim.y + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    float *out = p.dCB + ((int64_t)blockIdx.z * gridDim.x + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -583,7 +588,7 @@ template <typename T>
 static int launch_dcb_t(const bimamba2_params *p) {
     const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
     const int slices = dcb_slices(p);
-    dim3 grid(nqt * nqt, p->batch * nc * p->ngroups, slices);
+    dim3 grid(p->batch * nc * p->ngroups, nqt * nqt, slices);
     constexpr int VS = 16 / (int)sizeof(T);
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     bool fast = p->headdim % (sizeof(T) == 2 ? 64 : 16) == 0 && al(p->x) && p->x_sb % VS == 0 && p->x_sl % VS == 0 && p->x_sh % VS == 0;

@@ -100,14 +100,20 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_fwd_kernel(const bimamba2_
 // gradient of the chunk-entry states (DSTATES = true):  dprev_f[p,n] = sum_k dy[k,p] C[k,n] e^{cs_f[k]},
 //                                 dprev_b with e^{cs_b[k]}
 // =========================================================================================================
-template <typename T, bool DSTATES>
+// Both operands have K = chunk position as their slow dimension, so both are staged transposed (8x8 in-register
+// transposes) into LDS, KH positions at a time; the decay weights are applied to the B-side image while staging.
+template <typename T, bool DSTATES, bool FAST>
 __global__ __launch_bounds__(NTHREADS) void chunk_state_kernel(const bimamba2_params p, int nc) {
-    constexpr int LD = Mma<T>::LD;
-    __shared__ __attribute__((aligned(16))) T As[64 * LD];
-    __shared__ __attribute__((aligned(16))) T Bf[64 * LD];
-    __shared__ __attribute__((aligned(16))) T Bb[64 * LD];
+    typedef Mma<T> M;
+    constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
+    constexpr int KH = sizeof(T) == 2 ? 128 : 64;          // chunk positions staged per round
+    constexpr int LDX = KH + 16 / (int)sizeof(T);
+    __shared__ __attribute__((aligned(16))) T xT[64 * LDX];
+    __shared__ __attribute__((aligned(16))) T Bf[64 * LDX];
+    __shared__ __attribute__((aligned(16))) T Bb[64 * LDX];
     __shared__ float wf[BIMAMBA2_MAX_CHUNK], wb[BIMAMBA2_MAX_CHUNK];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
     const int nt = blockIdx.x, pt = blockIdx.y;
     const int h = blockIdx.z % p.nheads, bc = blockIdx.z / p.nheads, c = bc % nc, b = bc / nc;
     const int g = h / (p.nheads / p.ngroups);
@@ -146,15 +152,25 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_kernel(const bimamba2_pa
     else { bs = p.B_sl; bp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * bs + g * p.B_sg; }
     bp += nt * 64;
     f32x4 accf[4] = {}, accb[4] = {};
-    for (int k0 = 0; k0 < limit; k0 += BK) {
+    for (int k0 = 0; k0 < limit; k0 += KH) {
+        __syncthreads();       // weights written / previous round consumed
+        const int kv = limit - k0;
+        stage_transposed<T, KH, 64, LDX, FAST>(xT, xp + (int64_t)k0 * xs, xs, kv, P - pt * 64,
+                                               [&](int k) { return k < kv ? 1.f : 0.f; });
+        stage_transposed2<T, KH, 64, LDX, FAST>(Bf, Bb, bp + (int64_t)k0 * bs, bs, kv, N - nt * 64,
+                                                [&](int k) { return k < kv ? wf[k0 + k] : 0.f; },
+                                                [&](int k) { return k < kv ? wb[k0 + k] : 0.f; });
         __syncthreads();
-        tile_load_rcontig<T, T, 64>(As, xp + k0 * xs, xs, P - pt * 64, limit - k0, Ident());
-        tile_load_rcontig2<T, T, 64>(
-            Bf, Bb, bp + k0 * bs, bs, N - nt * 64, limit - k0,
-            [&](int, int k, float v) { return v * wf[k0 + k]; }, [&](int, int k, float v) { return v * wb[k0 + k]; });
-        __syncthreads();
-        mma_tile<T, 4>(accf, As + wave * 16 * LD, Bf, lane);
-        mma_tile<T, 4>(accb, As + wave * 16 * LD, Bb, lane);
+        const int kend = min(KH, (kv + KSTEP - 1) / KSTEP * KSTEP);
+        for (int ks = 0; ks < kend; ks += KSTEP) {
+            const int kq = ks + lg * KPL;
+            const typename M::Frag a = M::load(xT + xt_index<T, LDX>(wave * 16 + lr, kq));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                accf[j] = M::mma(a, M::load(Bf + xt_index<T, LDX>(j * 16 + lr, kq)), accf[j]);
+                accb[j] = M::mma(a, M::load(Bb + xt_index<T, LDX>(j * 16 + lr, kq)), accb[j]);
+            }
+        }
     }
     float *of = (DSTATES ? p.dstates_f : p.states_f) + (int64_t)blockIdx.z * P * N;
     float *ob = (DSTATES ? p.dstates_b : p.states_b) + (int64_t)blockIdx.z * P * N;
@@ -162,7 +178,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_kernel(const bimamba2_pa
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int pp = pt * 64 + wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
+            const int pp = pt * 64 + wave * 16 + lg * 4 + i, n = nt * 64 + j * 16 + lr;
             if (pp < P && n < N) {
                 of[(int64_t)pp * N + n] = accf[j][i];
                 ob[(int64_t)pp * N + n] = accb[j][i];
@@ -261,12 +277,38 @@ int launch_bmm_chunk_fwd(const bimamba2_params *p) {
     return check_launch();
 }
 
-int launch_chunk_state(const bimamba2_params *p, bool dstates) {
+template <typename T>
+static int launch_chunk_state_t(const bimamba2_params *p, bool dstates) {
     const int nc = nchunks(p);
     dim3 grid((p->dstate + 63) / 64, (p->headdim + 63) / 64, p->batch * nc * p->nheads);
-    if (dstates) { BM2_DISPATCH_T(p, chunk_state_kernel, grid, true) }
-    else { BM2_DISPATCH_T(p, chunk_state_kernel, grid, false) }
+    constexpr int VS = 16 / (int)sizeof(T);
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % VS == 0 && b % VS == 0 && c % VS == 0; };
+    bool fast = p->headdim % 64 == 0 && p->dstate % 64 == 0;
+    if (dstates) {
+        fast = fast && al(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg);
+        fast = fast && (p->has_z ? al(p->dout_x) : (al(p->dout) && mult(p->dout_sb, p->dout_sl, p->dout_sh)));
+    } else {
+        fast = fast && al(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
+    }
+    hipStream_t s = stream_of(p);
+    if (dstates) {
+        if (fast) hipLaunchKernelGGL((chunk_state_kernel<T, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+        else hipLaunchKernelGGL((chunk_state_kernel<T, true, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
+    } else {
+        if (fast) hipLaunchKernelGGL((chunk_state_kernel<T, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+        else hipLaunchKernelGGL((chunk_state_kernel<T, false, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
+    }
     return check_launch();
+}
+
+int launch_chunk_state(const bimamba2_params *p, bool dstates) {
+    switch (p->dtype) {
+        case BIMAMBA2_F32: return launch_chunk_state_t<float>(p, dstates);
+        case BIMAMBA2_BF16: return launch_chunk_state_t<bf16_t>(p, dstates);
+        case BIMAMBA2_F16: return launch_chunk_state_t<f16_t>(p, dstates);
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
 }
 
 int launch_state_passing_fwd(const bimamba2_params *p) {

@@ -25,54 +25,6 @@ static inline hipStream_t stream_of(const bimamba2_params *p) { return reinterpr
 
 constexpr float LOG2E = 1.4426950408889634f;
 
-// LDS image of the K operand: element (r, k) of a [R][KTOT] matrix lives at r*LDX + (16-byte chunk of k, XORed
-// with (r/VS)&7) so that neither the staging writes (rows VS apart) nor the fragment reads (consecutive rows)
-// pile up on the same banks.
-template <typename T, int LDX>
-__device__ __forceinline__ int xt_index(int r, int k) {
-    constexpr int VS = 16 / sizeof(T);
-    const int chunk = (k / VS) ^ ((r / VS) & 7);
-    return r * LDX + chunk * VS + (k % VS);
-}
-
-// Stage src[k][r] (r contiguous, row stride ks) for k < KTOT, r < RTOT into dst as (r, k), scaled by scale(k);
-// rows k >= kvalid and columns r >= rvalid read as 0.  Each thread moves VS x VS blocks: VS 16-byte reads along r,
-// transposed in registers, VS 16-byte LDS writes along k.
-// FAST: every 16-byte read is known to be aligned and inside the column range; rows past kvalid are read from the
-// last valid row and zeroed by scale().
-template <typename T, int KTOT, int RTOT, int LDX, bool FAST, class F>
-__device__ __forceinline__ void stage_transposed(T *dst, const T *src, int64_t ks, int kvalid, int rvalid, F scale) {
-    constexpr int VS = 16 / sizeof(T), RB = RTOT / VS, NB = (KTOT / VS) * RB;
-    const bool vec = FAST || aligned16(src, ks);
-    for (int blk = threadIdx.x; blk < NB; blk += blockDim.x) {
-        const int rb = blk % RB, kb = blk / RB;
-        float v[VS][VS];
-#pragma unroll
-        for (int kk = 0; kk < VS; ++kk) {
-            const int k = kb * VS + kk;
-            const T *row = src + (int64_t)(FAST ? min(k, kvalid - 1) : k) * ks + rb * VS;
-            if (FAST || (vec && k < kvalid && rb * VS + VS <= rvalid)) {
-                Vec16<T> raw = *reinterpret_cast<const Vec16<T> *>(row);
-#pragma unroll
-                for (int i = 0; i < VS; ++i) v[kk][i] = to_f(raw.v[i]);
-            } else {
-#pragma unroll
-                for (int i = 0; i < VS; ++i) v[kk][i] = (k < kvalid && rb * VS + i < rvalid) ? to_f(row[i]) : 0.f;
-            }
-            const float sc = scale(k);
-#pragma unroll
-            for (int i = 0; i < VS; ++i) v[kk][i] *= sc;
-        }
-#pragma unroll
-        for (int rr = 0; rr < VS; ++rr) {
-            Vec16<T> o;
-#pragma unroll
-            for (int kk = 0; kk < VS; ++kk) o.v[kk] = from_f<T>(v[kk][rr]);
-            *reinterpret_cast<Vec16<T> *>(dst + xt_index<T, LDX>(rb * VS + rr, kb * VS)) = o;
-        }
-    }
-}
-
 constexpr int SCAN_WAVES = 8, SCAN_THREADS = 64 * SCAN_WAVES;
 
 // FAST = true is chosen by the launcher when chunk_size % 32 == 0, headdim is a multiple of the column tile,
