@@ -178,7 +178,7 @@ def main():
     nqt = (w["chunk_size"] + 63) // 64
     c.new("da_intra", bhcq[:3] + (nqt * nqt, 2, 64))
     cbs = (w["batch"], nc, w["ngroups"], w["chunk_size"], w["chunk_size"])
-    c.new("CB", cbs); c.new("dCB", (4,) + cbs); c.new("CBT", cbs)
+    c.new("CB", cbs); c.new("dCB", (4,) + cbs); c.new("dCBT", (4,) + cbs); c.new("CBT", cbs)
     sts = (w["batch"], nc, w["nheads"], w["headdim"], w["dstate"])
     for f in ("states_f", "states_b", "dstates_f", "dstates_b"):
         c.new(f, sts)

@@ -27,7 +27,7 @@ class Params(ctypes.Structure):
         + [(n, _vp) for n in ("x", "dt", "Bm", "Cm", "z", "dout", "A", "D", "dt_bias",
                               "out", "out_x", "final_f", "final_b",
                               "dx", "ddt", "dB", "dC", "dz", "dA", "dD", "ddt_bias",
-                              "dt_out", "cs_f", "cs_b", "CB", "dCB", "CBT", "states_f", "states_b",
+                              "dt_out", "cs_f", "cs_b", "CB", "dCB", "CBT", "dCBT", "states_f", "states_b",
                               "dstates_f", "dstates_b", "dout_x",
                               "ddt_direct", "u_f", "u_b", "v_f", "v_b", "da_intra",
                               "ddA_chunk_f", "ddA_chunk_b", "dBs", "dCs", "red", "workspace")]

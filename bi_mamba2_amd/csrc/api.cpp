@@ -70,6 +70,7 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     if (is_bwd) {
         const size_t nqt = (Q + 63) / 64;
         need_f(q->dCB, cbn * dcb_slices(q));
+        need_f(q->dCBT, cbn * dcb_slices(q));
         need_f(q->CBT, cbn);
         need_f(q->dstates_f, stn);
         need_f(q->dstates_b, stn);
@@ -209,14 +210,14 @@ int bimamba2_chunk_scan_bwd_dc(const bimamba2_params *p) {
 int bimamba2_chunk_scan_bwd_dcb(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->x); REQUIRE(p->CB); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
-    REQUIRE(p->dCB); REQUIRE(p->da_intra);
+    REQUIRE(p->dCB); REQUIRE(p->dCBT); REQUIRE(p->da_intra);
     if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
     return launch_bwd_dcb(p);
 }
 
 int bimamba2_bmm_chunk_bwd(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->Bm); REQUIRE(p->Cm); REQUIRE(p->dCB); REQUIRE(p->dBs); REQUIRE(p->dCs); REQUIRE(p->dB); REQUIRE(p->dC);
+    REQUIRE(p->Bm); REQUIRE(p->Cm); REQUIRE(p->dCB); REQUIRE(p->dCBT); REQUIRE(p->dBs); REQUIRE(p->dCs); REQUIRE(p->dB); REQUIRE(p->dC);
     return launch_bmm_chunk_bwd(p);
 }
 

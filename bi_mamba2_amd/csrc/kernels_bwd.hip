@@ -555,14 +555,24 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
             }
         }
     }
-    float *out = p.dCB + ((int64_t)blockIdx.z * gridDim.x + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    const int64_t oo = ((int64_t)blockIdx.z * gridDim.x + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    float *out = p.dCB + oo, *outT = p.dCBT + oo;       // dCBT[s, t] = dCB[t, s], read by the dB product
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 4; ++j) {
+        const int s = s0 + j * 16 + lr;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int t = t0 + tl[i], s = s0 + j * 16 + lr;
+            const int t = t0 + tl[i];
             if (t < Q && s < Q) out[(int64_t)t * Q + s] = dcb[j][i];
         }
+        if (s < Q) {
+            if (t0 + tl[0] + 3 < Q && Q % 4 == 0) *reinterpret_cast<f32x4 *>(outT + (int64_t)s * Q + t0 + tl[0]) = dcb[j];
+            else
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (t0 + tl[i] < Q) outT[(int64_t)s * Q + t0 + tl[i]] = dcb[j][i];
+        }
+    }
 }
 
 // dst[i] += sum_{s=1..nslices-1} dst[s*n + i]
@@ -601,6 +611,7 @@ static int launch_dcb_t(const bimamba2_params *p) {
         if (n % 4) return BIMAMBA2_EUNSUPPORTED;
         const int blocks = (int)std::min<size_t>((n / 4 + NTHREADS - 1) / NTHREADS, 4096);
         hipLaunchKernelGGL(sum_slices_kernel, dim3(blocks), dim3(NTHREADS), 0, stream_of(p), p->dCB, n / 4, slices);
+        hipLaunchKernelGGL(sum_slices_kernel, dim3(blocks), dim3(NTHREADS), 0, stream_of(p), p->dCBT, n / 4, slices);
     }
     return check_launch();
 }
@@ -615,60 +626,115 @@ int launch_bwd_dcb(const bimamba2_params *p) {
 }
 
 // =========================================================================================================
-// which = 0 : dB[s,n] = dBs[s,n] + sum_t dCB[t,s] C[t,n]      which = 1 : dC[t,n] = dCs[t,n] + sum_s dCB[t,s] B[s,n]
+// which = 0 : dB[s,n] = sum_slices dBs[s,n] + sum_t dCBT[s,t] C[t,n]     which = 1 : dC[t,n] = sum dCs + sum_s dCB[t,s] B[s,n]
+// One workgroup: 64 rows x 64 dstate columns of one (b, c, g).  The K operand (C or B rows of the chunk) is staged
+// transposed in LDS once; the A operand is read from the float32 dCB / dCBT rows straight into MFMA operand layout.
 // =========================================================================================================
-template <typename T>
+template <typename T, int QP>
 __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_params p, int nc, int nslices) {
-    constexpr int LD = Mma<T>::LD;
-    __shared__ __attribute__((aligned(16))) T As[64 * LD];
-    __shared__ __attribute__((aligned(16))) T Bs[64 * LD];
+    typedef Mma<T> M;
+    constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
+    constexpr int LDX = QP + 16 / (int)sizeof(T);
+    __shared__ __attribute__((aligned(16))) T kT[64 * LDX];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
     const int nt = blockIdx.x, rt = blockIdx.y;
     const int which = blockIdx.z & 1, bcg = blockIdx.z >> 1;
     const int g = bcg % p.ngroups, bc = bcg / p.ngroups, c = bc % nc, b = bc / nc;
     const int Q = p.chunk_size, N = p.dstate;
     const int limit = min(Q, p.seqlen - c * Q);
     const int r0 = rt * 64;
-    const float *dcb = p.dCB + (int64_t)bcg * Q * Q;
     const T *op;
     int64_t os;
     if (which == 0) { os = p.C_sl; op = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * os + g * p.C_sg + nt * 64; }
     else { os = p.B_sl; op = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * os + g * p.B_sg + nt * 64; }
+    stage_transposed<T, QP, 64, LDX, false>(kT, op, os, limit, N - nt * 64, [&](int k) { return 1.f; });
+    __syncthreads();
+    const float *arow = (which == 0 ? p.dCBT : p.dCB) + (int64_t)bcg * Q * Q + (int64_t)min(r0 + wave * 16 + lr, Q - 1) * Q;
+    const bool cvec = Q % 4 == 0;
     f32x4 acc[4] = {};
-    for (int k0 = 0; k0 < limit; k0 += BK) {
-        __syncthreads();
-        if (which == 0) tile_load_rcontig<T, float, 64>(As, dcb + (int64_t)k0 * Q + r0, Q, Q - r0, Q - k0, Ident());
-        else tile_load_kcontig<T, float, 64>(As, dcb + (int64_t)r0 * Q + k0, Q, Q - r0, Q - k0, Ident());
-        tile_load_rcontig<T, T, 64>(Bs, op + k0 * os, os, N - nt * 64, limit - k0, Ident());
-        __syncthreads();
-        mma_tile<T, 4>(acc, As + wave * 16 * LD, Bs, lane);
+    for (int k0 = 0; k0 < limit; k0 += KSTEP) {
+        const int kb = k0 + lg * KPL;
+        float v[KPL];
+        if (cvec && kb + KPL <= Q) {
+            if (KPL >= 4) {
+#pragma unroll
+                for (int i = 0; i < KPL; i += 4) {
+                    const float4 t4 = *reinterpret_cast<const float4 *>(arow + kb + i);
+                    v[i] = t4.x; v[(i + 1) % KPL] = t4.y; v[(i + 2) % KPL] = t4.z; v[(i + 3) % KPL] = t4.w;
+                }
+            } else {
+                v[0] = arow[kb];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < KPL; ++i) v[i] = kb + i < Q ? arow[kb + i] : 0.f;
+        }
+        const typename M::Frag af = M::pack(v);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = M::mma(af, M::load(kT + xt_index<T, LDX>(j * 16 + lr, kb)), acc[j]);
     }
     const float *res = which == 0 ? p.dBs : p.dCs;
     T *out = reinterpret_cast<T *>(which == 0 ? p.dB : p.dC);
+    const int64_t slice = (int64_t)p.batch * p.seqlen * p.ngroups * N;
+    // pass the tile through LDS so that the slices are read and the result is written
+    // as 16-byte vectors along dstate
+    constexpr int VS = 16 / (int)sizeof(T), SLD = 64 + 4;
+    __shared__ __attribute__((aligned(16))) float stg[64 * SLD];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = r0 + wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
-            if (r < limit && n < N) {
-                const int64_t a = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n;
-                float v = acc[j][i];
-                for (int sl = 0; sl < nslices; ++sl) v += res[a + (int64_t)sl * p.batch * p.seqlen * p.ngroups * N];
-                out[a] = from_f<T>(v);
-            }
+        for (int i = 0; i < 4; ++i) stg[(wave * 16 + lg * 4 + i) * SLD + j * 16 + lr] = acc[j][i];
+    __syncthreads();
+    const bool ovec = N % VS == 0;
+    for (int id = threadIdx.x; id < 64 * (64 / VS); id += NTHREADS) {
+        const int rl = id / (64 / VS), cc = (id % (64 / VS)) * VS;
+        const int r = r0 + rl, n = nt * 64 + cc;
+        if (r >= limit || n >= N) continue;
+        const int64_t a = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n;
+        float v[VS];
+#pragma unroll
+        for (int i = 0; i < VS; ++i) v[i] = stg[rl * SLD + cc + i];
+        if (ovec) {
+            for (int sl = 0; sl < nslices; ++sl)
+#pragma unroll
+                for (int i = 0; i < VS; i += 4) {
+                    const float4 t4 = *reinterpret_cast<const float4 *>(res + a + sl * slice + i);
+                    v[i] += t4.x; v[i + 1] += t4.y; v[i + 2] += t4.z; v[i + 3] += t4.w;
+                }
+            Vec16<T> ov;
+#pragma unroll
+            for (int i = 0; i < VS; ++i) ov.v[i] = from_f<T>(v[i]);
+            *reinterpret_cast<Vec16<T> *>(out + a) = ov;
+        } else {
+#pragma unroll
+            for (int i = 0; i < VS; ++i)
+                if (n + i < N) {
+                    float u = v[i];
+                    for (int sl = 0; sl < nslices; ++sl) u += res[a + sl * slice + i];
+                    out[a + i] = from_f<T>(u);
+                }
         }
+    }
+}
+
+template <typename T>
+static int launch_bmm_bwd_t(const bimamba2_params *p) {
+    const int nc = nchunks(p), Q = p->chunk_size;
+    dim3 grid((p->dstate + 63) / 64, (Q + 63) / 64, p->batch * nc * p->ngroups * 2);
+    if (Q <= 64) hipLaunchKernelGGL((bmm_chunk_bwd_kernel<T, 64>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p));
+    else if (Q <= 128) hipLaunchKernelGGL((bmm_chunk_bwd_kernel<T, 128>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p));
+    else hipLaunchKernelGGL((bmm_chunk_bwd_kernel<T, 256>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p));
+    return check_launch();
 }
 
 int launch_bmm_chunk_bwd(const bimamba2_params *p) {
-    const int nc = nchunks(p);
-    dim3 grid((p->dstate + 63) / 64, (p->chunk_size + 63) / 64, p->batch * nc * p->ngroups * 2);
     switch (p->dtype) {
-        case BIMAMBA2_F32: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<float>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p)); break;
-        case BIMAMBA2_BF16: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p)); break;
-        case BIMAMBA2_F16: hipLaunchKernelGGL(bmm_chunk_bwd_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p)); break;
+        case BIMAMBA2_F32: return launch_bmm_bwd_t<float>(p);
+        case BIMAMBA2_BF16: return launch_bmm_bwd_t<bf16_t>(p);
+        case BIMAMBA2_F16: return launch_bmm_bwd_t<f16_t>(p);
         default: return BIMAMBA2_EUNSUPPORTED;
     }
-    return check_launch();
 }
 
 // =========================================================================================================

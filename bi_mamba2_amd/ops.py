@@ -355,6 +355,7 @@ def _chunk_scan_bwd_dcb(x, dt, dA_cumsum_f, dA_cumsum_b, dout, CB, ngroups=1):
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     nsl = max(1, min(4, nheads // ngroups // 32))      # head slices, added up in place by the kernel launcher
     dCB = c.new("dCB", (nsl, batch, nchunks, ngroups, chunk_size, chunk_size))[0]
+    c.new("dCBT", (nsl, batch, nchunks, ngroups, chunk_size, chunk_size))
     nqt = (chunk_size + 63) // 64
     da = c.new("da_intra", (batch, nheads, nchunks, nqt * nqt, 2, 64))
     c.run("bimamba2_chunk_scan_bwd_dcb")
@@ -369,7 +370,8 @@ def _bmm_chunk_bwd(B, C, dCB, dBs, dCs):
     # nheads is only used to tell the kernel how many slices to add up
     c = _Call(batch, seqlen, ngroups * 4 * dBs.shape[0], 1, ngroups, dstate, chunk_size, B.dtype, B.device)
     c.set_B(B); c.set_C(C)
-    c.put("dCB", dCB, torch.float32); c.put("dBs", dBs, torch.float32); c.put("dCs", dCs, torch.float32)
+    c.put("dCB", dCB, torch.float32); c.put("dCBT", dCB.transpose(-1, -2).contiguous(), torch.float32)
+    c.put("dBs", dBs, torch.float32); c.put("dCs", dCs, torch.float32)
     dB = torch.zeros(B.shape, device=B.device, dtype=B.dtype); c.put("dB", dB)
     dC = torch.zeros(B.shape, device=B.device, dtype=B.dtype); c.put("dC", dC)
     c.run("bimamba2_bmm_chunk_bwd")

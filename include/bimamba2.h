@@ -79,6 +79,7 @@ typedef struct bimamba2_params {
     float *CB;
     float *dCB;                     /* room for min(4, max(1, H/G/32)) copies: head-slice partial sums, added up in place */
     float *CBT;                     /* optional: CB transposed per chunk, CBT[.., s, l] = CB[.., l, s] */
+    float *dCBT;                    /* dCB transposed per chunk (same number of copies as dCB) */
     float *states_f, *states_b;     /* chunk states, overwritten in place by the inter-chunk scan */
     float *dstates_f, *dstates_b;
     void *dout_x;                   /* dout * silu(z), element type `dtype` */
@@ -149,10 +150,10 @@ int bimamba2_chunk_state_bwd_db(const bimamba2_params *p);
 /* dout, states_f/b, cs, Cm -> dCs, u_f, u_b.  Replaces _chunk_scan_bwd_dC
  * (src/ssd/bi/ssd_chunk_scan.py:1829-1877); u_* are its ddA_cumsum_prev terms. */
 int bimamba2_chunk_scan_bwd_dc(const bimamba2_params *p);
-/* x, dout, dt_out, cs, CB -> dCB, da_intra.  Replaces _chunk_scan_bwd_dcb (src/ssd/bi/ssd_chunk_scan.py:1880-1909)
+/* x, dout, dt_out, cs, CB -> dCB, dCBT, da_intra.  Replaces _chunk_scan_bwd_dcb (src/ssd/bi/ssd_chunk_scan.py:1880-1909)
  * and _chunk_scan_bwd_ddAcs_stable_fwd/_bwd (src/ssd/bi/ssd_chunk_scan.py:2036-2098) in one pass. */
 int bimamba2_chunk_scan_bwd_dcb(const bimamba2_params *p);
-/* dCB, Cm, Bm, dBs, dCs -> dB, dC.  Replaces the two _bmm_chunk_bwd calls (src/ssd/bi/ssd_bmm.py:211-262). */
+/* dCB, dCBT, Cm, Bm, dBs, dCs -> dB, dC.  Replaces the two _bmm_chunk_bwd calls (src/ssd/bi/ssd_bmm.py:211-262). */
 int bimamba2_bmm_chunk_bwd(const bimamba2_params *p);
 /* da_intra, u, v, ddA_chunk, ddt_direct, dt, A, dt_bias -> ddt, dA, ddt_bias.  Replaces the host-side
  * scans (src/ssd/bi/ssd_combined.py:456-466) and _chunk_cumsum_bwd (src/ssd/bi/ssd_chunk_state.py:727-761). */
