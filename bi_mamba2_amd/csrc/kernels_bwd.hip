@@ -184,130 +184,245 @@ int launch_state_passing_bwd(const bimamba2_params *p) {
 constexpr int DBDC_HEADS = 4;
 static inline int dbdc_slices(const bimamba2_params *p) { return (p->nheads / p->ngroups + DBDC_HEADS - 1) / DBDC_HEADS; }
 
-template <typename T, int NT, bool IS_DB>
-__global__ __launch_bounds__(NTHREADS) void bwd_dbdc_kernel(const bimamba2_params p, int nc) {
-    constexpr int LD = Mma<T>::LD;
-    __shared__ __attribute__((aligned(16))) T As[64 * LD];
-    __shared__ __attribute__((aligned(16))) T Bf[64 * LD];
-    __shared__ __attribute__((aligned(16))) T Bb[64 * LD];
-    __shared__ float sfs[64], sbs[64];
+// The A operand (x or dout rows, K = headdim contiguous) is read from global memory straight into MFMA operand
+// registers; the states, stored [p][n], are staged transposed ([n][p], 64 x 64 at a time) in LDS, double-buffered for
+// 16-bit types so that one barrier per step suffices.
+constexpr int DBDC_WAVES = 8, DBDC_THREADS = 64 * DBDC_WAVES;
+
+// 8 waves; wave w owns QT 16-row tiles: the workgroup covers 128*QT rows, so that with QT = 2 a 256-row chunk reads
+// each state once.  Global memory latency is hidden by software pipelining over "steps" (head, dstate tile, headdim
+// chunk): the state blocks and A fragments of step s+1 are requested into registers before step s is multiplied, and
+// only then written to the LDS image.
+template <typename T, int NT, int QT, bool IS_DB, bool FAST>
+__global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_params p, int nc) {
+    typedef Mma<T> M;
+    constexpr int KPL = M::KPL, KSTEP = M::KSTEP, KC = 64, NKS = KC / KSTEP;
+    constexpr int VK = 16 / (int)sizeof(T);                                // image rows (k) per staged block; 4 columns (n)
+    constexpr int LDX = KC + VK;
+    constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;
+    constexpr int ROWS = DBDC_WAVES * 16 * QT;
+    constexpr int NBLK = (KC / VK) * (64 / 4);                             // staged blocks per 64 x 64 state tile
+    static_assert(2 * NBLK <= DBDC_THREADS, "one staged block per thread");
+    __shared__ __attribute__((aligned(16))) T sF[NBUF][64 * LDX];
+    __shared__ __attribute__((aligned(16))) T sB[NBUF][64 * LDX];
+    __shared__ float sfs[DBDC_HEADS][ROWS], sbs[DBDC_HEADS][ROWS];         // row scales of the heads of this slice
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lr = lane & 15, lg = lane >> 4;
     // blockIdx.x = (b, c, g) varies fastest: consecutive workgroups are dealt round-robin to the 8 XCDs, so the row
     // tiles of one (b, c, g), which read the same states, land on the same XCD and share its L2
     const int rt = blockIdx.y;
     const int g = blockIdx.x % p.ngroups, bc = blockIdx.x / p.ngroups, c = bc % nc, b = bc / nc;
     const int Q = p.chunk_size, N = p.dstate, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
     const int limit = min(Q, p.seqlen - c * Q);
-    const int r0 = rt * 64;
+    const int r0 = rt * ROWS;
+    // blockIdx.z selects a slice of DBDC_HEADS heads of the group; its partial sum goes to slice blockIdx.z of the
+    // output, and bmm_chunk_bwd adds the slices up
+    const int hh0 = blockIdx.z * DBDC_HEADS, hh_end = min(hpg, hh0 + DBDC_HEADS);
+    const int nkc = (P + KC - 1) / KC, nnt = (N + 63) / 64;
+    const int per_head = nnt * nkc, nsteps = (hh_end - hh0) * per_head;
+
+    // ---- software pipeline, stage 1: requests for a step (state blocks of two tiles, A fragments) ----
+    Vec16<float> sreg[VK];                                                 // one VK x 4 block of a state tile
+    typename M::Frag af[QT][NKS];
+    int arow[QT];                                                          // this lane's A-operand rows
+#pragma unroll
+    for (int q = 0; q < QT; ++q) arow[q] = min(r0 + (wave * QT + q) * 16 + lr, limit - 1);
+    const int sblk = threadIdx.x % NBLK, stile = threadIdx.x / NBLK;       // stile 0: forward state, 1: reverse state
+    const int s_rb = sblk % 16, s_kb = sblk / 16;
+    auto request = [&](int step) __attribute__((always_inline)) {
+        const int hh = hh0 + step / per_head, rem = step % per_head, nt = rem / nkc, kc = rem % nkc;
+        const int h = g * hpg + hh;
+        if (stile < 2) {
+            const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * N;
+            const float *st = (IS_DB ? (stile ? p.dstates_b : p.dstates_f) : (stile ? p.states_b : p.states_f)) + so;
+#pragma unroll
+            for (int kk = 0; kk < VK; ++kk) {
+                const int pp = kc * KC + s_kb * VK + kk, n = nt * 64 + s_rb * 4;
+                if (FAST) sreg[kk] = *reinterpret_cast<const Vec16<float> *>(st + (int64_t)pp * N + n);
+                else
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) sreg[kk].v[i] = (pp < P && n + i < N) ? st[(int64_t)pp * N + n + i] : 0.f;
+            }
+        }
+        const T *ap;
+        int64_t as;
+        if (IS_DB) { as = p.x_sl; ap = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * as + h * p.x_sh; }
+        else if (p.has_z) { as = (int64_t)H * P; ap = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * as + (int64_t)h * P; }
+        else { as = p.dout_sl; ap = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * as + h * p.dout_sh; }
+#pragma unroll
+        for (int q = 0; q < QT; ++q)
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                const int kb = kc * KC + ks * KSTEP + lg * KPL;
+                const T *row = ap + (int64_t)arow[q] * as;
+                if (FAST) af[q][ks] = M::load(row + kb);
+                else {
+                    float v[KPL];
+#pragma unroll
+                    for (int i = 0; i < KPL; ++i) v[i] = kb + i < P ? to_f(row[kb + i]) : 0.f;
+                    af[q][ks] = M::pack(v);
+                }
+            }
+    };
+    // stage 2: the requested state block goes, transposed, into the LDS image (r = n, k = p)
+    auto commit = [&](int buf) __attribute__((always_inline)) {
+        if (stile < 2) {
+            T *dst = stile ? sB[buf] : sF[buf];
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                Vec16<T> o;
+#pragma unroll
+                for (int kk = 0; kk < VK; ++kk) o.v[kk] = from_f<T>(sreg[kk].v[rr]);
+                *reinterpret_cast<Vec16<T> *>(dst + xt_index<T, LDX>(s_rb * 4 + rr, s_kb * VK)) = o;
+            }
+        }
+    };
+    request(0);
+
+    int tl[QT][4];                                                         // rows of this lane's accumulator elements
+#pragma unroll
+    for (int q = 0; q < QT; ++q)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tl[q][i] = (wave * QT + q) * 16 + lg * 4 + i;
+    // row scales of every head of the slice
+    for (int idx = threadIdx.x; idx < (hh_end - hh0) * ROWS; idx += DBDC_THREADS) {
+        const int hh = idx / ROWS, rl = idx % ROWS, r = r0 + rl;
+        const int64_t o = (((int64_t)b * H + g * hpg + hh0 + hh) * nc + c) * Q;
+        float f = 0.f, rv = 0.f;
+        if (r < limit) {
+            if (IS_DB) {
+                const float d = p.dt_out[o + r];
+                f = d * __expf(p.cs_f[o + Q - 1] - p.cs_f[o + r]);
+                rv = d * __expf(p.cs_b[o] - p.cs_b[o + r]);
+            } else {
+                f = __expf(p.cs_f[o + r]);
+                rv = __expf(p.cs_b[o + r]);
+            }
+        }
+        sfs[hh][rl] = f;
+        sbs[hh][rl] = rv;
+    }
     // B or C values of this lane's output elements
     const T *cbp;
     int64_t cbs;
     if (IS_DB) { cbs = p.B_sl; cbp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + ((int64_t)c * Q + r0) * cbs + g * p.B_sg; }
     else { cbs = p.C_sl; cbp = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + ((int64_t)c * Q + r0) * cbs + g * p.C_sg; }
-    float creg[NT][4][4];
+    float creg[NT][QT][4][4];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int q = 0; q < QT; ++q)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int rl = wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
-                creg[nt][j][i] = (r0 + rl < limit && n < N) ? to_f(cbp[(int64_t)rl * cbs + n]) : 0.f;
-            }
-    f32x4 tot[NT][4] = {};
-    // blockIdx.z selects a slice of DBDC_HEADS heads of the group; its partial sum goes to slice blockIdx.z of the
-    // output, and bmm_chunk_bwd adds the slices up
-    const int hh_end = min(hpg, ((int)blockIdx.z + 1) * DBDC_HEADS);
-    for (int hh = blockIdx.z * DBDC_HEADS; hh < hh_end; ++hh) {
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = nt * 64 + j * 16 + lr;
+                    creg[nt][q][j][i] = (r0 + tl[q][i] < limit && n < N) ? to_f(cbp[(int64_t)tl[q][i] * cbs + n]) : 0.f;
+                }
+    f32x4 tot[NT][QT][4] = {};
+
+    int step = 0;
+    for (int hh = hh0; hh < hh_end; ++hh) {
         const int h = g * hpg + hh;
         const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
-        __syncthreads();
-        if (threadIdx.x < 64) {
-            const int r = r0 + threadIdx.x;
-            float f = 0.f, s = 0.f;
-            if (r < limit) {
-                if (IS_DB) {
-                    const float d = p.dt_out[o + r];
-                    f = d * __expf(p.cs_f[o + Q - 1] - p.cs_f[o + r]);
-                    s = d * __expf(p.cs_b[o] - p.cs_b[o + r]);
-                } else {
-                    f = __expf(p.cs_f[o + r]);
-                    s = __expf(p.cs_b[o + r]);
-                }
-            }
-            sfs[threadIdx.x] = f;
-            sbs[threadIdx.x] = s;
-        }
-        const T *ap;
-        int64_t as;
-        if (IS_DB) { as = p.x_sl; ap = reinterpret_cast<const T *>(p.x) + b * p.x_sb + ((int64_t)c * Q + r0) * as + h * p.x_sh; }
-        else if (p.has_z) { as = (int64_t)H * P; ap = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q + r0) * as + (int64_t)h * P; }
-        else { as = p.dout_sl; ap = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + ((int64_t)c * Q + r0) * as + h * p.dout_sh; }
-        const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * N;
-        const float *s1 = (IS_DB ? p.dstates_f : p.states_f) + so;
-        const float *s2 = (IS_DB ? p.dstates_b : p.states_b) + so;
-        float uf[4] = {0.f, 0.f, 0.f, 0.f}, ub[4] = {0.f, 0.f, 0.f, 0.f};
-        float sfr[4], sbr[4];
+        float uf[QT][4], ub[QT][4];
+#pragma unroll
+        for (int q = 0; q < QT; ++q)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { uf[q][i] = 0.f; ub[q][i] = 0.f; }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            if (nt * 64 >= N) break;
-            f32x4 tf[4] = {}, tb[4] = {};
-            for (int k0 = 0; k0 < P; k0 += BK) {
-                __syncthreads();
-                tile_load_kcontig<T, T, 64>(As, ap + k0, as, limit - r0, P - k0, Ident());
-                // state[p][n] -> [n][p]: element (r = n, k = p) at s + k*N + n
-                tile_load_rcontig<T, float, 64>(Bf, s1 + (int64_t)k0 * N + nt * 64, N, N - nt * 64, P - k0, Ident());
-                tile_load_rcontig<T, float, 64>(Bb, s2 + (int64_t)k0 * N + nt * 64, N, N - nt * 64, P - k0, Ident());
-                __syncthreads();
-                mma_tile<T, 4>(tf, As + wave * 16 * LD, Bf, lane);
-                mma_tile<T, 4>(tb, As + wave * 16 * LD, Bb, lane);
-            }
+            if (nt >= nnt) break;
+            f32x4 tf[QT][4] = {}, tb[QT][4] = {};
+            for (int kc = 0; kc < nkc; ++kc, ++step) {
+                const int buf = NBUF == 2 ? (step & 1) : 0;
+                if (NBUF == 1) __syncthreads();            // the single image is still being read by slower waves
+                commit(buf);
+                typename M::Frag afc[QT][NKS];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int rl = wave * 16 + (lane >> 4) * 4 + i;
-                sfr[i] = sfs[rl];
-                sbr[i] = sbs[rl];
+                for (int q = 0; q < QT; ++q)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    uf[i] += tf[j][i] * creg[nt][j][i];
-                    ub[i] += tb[j][i] * creg[nt][j][i];
-                    tot[nt][j][i] += sfr[i] * tf[j][i] + sbr[i] * tb[j][i];
+                    for (int ks = 0; ks < NKS; ++ks) afc[q][ks] = af[q][ks];
+                __syncthreads();
+                if (step + 1 < nsteps) request(step + 1);  // in flight while this step is multiplied
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks) {
+                    const int kq = ks * KSTEP + lg * KPL;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const typename M::Frag bff = M::load(sF[buf] + xt_index<T, LDX>(j * 16 + lr, kq));
+                        const typename M::Frag bfb = M::load(sB[buf] + xt_index<T, LDX>(j * 16 + lr, kq));
+#pragma unroll
+                        for (int q = 0; q < QT; ++q) {
+                            tf[q][j] = M::mma(afc[q][ks], bff, tf[q][j]);
+                            tb[q][j] = M::mma(afc[q][ks], bfb, tb[q][j]);
+                        }
+                    }
                 }
             }
+#pragma unroll
+            for (int q = 0; q < QT; ++q)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float sf = sfs[hh - hh0][tl[q][i]], sb = sbs[hh - hh0][tl[q][i]];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        uf[q][i] += tf[q][j][i] * creg[nt][q][j][i];
+                        ub[q][i] += tb[q][j][i] * creg[nt][q][j][i];
+                        tot[nt][q][j][i] += sf * tf[q][j][i] + sb * tb[q][j][i];
+                    }
+                }
         }
         float *of = IS_DB ? p.v_f : p.u_f, *ob = IS_DB ? p.v_b : p.u_b;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = r0 + wave * 16 + (lane >> 4) * 4 + i;
-            const float a = row16_sum(uf[i]) * sfr[i], bb = row16_sum(ub[i]) * sbr[i];
-            if ((lane & 15) == 0 && r < Q) {
-                of[o + r] = a;
-                ob[o + r] = bb;
+        for (int q = 0; q < QT; ++q)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float a = row16_sum(uf[q][i]) * sfs[hh - hh0][tl[q][i]], bb = row16_sum(ub[q][i]) * sbs[hh - hh0][tl[q][i]];
+                if (lr == 0 && r0 + tl[q][i] < Q) {
+                    of[o + r0 + tl[q][i]] = a;
+                    ob[o + r0 + tl[q][i]] = bb;
+                }
             }
-        }
     }
     float *out = (IS_DB ? p.dBs : p.dCs) + (int64_t)blockIdx.z * p.batch * p.seqlen * p.ngroups * N;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int q = 0; q < QT; ++q)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int r = r0 + wave * 16 + (lane >> 4) * 4 + i, n = nt * 64 + j * 16 + (lane & 15);
-                if (r < limit && n < N)
-                    out[(((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n] = tot[nt][j][i];
-            }
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = nt * 64 + j * 16 + lr, r = r0 + tl[q][i];
+                    if (r < limit && n < N)
+                        out[(((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n] = tot[nt][q][j][i];
+                }
 }
 
 template <typename T, bool IS_DB>
 static int launch_dbdc_t(const bimamba2_params *p) {
     const int nc = nchunks(p);
-    dim3 grid(p->batch * nc * p->ngroups, (p->chunk_size + 63) / 64, dbdc_slices(p));
     const int nt = (p->dstate + 63) / 64;
-    if (nt == 1) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 1, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
-    else if (nt == 2) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 2, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
-    else if (nt <= 4) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 4, IS_DB>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    const int qt = (p->chunk_size > 128 && nt == 1) ? 2 : 1;          // 16-row tiles per wave
+    const int rows = DBDC_WAVES * 16 * qt;
+    dim3 grid(p->batch * nc * p->ngroups, (p->chunk_size + rows - 1) / rows, dbdc_slices(p));
+    constexpr int VS = 16 / (int)sizeof(T);
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    bool fast = p->headdim % 64 == 0 && p->dstate % 64 == 0;
+    if (IS_DB) fast = fast && al(p->x) && p->x_sb % VS == 0 && p->x_sl % VS == 0 && p->x_sh % VS == 0;
+    else fast = fast && (p->has_z ? al(p->dout_x) : (al(p->dout) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && p->dout_sh % VS == 0));
+#define BM2_DBDC(NTV, QTV)                                                                                                    \
+    do {                                                                                                                  \
+        if (fast) hipLaunchKernelGGL((bwd_dbdc_kernel<T, NTV, QTV, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc); \
+        else hipLaunchKernelGGL((bwd_dbdc_kernel<T, NTV, QTV, IS_DB, false>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);     \
+    } while (0)
+    if (nt == 1 && qt == 2) BM2_DBDC(1, 2);
+    else if (nt == 1) BM2_DBDC(1, 1);
+    else if (nt == 2) BM2_DBDC(2, 1);
+    else if (nt <= 4) BM2_DBDC(4, 1);
     else return BIMAMBA2_EUNSUPPORTED;
+#undef BM2_DBDC
     return check_launch();
 }
 
