@@ -501,12 +501,22 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
     for (int hbase = h_begin; hbase < h_end; hbase += DCB_HEADS) {
         const int nh = min(DCB_HEADS, h_end - hbase);
         __syncthreads();
-        for (int idx = threadIdx.x; idx < nh * 5 * 64; idx += NTHREADS) {
-            const int hh = idx / 320, which = (idx % 320) / 64, q = idx % 64;
-            const int64_t o = (((int64_t)b * H + g * hpg + hbase + hh) * nc + c) * Q;
-            const int pos = min((which < 2 ? t0 : s0) + q, Q - 1);
-            const float *src = which == 0 || which == 2 ? p.cs_f : (which == 4 ? p.dt_out : p.cs_b);
-            cst[hh][which][q] = src[o + pos];
+        for (int base = 0; base < nh * 5 * 64; base += NTHREADS * 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {                   // eight independent loads in flight per thread
+                const int idx = base + u * NTHREADS + threadIdx.x;
+                const int hh = idx / 320, which = (idx % 320) / 64, q = idx % 64;
+                const int64_t o = (((int64_t)b * H + g * hpg + hbase + min(hh, nh - 1)) * nc + c) * Q;
+                const int pos = min((which < 2 ? t0 : s0) + q, Q - 1);
+                const float *src = which == 0 || which == 2 ? p.cs_f : (which == 4 ? p.dt_out : p.cs_b);
+                v[u] = src[o + pos];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = base + u * NTHREADS + threadIdx.x;
+                if (idx < nh * 5 * 64) cst[idx / 320][(idx % 320) / 64][idx % 64] = v[u];
+            }
         }
         __syncthreads();
         if (!live) {
