@@ -22,6 +22,60 @@ __device__ __forceinline__ float to_f(bf16_t v) { return static_cast<float>(v); 
 __device__ __forceinline__ float to_f(f16_t v) { return static_cast<float>(v); }
 template <typename T> __device__ __forceinline__ T from_f(float v) { return static_cast<T>(v); }
 
+// ---- LDS accesses issued from inline assembly ---------------------------------------------------------------
+// While a direct global->LDS load (global_load_lds) is in flight, the compiler makes every LDS access it knows of wait for
+// ALL outstanding vector memory operations, which defeats prefetching through LDS.  These accessors hide the DS
+// instruction from it.  Protocol: raw_lds_read / raw_lds_write any number of times, then raw_lds_wait(), then
+// raw_lds_use(v) on every value read before its first use (the empty asm ties the value to the wait, in program order).
+// With RAW = false they are ordinary accesses and the other two are no-ops.
+__device__ __forceinline__ unsigned lds_addr(const void *p) {
+    return (unsigned)(size_t)(const __attribute__((address_space(3))) void *)p;
+}
+template <typename V, bool RAW = true> __device__ __forceinline__ V raw_lds_read(const void *p) {
+    if constexpr (!RAW) return *reinterpret_cast<const V *>(p);
+    else {
+        V v;
+        static_assert(sizeof(V) == 16 || sizeof(V) == 4, "raw_lds_read: 4 or 16 bytes");
+        if constexpr (sizeof(V) == 16) asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+        else asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(lds_addr(p)) : "memory");
+        return v;
+    }
+}
+// the same on an LDS byte address with a compile-time offset (goes into the instruction's offset field)
+template <typename V, int OFF> __device__ __forceinline__ V raw_lds_read_at(unsigned addr) {
+    V v;
+    static_assert(sizeof(V) == 16 || sizeof(V) == 4, "raw_lds_read_at: 4 or 16 bytes");
+    static_assert(OFF >= 0 && OFF < 65536, "DS offset field is 16 bits");
+    if constexpr (sizeof(V) == 16) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    else asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF> __device__ __forceinline__ void raw_lds_write_at(unsigned addr, float v) {
+    static_assert(OFF >= 0 && OFF < 65536, "DS offset field is 16 bits");
+    asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
+}
+template <int OFF> __device__ __forceinline__ void raw_lds_write128_at(unsigned addr, f32x4 v) {
+    static_assert(OFF >= 0 && OFF < 65536, "DS offset field is 16 bits");
+    asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
+}
+template <bool RAW = true> __device__ __forceinline__ void raw_lds_write(float *p, float v) {
+    if constexpr (!RAW) *p = v;
+    else asm volatile("ds_write_b32 %0, %1" ::"v"(lds_addr(p)), "v"(v) : "memory");
+}
+template <bool RAW = true> __device__ __forceinline__ void raw_lds_wait() {
+    if constexpr (RAW) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+// Workgroup barrier to go with them: __syncthreads() carries fences that drain every outstanding vector memory operation
+// when a direct global->LDS load is in flight; the bare barrier does not.  All LDS traffic around it must be raw and
+// settled with raw_lds_wait() (writes) resp. the caller's own vmcnt wait (direct loads) beforehand.
+template <bool RAW = true> __device__ __forceinline__ void raw_lds_barrier() {
+    if constexpr (RAW) __builtin_amdgcn_s_barrier();
+    else __syncthreads();
+}
+template <bool RAW = true, typename V> __device__ __forceinline__ void raw_lds_use(V &v) {
+    if constexpr (RAW) asm volatile("" : "+v"(v));
+}
+
 // ---- MFMA 16x16 fragments -----------------------------------------------------------------------------
 // Output tile D (16x16, f32): lane l holds rows 4*(l/16)+i (i=0..3) of column l%16.
 // A operand: lane l holds KPL consecutive k of row l%16 starting at KPL*(l/16); B operand likewise for

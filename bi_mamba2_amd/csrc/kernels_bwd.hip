@@ -457,6 +457,98 @@ constexpr int DCB_HEADS = 32;
 constexpr int DCB_SLICES_MAX = 4;
 constexpr int DCB_VEC = 2 * 64;      // floats per tile and head in da_intra
 
+// Per head: turns the G tile (acc) into this head's share of dCB (added to dcb) and into the column / row sums of W that
+// chunk_cumsum_bwd assembles.  cs = {cs_f[t], cs_b[t], cs_f[s], cs_b[s], dt[s]} of the tile (LDS), pb = exchange buffer
+// of the four waves (LDS), tv = the (tile, head) slot of da_intra.  Contains one workgroup barrier.
+template <typename T>
+__device__ __forceinline__ void dcb_finish_head(f32x4 (&acc)[4], f32x4 (&dcb)[4], const f32x4 (&cbr)[4], const float (*cs)[64],
+                                                float (*pb)[64], float *tv, const int (&tl)[4], int st, int tt) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lr = lane & 15;
+    float cft[4], cbt[4], dtv[4], cfs[4], cbs[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        cft[i] = cs[0][tl[i]];
+        cbt[i] = cs[1][tl[i]];
+        cfs[i] = cs[2][i * 16 + lr];
+        cbs[i] = cs[3][i * 16 + lr];
+        dtv[i] = cs[4][i * 16 + lr];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+    }
+    // column sums (this wave's 16 rows) and row sums of W; on the diagonal tile one pair per direction
+    float cwa[4], cwb[4], rwa[4] = {0.f, 0.f, 0.f, 0.f}, rwb[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int sl = j * 16 + lr;
+        float ca = 0.f, cb2 = 0.f;
+        if (st != tt) {
+            // one direction only: forward below the diagonal, reverse above it
+            const float csv = st < tt ? cfs[j] : cbs[j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float v = acc[j][i] * dtv[j] * __expf((st < tt ? cft[i] : cbt[i]) - csv);
+                dcb[j][i] += v;
+                const float w = v * cbr[j][i];
+                ca += w;
+                rwa[i] += w;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float gv = acc[j][i] * dtv[j];
+                const float f = (sl <= tl[i]) ? gv * __expf(cft[i] - cfs[j]) : 0.f;
+                const float r = (sl >= tl[i]) ? gv * __expf(cbt[i] - cbs[j]) : 0.f;
+                dcb[j][i] += f + r;
+                const float wf = (sl < tl[i]) ? f * cbr[j][i] : 0.f;
+                const float wb = (sl > tl[i]) ? r * cbr[j][i] : 0.f;
+                ca += wf; rwa[i] += wf;
+                cb2 += wb; rwb[i] += wb;
+            }
+        }
+        cwa[j] = ca;
+        cwb[j] = cb2;
+    }
+    // hand the sums to the other waves through LDS (double-buffered by head parity)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float v = cwa[j];
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        if (lane < 16) pb[wave][j * 16 + lane] = v;
+        if (st == tt) {
+            float u = cwb[j];
+            u += __shfl_xor(u, 16, 64);
+            u += __shfl_xor(u, 32, 64);
+            if (lane < 16) pb[4 + wave][j * 16 + lane] = u;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float r = row16_sum(rwa[i]);
+        if (lr == 0) pb[8][tl[i]] = r;
+        if (st == tt) {
+            const float u = row16_sum(rwb[i]);
+            if (lr == 0) pb[9][tl[i]] = u;
+        }
+    }
+    __syncthreads();
+    // off-diagonal: [0] = column sums, [1] = row sums.  diagonal: [0] = cw_f - rw_f, [1] = cw_b - rw_b
+    // (the consumer turns them into the tile's own contribution with a prefix resp. suffix sum)
+    if (threadIdx.x < 128) {
+        const int q = threadIdx.x & 63, which = threadIdx.x >> 6;
+        const int base = (st != tt || which == 0) ? 0 : 4;
+        float a0 = pb[base][q], a1 = pb[base + 1][q];
+        float a2 = pb[base + 2][q], a3 = pb[base + 3][q];
+        float r8 = pb[st != tt ? 8 : 8 + which][q];
+            float v;
+        if (st != tt) v = which == 0 ? a0 + a1 + a2 + a3 : r8;
+        else v = a0 + a1 + a2 + a3 - r8;
+        tv[which * 64 + q] = v;
+    }
+}
+
 template <typename T, bool FAST>
 __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params p, int nc, int nqt) {
     typedef Mma<T> M;
@@ -570,83 +662,8 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
         };
         f32x4 acc[4] = {};
         auto finish_head = [&](int hh) __attribute__((always_inline)) {
-            const float(*cs)[64] = cst[hh];
-            float cft[4], cbt[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { cft[i] = cs[0][tl[i]]; cbt[i] = cs[1][tl[i]]; }
-            // column sums (this wave's 16 rows) and row sums of W; on the diagonal tile one pair per direction
-            float cwa[4], cwb[4], rwa[4] = {0.f, 0.f, 0.f, 0.f}, rwb[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int sl = j * 16 + lr;
-                const float dtv = cs[4][sl];
-                float ca = 0.f, cb2 = 0.f;
-                if (st != tt) {
-                    // one direction only: forward below the diagonal, reverse above it
-                    const float csv = st < tt ? cs[2][sl] : cs[3][sl];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float v = acc[j][i] * dtv * __expf((st < tt ? cft[i] : cbt[i]) - csv);
-                        dcb[j][i] += v;
-                        const float w = v * cbr[j][i];
-                        ca += w;
-                        rwa[i] += w;
-                    }
-                } else {
-                    const float cfs = cs[2][sl], cbs = cs[3][sl];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float gv = acc[j][i] * dtv;
-                        const float f = (sl <= tl[i]) ? gv * __expf(cft[i] - cfs) : 0.f;
-                        const float r = (sl >= tl[i]) ? gv * __expf(cbt[i] - cbs) : 0.f;
-                        dcb[j][i] += f + r;
-                        const float wf = (sl < tl[i]) ? f * cbr[j][i] : 0.f;
-                        const float wb = (sl > tl[i]) ? r * cbr[j][i] : 0.f;
-                        ca += wf; rwa[i] += wf;
-                        cb2 += wb; rwb[i] += wb;
-                    }
-                }
-                cwa[j] = ca;
-                cwb[j] = cb2;
-            }
-            // hand the sums to the other waves through LDS (double-buffered by head parity)
-            float(*pb)[64] = part[hh & 1];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float v = cwa[j];
-                v += __shfl_xor(v, 16, 64);
-                v += __shfl_xor(v, 32, 64);
-                if (lane < 16) pb[wave][j * 16 + lane] = v;
-                if (st == tt) {
-                    float u = cwb[j];
-                    u += __shfl_xor(u, 16, 64);
-                    u += __shfl_xor(u, 32, 64);
-                    if (lane < 16) pb[4 + wave][j * 16 + lane] = u;
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float r = row16_sum(rwa[i]);
-                if (lr == 0) pb[8][tl[i]] = r;
-                if (st == tt) {
-                    const float u = row16_sum(rwb[i]);
-                    if (lr == 0) pb[9][tl[i]] = u;
-                }
-            }
-            __syncthreads();
-            // off-diagonal: [0] = column sums, [1] = row sums.  diagonal: [0] = cw_f - rw_f, [1] = cw_b - rw_b
-            // (the consumer turns them into the tile's own contribution with a prefix resp. suffix sum)
-            if (threadIdx.x < 128) {
-                const int h = g * hpg + hbase + hh;
-                const int64_t o = (((int64_t)b * H + h) * nc + c);
-                float *tv = p.da_intra + (o * nqt * nqt + tile) * DCB_VEC;
-                const int q = threadIdx.x & 63, which = threadIdx.x >> 6;
-                float v;
-                if (st != tt) v = which == 0 ? pb[0][q] + pb[1][q] + pb[2][q] + pb[3][q] : pb[8][q];
-                else if (which == 0) v = pb[0][q] + pb[1][q] + pb[2][q] + pb[3][q] - pb[8][q];
-                else v = pb[4][q] + pb[5][q] + pb[6][q] + pb[7][q] - pb[9][q];
-                tv[which * 64 + q] = v;
-            }
+            const int64_t o = (((int64_t)b * H + g * hpg + hbase + hh) * nc + c);
+            dcb_finish_head<T>(acc, dcb, cbr, cst[hh], part[hh & 1], p.da_intra + (o * nqt * nqt + tile) * DCB_VEC, tl, st, tt);
         };
         issue(0);
         for (int it = 0; it < nit; ++it) {
@@ -719,6 +736,378 @@ int dcb_slices(const bimamba2_params *p) {
     return std::max(1, std::min(DCB_SLICES_MAX, hpg / 32));
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Variant for 16-bit types with headdim % 64 == 0, chunk_size % 64 == 0 and aligned operands.
+//
+// The kernel is bound by its instruction count, not by memory, so everything per head is pared down:
+//  * the dout tile, the x tile and the decay vectors of each (head, 64-wide headdim chunk) step travel from global memory
+//    straight into a ring of LDS slots (global_load_lds, 16 bytes per lane, no registers, no address arithmetic beyond
+//    one 64-bit add per request), two steps ahead of the one being multiplied; 16-byte units are XOR-swizzled by the row
+//    so that the fragment reads spread over the banks;
+//  * a wave owns 16 rows t; against a block of 16 columns s that lies wholly below (s < t) or above (s > t) the diagonal
+//    the decay factor separates, exp(cs[t] - cs[s]) = exp(cs[t] - m) * exp(m - cs[s]) with m taken at the edge of the
+//    wave's rows nearest to the columns, so that both factors are <= 1 for A <= 0: 8 exponentials instead of 16 per
+//    block and the factors move out of the row and column sums.  Only the 16x16 block on the diagonal takes the masked
+//    two-direction path;
+//  * the column sums over the four 16-lane groups come from one MFMA with a matrix of ones per column block.
+// ---------------------------------------------------------------------------------------------------------
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    // at most N vector-memory operations of this wave outstanding; lgkmcnt / expcnt fields left at "no wait"
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+typedef const __attribute__((address_space(1))) void *gbl_ptr_t;
+
+// sum of v over the four lanes l%16, l%16+16, l%16+32, l%16+48, delivered to all of them: D = ones(16x4) * B where lane l
+// supplies B[k = l/16][n = l%16]
+__device__ __forceinline__ float lanegroup_sum_mfma(float v) {
+    const f32x4 d = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, v, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    return d[0];
+}
+
+constexpr int DCB_RING = 3;
+constexpr int DCB_TILE_B = 64 * 64 * 2;                    // one 64 x 64 tile of 16-bit elements
+constexpr int DCB_CS_OFF = 2 * DCB_TILE_B;                 // cs_f[t], cs_b[t], cs_f[s], cs_b[s], dt[s]: 5 x 64 floats
+constexpr int DCB_SLOT_B = DCB_CS_OFF + 5 * 64 * 4;
+constexpr int DCB_PART_OFF = DCB_RING * DCB_SLOT_B;        // per-wave column sums (f: 0-3, b: 4-7), row sums (f: 8, b: 9)
+constexpr int DCB_PART_B = 10 * 64 * 4;
+
+#ifdef BM2_DBG_TIME
+#define TSR(k) do { long long _t = wall_clock64(); ph[k] += _t - tlast; tlast = _t; } while (0)
+#else
+#define TSR(k)
+#endif
+
+template <typename T>
+__global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_params p, int nc, int nqt) {
+    typedef Mma<T> M;
+    typedef typename M::Frag Frag;
+    static_assert(sizeof(T) == 2, "ring variant is for 16-bit operands");
+    constexpr int KC = 64, NKS = 2;                            // 64 headdim columns = 8 units of 16 bytes per row
+    __shared__ __attribute__((aligned(16))) unsigned char smem[DCB_PART_OFF + 2 * DCB_PART_B];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lr = lane & 15, lg = lane >> 4;
+    // the tiles on the diagonal cost more: they come first in launch order, which spreads them over the compute units
+    int tt, st;
+    if ((int)blockIdx.y < nqt) tt = st = blockIdx.y;
+    else {
+        const int k = blockIdx.y - nqt;
+        tt = k / (nqt - 1);
+        st = k % (nqt - 1);
+        st += st >= tt;
+    }
+    const int tile = tt * nqt + st;
+    const int g = blockIdx.x % p.ngroups, bc = blockIdx.x / p.ngroups, c = bc % nc, b = bc / nc;
+    const int Q = p.chunk_size, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int t0 = tt * 64, s0 = st * 64;
+    const bool live = t0 < limit && s0 < limit;
+    const int trow = wave * 16 + lg * 4;                       // first of this lane's four accumulator rows
+    f32x4 cbr[4] = {}, dcb[4] = {};
+    const int hps = (hpg + gridDim.z - 1) / gridDim.z;
+    const int h_begin = blockIdx.z * hps, h_end = min(hpg, h_begin + hps);
+    const int nkc = P / KC, nhs = h_end - h_begin, nit = nhs * nkc;
+    const int h0 = g * hpg + h_begin;
+    const int64_t tv_head = (int64_t)nc * nqt * nqt * DCB_VEC;
+    float *tv0 = p.da_intra + ((((int64_t)b * H + h0) * nc + c) * nqt * nqt + tile) * DCB_VEC;
+    if (!live) {
+        for (int hh = 0; hh < nhs; ++hh)
+            for (int i = threadIdx.x; i < DCB_VEC; i += NTHREADS) tv0[hh * tv_head + i] = 0.f;
+    } else {
+        const unsigned sbase = lds_addr(smem);
+        // ---- requests: unit u = i*256 + thread of a 64 x 64 tile is row r = u / 8, 16-byte chunk (u % 8) ^ (r % 8)
+        const T *ysrc[2], *xsrc[2];
+        int64_t y_head, y_row;
+        {
+            const T *yp;
+            if (p.has_z) { y_row = (int64_t)H * P; y_head = P; yp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * y_row + (int64_t)h0 * P; }
+            else { y_row = p.dout_sl; y_head = p.dout_sh; yp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * y_row + h0 * p.dout_sh; }
+            const T *xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h0 * p.x_sh;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int u = i * NTHREADS + threadIdx.x, r = u >> 3, col = ((u & 7) ^ (r & 7)) * 8;
+                ysrc[i] = yp + (int64_t)min(t0 + r, limit - 1) * y_row + col;
+                xsrc[i] = xp + (int64_t)min(s0 + r, limit - 1) * p.x_sl + col;
+            }
+        }
+        const float *csrc;                                     // threads 0..79: 16-byte unit of the five decay vectors
+        {
+            const int which = min((int)threadIdx.x >> 4, 4), j4 = (threadIdx.x & 15) * 4;
+            const int64_t o = (((int64_t)b * H + h0) * nc + c) * Q + (which < 2 ? t0 : s0) + j4;
+            csrc = (which == 0 || which == 2 ? p.cs_f : (which == 4 ? p.dt_out : p.cs_b)) + o;
+        }
+        const int64_t x_head = p.x_sh, cs_head = (int64_t)nc * Q;
+        int ikc = 0;
+        // requests one step into `slot` and moves the source pointers on to the next step
+        auto issue = [&](int slot) __attribute__((always_inline)) {
+            unsigned char *sl = smem + slot * DCB_SLOT_B + wave * 1024;
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)ysrc[0], (lds_ptr_t)(sl), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)ysrc[1], (lds_ptr_t)(sl + 4096), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)xsrc[0], (lds_ptr_t)(sl + DCB_TILE_B), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)xsrc[1], (lds_ptr_t)(sl + DCB_TILE_B + 4096), 16, 0, 0);
+            if (threadIdx.x < 80) __builtin_amdgcn_global_load_lds((gbl_ptr_t)csrc, (lds_ptr_t)(sl + DCB_CS_OFF), 16, 0, 0);
+            const bool last = ++ikc == nkc;
+            if (last) ikc = 0;
+            const int64_t dy = last ? y_head - (nkc - 1) * KC : KC, dx = last ? x_head - (nkc - 1) * KC : KC;
+            ysrc[0] += dy; ysrc[1] += dy;
+            xsrc[0] += dx; xsrc[1] += dx;
+            if (last) csrc += cs_head;
+        };
+        // ---- per-lane LDS byte offsets inside a slot
+        unsigned a_off[NKS], b_off[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const int ch = (ks * 4 + lg) ^ (lr & 7);
+            a_off[ks] = ((wave * 16 + lr) * 8 + ch) * 16;
+            b_off[ks] = DCB_TILE_B + (lr * 8 + ch) * 16;       // column block j adds j * 2048
+        }
+        const unsigned ct_off = DCB_CS_OFF + trow * 4, cc_off = DCB_CS_OFF + lr * 4, cm_off = DCB_CS_OFF + wave * 64;
+        const int rows_left = limit - t0 - trow;               // accumulator rows i >= rows_left lie past the sequence end
+
+        f32x4 acc[4] = {};
+        issue(0);
+        if (nit > 1) issue(1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float *cbg = p.CB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int t = t0 + trow + i, s = s0 + j * 16 + lr;
+                cbr[j][i] = (t < limit && s < limit) ? cbg[(int64_t)t * Q + s] : 0.f;
+            }
+        }
+        // settle these register loads here: inside the loop a wait for them would drain the ring's requests as well
+        wait_vmcnt<0>();
+#ifdef BM2_DBG_TIME
+        long long ph[12] = {}, tlast = wall_clock64();
+        const long long tstart = tlast;
+#endif
+        int slot = 0, slot2 = 2 % DCB_RING, kc = 0, par = 0;
+        float *tv = tv0 + (wave & 1) * 64 + lane;
+        for (int it = 0; it < nit; ++it) {
+            if (it + 2 < nit) issue(slot2);
+            TSR(0);
+            // the requests of step `it` went out before those of the (up to two) steps after it; waves 0 and 1 make
+            // five requests per step, the others four
+            const int newer = min(2, nit - 1 - it);
+            if (wave < 2) {
+                if (newer == 2) wait_vmcnt<10>();
+                else if (newer == 1) wait_vmcnt<5>();
+                else wait_vmcnt<0>();
+            } else {
+                if (newer == 2) wait_vmcnt<8>();
+                else if (newer == 1) wait_vmcnt<4>();
+                else wait_vmcnt<0>();
+            }
+            TSR(1);
+            raw_lds_barrier();
+            TSR(2);
+            const unsigned sb = sbase + slot * DCB_SLOT_B;
+            Frag af[NKS], bf[4][NKS];
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                af[ks] = raw_lds_read_at<Frag, 0>(sb + a_off[ks]);
+                bf[0][ks] = raw_lds_read_at<Frag, 0>(sb + b_off[ks]);
+                bf[1][ks] = raw_lds_read_at<Frag, 2048>(sb + b_off[ks]);
+                bf[2][ks] = raw_lds_read_at<Frag, 4096>(sb + b_off[ks]);
+                bf[3][ks] = raw_lds_read_at<Frag, 6144>(sb + b_off[ks]);
+            }
+            raw_lds_wait();
+            TSR(3);
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                raw_lds_use(af[ks]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    raw_lds_use(bf[j][ks]);
+                    acc[j] = M::mma(af[ks], bf[j][ks], acc[j]);
+                }
+            }
+#ifdef BM2_DBG_TIME
+            asm volatile("" ::"v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3]));
+#endif
+            TSR(4);
+            if (++kc < nkc) {
+                raw_lds_barrier();         // the slot is overwritten by the requests of the next iteration
+            } else {
+                kc = 0;
+                // ---- decay vectors of this head
+                f32x4 cft_ = raw_lds_read_at<f32x4, 0>(sb + ct_off), cbt_ = raw_lds_read_at<f32x4, 256>(sb + ct_off);
+                float cfs[4], cbs[4], dts[4];
+                cfs[0] = raw_lds_read_at<float, 512>(sb + cc_off); cfs[1] = raw_lds_read_at<float, 512 + 64>(sb + cc_off);
+                cfs[2] = raw_lds_read_at<float, 512 + 128>(sb + cc_off); cfs[3] = raw_lds_read_at<float, 512 + 192>(sb + cc_off);
+                cbs[0] = raw_lds_read_at<float, 768>(sb + cc_off); cbs[1] = raw_lds_read_at<float, 768 + 64>(sb + cc_off);
+                cbs[2] = raw_lds_read_at<float, 768 + 128>(sb + cc_off); cbs[3] = raw_lds_read_at<float, 768 + 192>(sb + cc_off);
+                dts[0] = raw_lds_read_at<float, 1024>(sb + cc_off); dts[1] = raw_lds_read_at<float, 1024 + 64>(sb + cc_off);
+                dts[2] = raw_lds_read_at<float, 1024 + 128>(sb + cc_off); dts[3] = raw_lds_read_at<float, 1024 + 192>(sb + cc_off);
+                // reference points: cs_f at the first, cs_b at the last of the wave's 16 rows
+                float mf = raw_lds_read_at<float, 0>(sb + cm_off), mb = raw_lds_read_at<float, 256 + 60>(sb + cm_off);
+                raw_lds_wait();
+                raw_lds_use(cft_); raw_lds_use(cbt_); raw_lds_use(mf); raw_lds_use(mb);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { raw_lds_use(cfs[j]); raw_lds_use(cbs[j]); raw_lds_use(dts[j]); }
+                TSR(5);
+                if (rows_left < 4) {
+                    // rows past the end of the sequence were read from a valid row: drop them
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (i >= rows_left) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) acc[j][i] = 0.f;
+                        }
+                }
+                // W = dCB_h * CB; col*[j]: this lane's part of the column sums, row*[i]: of the row sums
+                float colF[4], colB[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4], rowB[4] = {0.f, 0.f, 0.f, 0.f};
+                // one 16 x 16 block whose columns lie on one side of the wave's rows: factors E (rows) and Fd (columns)
+                auto sep_block = [&](int j, const float (&E)[4], float Fd, float &col, float (&rp)[4]) __attribute__((always_inline)) {
+                    float cp = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float a = acc[j][i], y = a * cbr[j][i];
+                        cp = __builtin_fmaf(y, E[i], cp);
+                        rp[i] = __builtin_fmaf(y, Fd, rp[i]);
+                        dcb[j][i] = __builtin_fmaf(a * E[i], Fd, dcb[j][i]);
+                    }
+                    col = cp * Fd;
+                };
+                if (st != tt) {
+                    const bool lower = st < tt;                // forward direction below the diagonal, reverse above it
+                    float E[4], rp[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) E[i] = __expf(lower ? cft_[i] - mf : cbt_[i] - mb);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) sep_block(j, E, dts[j] * __expf(lower ? mf - cfs[j] : mb - cbs[j]), colF[j], rp);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) rowF[i] = rp[i] * E[i];
+                } else {
+                    float Ef[4], Eb[4], rpf[4] = {0.f, 0.f, 0.f, 0.f}, rpb[4] = {0.f, 0.f, 0.f, 0.f};
+                    float df[4] = {0.f, 0.f, 0.f, 0.f}, db[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { Ef[i] = __expf(cft_[i] - mf); Eb[i] = __expf(cbt_[i] - mb); }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (j < wave) { sep_block(j, Ef, dts[j] * __expf(mf - cfs[j]), colF[j], rpf); }
+                        else if (j > wave) { colF[j] = 0.f; sep_block(j, Eb, dts[j] * __expf(mb - cbs[j]), colB[j], rpb); }
+                        else {
+                            // the block on the diagonal: both directions, masked element by element
+                            float ca = 0.f, cb2 = 0.f;
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) {
+                                const int ti = lg * 4 + i;     // row and column (lr) inside the block
+                                const float gv = acc[j][i] * dts[j];
+                                const float f = (lr <= ti) ? gv * __expf(cft_[i] - cfs[j]) : 0.f;
+                                const float r = (lr >= ti) ? gv * __expf(cbt_[i] - cbs[j]) : 0.f;
+                                dcb[j][i] += f + r;
+                                const float wf = (lr < ti) ? f * cbr[j][i] : 0.f;
+                                const float wb = (lr > ti) ? r * cbr[j][i] : 0.f;
+                                ca += wf; df[i] += wf;
+                                cb2 += wb; db[i] += wb;
+                            }
+                            colF[j] = ca;
+                            colB[j] = cb2;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { rowF[i] = __builtin_fmaf(rpf[i], Ef[i], df[i]); rowB[i] = __builtin_fmaf(rpb[i], Eb[i], db[i]); }
+                }
+#ifdef BM2_DBG_TIME
+                asm volatile("" ::"v"(colF[0]), "v"(colF[1]), "v"(colF[2]), "v"(colF[3]), "v"(rowF[0]), "v"(rowF[1]), "v"(rowF[2]), "v"(rowF[3]));
+#endif
+                TSR(6);
+                // ---- hand the sums to the other waves through LDS (double-buffered by head parity)
+                const unsigned pb = sbase + DCB_PART_OFF + par * DCB_PART_B;
+                {
+                    float cs4[4], cs4b[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) cs4[j] = lanegroup_sum_mfma(colF[j]);
+                    if (st == tt) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) cs4b[j] = lanegroup_sum_mfma(colB[j]);
+                    }
+                    f32x4 rs, rsb;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) rs[i] = row16_sum(rowF[i]);
+                    if (st == tt) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) rsb[i] = row16_sum(rowB[i]);
+                    }
+                    const unsigned pw = pb + wave * 256 + lr * 4;
+                    if (lane < 16) {
+                        raw_lds_write_at<0>(pw, cs4[0]); raw_lds_write_at<64>(pw, cs4[1]);
+                        raw_lds_write_at<128>(pw, cs4[2]); raw_lds_write_at<192>(pw, cs4[3]);
+                        if (st == tt) {
+                            raw_lds_write_at<1024>(pw, cs4b[0]); raw_lds_write_at<1024 + 64>(pw, cs4b[1]);
+                            raw_lds_write_at<1024 + 128>(pw, cs4b[2]); raw_lds_write_at<1024 + 192>(pw, cs4b[3]);
+                        }
+                    }
+                    if (lr == 0) {
+                        raw_lds_write128_at<2048>(pb + trow * 4, rs);
+                        if (st == tt) raw_lds_write128_at<2048 + 256>(pb + trow * 4, rsb);
+                    }
+                }
+                raw_lds_wait();
+                TSR(7);
+                raw_lds_barrier();
+                TSR(8);
+                // off-diagonal: [0] = column sums, [1] = row sums.  diagonal: [0] = cw_f - rw_f, [1] = cw_b - rw_b
+                // (the consumer turns them into the tile's own contribution with a prefix resp. suffix sum)
+                if (wave < 2) {
+                    const unsigned pq = pb + lane * 4;
+                    float v;
+                    if (st != tt && wave == 1) {
+                        v = raw_lds_read_at<float, 2048>(pq);
+                        raw_lds_wait();
+                        raw_lds_use(v);
+                    } else {
+                        float a0, a1, a2, a3, r8 = 0.f;
+                        if (wave == 0) {
+                            a0 = raw_lds_read_at<float, 0>(pq); a1 = raw_lds_read_at<float, 256>(pq);
+                            a2 = raw_lds_read_at<float, 512>(pq); a3 = raw_lds_read_at<float, 768>(pq);
+                            if (st == tt) r8 = raw_lds_read_at<float, 2048>(pq);
+                        } else {
+                            a0 = raw_lds_read_at<float, 1024>(pq); a1 = raw_lds_read_at<float, 1024 + 256>(pq);
+                            a2 = raw_lds_read_at<float, 1024 + 512>(pq); a3 = raw_lds_read_at<float, 1024 + 768>(pq);
+                            r8 = raw_lds_read_at<float, 2048 + 256>(pq);
+                        }
+                        raw_lds_wait();
+                        raw_lds_use(a0); raw_lds_use(a1); raw_lds_use(a2); raw_lds_use(a3); raw_lds_use(r8);
+                        v = a0 + a1 + a2 + a3 - r8;
+                    }
+                    *tv = v;
+                }
+                tv += tv_head;
+                par ^= 1;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                TSR(9);
+            }
+            slot = slot + 1 == DCB_RING ? 0 : slot + 1;
+            slot2 = slot2 + 1 == DCB_RING ? 0 : slot2 + 1;
+        }
+#ifdef BM2_DBG_TIME
+        if (threadIdx.x == 0) {
+            long long *lg2 = reinterpret_cast<long long *>(p.workspace) + (blockIdx.y * gridDim.x + blockIdx.x) * 16;
+            for (int k = 0; k < 10; ++k) lg2[k] = ph[k];
+            lg2[10] = tstart; lg2[11] = tlast;
+        }
+#endif
+    }
+    const int64_t oo = ((int64_t)blockIdx.z * gridDim.x + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    float *out = p.dCB + oo, *outT = p.dCBT + oo;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int s = s0 + j * 16 + lr;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[(int64_t)(t0 + trow + i) * Q + s] = dcb[j][i];
+        *reinterpret_cast<f32x4 *>(outT + (int64_t)s * Q + t0 + trow) = dcb[j];
+    }
+}
+
+template <typename T> static void launch_dcb_ring(dim3 grid, const bimamba2_params *p, int nc, int nqt) {
+    if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((bwd_dcb_ring_kernel<T>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
+}
+
 template <typename T>
 static int launch_dcb_t(const bimamba2_params *p) {
     const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
@@ -728,7 +1117,8 @@ static int launch_dcb_t(const bimamba2_params *p) {
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     bool fast = p->headdim % (sizeof(T) == 2 ? 64 : 16) == 0 && al(p->x) && p->x_sb % VS == 0 && p->x_sl % VS == 0 && p->x_sh % VS == 0;
     fast = fast && (p->has_z ? al(p->dout_x) : (al(p->dout) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && p->dout_sh % VS == 0));
-    if (fast) hipLaunchKernelGGL((bwd_dcb_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
+    if (fast && sizeof(T) == 2 && p->chunk_size % 64 == 0) launch_dcb_ring<T>(grid, p, nc, nqt);
+    else if (fast) hipLaunchKernelGGL((bwd_dcb_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
     else hipLaunchKernelGGL((bwd_dcb_kernel<T, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
     if (slices > 1) {
         // (Q*Q is a multiple of 4 only when Q is even; odd chunk sizes are rejected by the 16-byte requirement below)
