@@ -10,6 +10,7 @@ duration measured here with HIP events on the launch stream) and a CPU baseline 
 flip-and-sum path in PyTorch on the host cores, on a bounded sample).
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -34,25 +35,29 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def stage_table(w, e):
-    """Algorithmic flops and bytes per launch of every stage kernel (e = bytes per element of x/B/C/z)."""
+def stage_table(w, e, fused=(False, False)):
+    """Algorithmic flops and bytes per launch of every stage kernel (e = bytes per element of x/B/C/z).
+    fused[0] / fused[1]: the forward scan / the dx kernel rebuilds its CB tiles from C and B instead of reading them."""
     B, L, H, P, G, N, Q = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate", "chunk_size"))
     nc = (L + Q - 1) // Q
     u, ug = B * nc * H, B * nc * G                 # (b, c, h) and (b, c, g) units
     T4, T2, T1 = B * L * H * P, B * L * G * N, B * H * nc * Q
     st = 4 * B * nc * H * P * N                     # one float32 state tensor
     cb = 4 * ug * Q * Q
+    scan_cb = [(u * 2 * Q * Q * N, e * T2) if f else (0, cb) for f in fused]   # (extra flops, bytes) for the CB tiles
     return {
         # entry point: (flops, bytes)
         "bimamba2_chunk_cumsum_fwd": (0, 4 * B * L * H + 3 * 4 * T1),
         "bimamba2_bmm_chunk_fwd": (ug * 2 * Q * Q * N, 2 * e * T2 + cb),
         "bimamba2_chunk_state_fwd": (u * 4 * P * N * Q, e * T4 + e * T2 + 3 * 4 * T1 + 2 * st),
         "bimamba2_state_passing_fwd": (0, 4 * st),
-        "bimamba2_chunk_scan_fwd": (u * (2 * Q * Q * P + 4 * Q * P * N), 4 * e * T4 + e * T2 + 3 * 4 * T1 + 2 * st + cb),
+        "bimamba2_chunk_scan_fwd": (u * (2 * Q * Q * P + 4 * Q * P * N) + scan_cb[0][0],
+                                    4 * e * T4 + e * T2 + 3 * 4 * T1 + 2 * st + scan_cb[0][1]),
         "bimamba2_chunk_scan_bwd_dz": (0, 5 * e * T4),
         "bimamba2_chunk_scan_bwd_dstates": (u * 4 * P * N * Q, e * T4 + e * T2 + 2 * 4 * T1 + 2 * st),
         "bimamba2_state_passing_bwd": (0, 6 * st),
-        "bimamba2_chunk_scan_bwd_dx": (u * (2 * Q * Q * P + 4 * Q * P * N), 3 * e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + cb),
+        "bimamba2_chunk_scan_bwd_dx": (u * (2 * Q * Q * P + 4 * Q * P * N) + scan_cb[1][0],
+                                       3 * e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + scan_cb[1][1]),
         "bimamba2_chunk_state_bwd_db": (u * 4 * Q * P * N, e * T4 + e * T2 + 5 * 4 * T1 + 2 * st + 4 * T2),
         "bimamba2_chunk_scan_bwd_dc": (u * 4 * Q * P * N, e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + 4 * T2),
         "bimamba2_chunk_scan_bwd_dcb": (u * 2 * Q * Q * P, 2 * e * T4 + 3 * 4 * T1 + 2 * cb + 4 * B * H * nc * ((Q + 63) // 64) ** 2 * 128),
@@ -192,12 +197,19 @@ def main():
     c.run("bimamba2_fwd")
     c.run("bimamba2_bwd")
     torch.cuda.synchronize()
-    table = stage_table(w, e)
+    reads_cb = [_lib.load().bimamba2_chunk_scan_reads_cb(ctypes.byref(c.p), d) for d in (0, 1)]
+    table = stage_table(w, e, fused=(reads_cb[0] == 0, reads_cb[1] == 0))
     kernels = {}
     reps = max(10, args.steps)
     for entry, (flops, nbytes) in table.items():
         if entry == "bimamba2_chunk_scan_bwd_dz" and not has_z:
             continue
+        # time the scan stages the way the composites launch them: without CB / CBT when the kernel rebuilds it
+        hidden = {"bimamba2_chunk_scan_fwd": ("CB", 0), "bimamba2_chunk_scan_bwd_dx": ("CBT", 1)}.get(entry)
+        kept = None
+        if hidden and reads_cb[hidden[1]] == 0:
+            kept = getattr(c.p, hidden[0])
+            setattr(c.p, hidden[0], None)
         for _ in range(3):
             c.run(entry)
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -206,6 +218,8 @@ def main():
             c.run(entry)
         ev1.record()
         torch.cuda.synchronize()
+        if kept is not None:
+            setattr(c.p, hidden[0], kept)
         us = ev0.elapsed_time(ev1) * 1e3 / reps
         kernels[entry] = {"us": round(us, 2), "gflop": round(flops / 1e9, 3), "mbytes": round(nbytes / 1e6, 2),
                           "tflops": round(flops / us / 1e6, 2), "gbs": round(nbytes / us / 1e3, 1)}

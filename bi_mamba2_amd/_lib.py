@@ -44,7 +44,7 @@ ENTRY_POINTS = (
     "bimamba2_chunk_scan_bwd_dcb", "bimamba2_bmm_chunk_bwd", "bimamba2_chunk_cumsum_bwd",
 )
 ALL_SYMBOLS = ENTRY_POINTS + ("bimamba2_strerror", "bimamba2_version", "bimamba2_params_size",
-                              "bimamba2_workspace_bytes")
+                              "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb")
 
 _lib = None
 
@@ -66,6 +66,8 @@ def load():
     lib.bimamba2_strerror.argtypes = [ctypes.c_int]
     lib.bimamba2_strerror.restype = ctypes.c_char_p
     lib.bimamba2_version.restype = ctypes.c_int
+    lib.bimamba2_chunk_scan_reads_cb.argtypes = [ctypes.POINTER(Params), ctypes.c_int]
+    lib.bimamba2_chunk_scan_reads_cb.restype = ctypes.c_int
     lib.bimamba2_params_size.restype = ctypes.c_size_t
     if lib.bimamba2_params_size() != ctypes.sizeof(Params):
         raise RuntimeError("bimamba2_params layout mismatch between the library and its Python mirror")

@@ -64,14 +64,14 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     need_f(q->dt_out, bhcq);
     need_f(q->cs_f, bhcq);
     need_f(q->cs_b, bhcq);
-    need_f(q->CB, cbn);
+    if (is_bwd || !scan_recomputes_cb(q, false)) need_f(q->CB, cbn);
     need_f(q->states_f, stn);
     need_f(q->states_b, stn);
     if (is_bwd) {
         const size_t nqt = (Q + 63) / 64;
         need_f(q->dCB, cbn * dcb_slices(q));
         need_f(q->dCBT, cbn * dcb_slices(q));
-        need_f(q->CBT, cbn);
+        if (!scan_recomputes_cb(q, true)) need_f(q->CBT, cbn);
         need_f(q->dstates_f, stn);
         need_f(q->dstates_b, stn);
         if (q->has_z && !q->dout_x)
@@ -119,6 +119,11 @@ size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd) {
     return carve(&q, is_bwd, nullptr);
 }
 
+int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int is_bwd) {
+    if (check_problem(p)) return 1;
+    return scan_recomputes_cb(p, is_bwd != 0) ? 0 : 1;
+}
+
 int bimamba2_chunk_cumsum_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->dt); REQUIRE(p->A); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
@@ -147,7 +152,8 @@ int bimamba2_state_passing_fwd(const bimamba2_params *p) {
 
 int bimamba2_chunk_scan_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->x); REQUIRE(p->Cm); REQUIRE(p->CB); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->x); REQUIRE(p->Cm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (!p->CB && !(p->Bm && scan_recomputes_cb(p, false))) return BIMAMBA2_EINVAL;   // without CB the kernel rebuilds it from Cm, Bm
     REQUIRE(p->states_f); REQUIRE(p->states_b); REQUIRE(p->out);
     if (p->has_D) REQUIRE(p->D);
     if (p->has_z) REQUIRE(p->z);
@@ -177,7 +183,8 @@ int bimamba2_state_passing_bwd(const bimamba2_params *p) {
 
 int bimamba2_chunk_scan_bwd_dx(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->CBT); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (!p->CBT && !(p->Cm && scan_recomputes_cb(p, true))) return BIMAMBA2_EINVAL;   // without CBT the kernel rebuilds it from Cm, Bm
     REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->dx); REQUIRE(p->ddt_direct);
     if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
     if (p->has_D) { REQUIRE(p->D); REQUIRE(p->dD); REQUIRE(p->red); }
@@ -235,9 +242,10 @@ int bimamba2_fwd(const bimamba2_params *p) {
     const size_t need = carve(&q, 0, p->workspace);
     if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
     TRY(bimamba2_chunk_cumsum_fwd(&q));
-    TRY(bimamba2_bmm_chunk_fwd(&q));
+    if (q.CB) TRY(bimamba2_bmm_chunk_fwd(&q));     // given by the caller, or carved because the scan kernel reads it
     TRY(bimamba2_chunk_state_fwd(&q));
     TRY(bimamba2_state_passing_fwd(&q));
+    if (scan_recomputes_cb(&q, false)) q.CB = nullptr;
     TRY(bimamba2_chunk_scan_fwd(&q));
     return BIMAMBA2_OK;
 }
@@ -249,19 +257,22 @@ int bimamba2_bwd(const bimamba2_params *p) {
     const size_t need = carve(&q, 1, p->workspace);
     if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
     if (p->fwd_saved) {
-        REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->CB); REQUIRE(p->CBT);
-        REQUIRE(p->states_f); REQUIRE(p->states_b);
+        REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
     } else {
         // recompute the forward intermediates (the reference does the same, src/ssd/bi/ssd_combined.py:373-380)
         TRY(bimamba2_chunk_cumsum_fwd(&q));
-        TRY(bimamba2_bmm_chunk_fwd(&q));
         TRY(bimamba2_chunk_state_fwd(&q));
         TRY(bimamba2_state_passing_fwd(&q));
     }
+    TRY(bimamba2_bmm_chunk_fwd(&q));               // CB for the dCB kernel, CB^T when the dx kernel reads it
     if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
     TRY(bimamba2_chunk_scan_bwd_dstates(&q));
     TRY(bimamba2_state_passing_bwd(&q));
-    TRY(bimamba2_chunk_scan_bwd_dx(&q));
+    {
+        bimamba2_params qx = q;
+        if (scan_recomputes_cb(&q, true)) qx.CBT = nullptr;
+        TRY(bimamba2_chunk_scan_bwd_dx(&qx));
+    }
     TRY(bimamba2_chunk_state_bwd_db(&q));
     TRY(bimamba2_chunk_scan_bwd_dc(&q));
     TRY(bimamba2_chunk_scan_bwd_dcb(&q));

@@ -22,6 +22,17 @@ __device__ __forceinline__ float to_f(bf16_t v) { return static_cast<float>(v); 
 __device__ __forceinline__ float to_f(f16_t v) { return static_cast<float>(v); }
 template <typename T> __device__ __forceinline__ T from_f(float v) { return static_cast<T>(v); }
 
+// ---- direct global -> LDS loads (global_load_lds): lane l's 16 bytes land at the wave-uniform LDS address + 16*l ----
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+typedef const __attribute__((address_space(1))) void *gbl_ptr_t;
+__device__ __forceinline__ void load16_to_lds(const void *src, void *lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)lds_wave_base, 16, 0, 0);
+}
+// at most N vector-memory operations of this wave outstanding; lgkmcnt / expcnt fields left at "no wait"
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
 // ---- LDS accesses issued from inline assembly ---------------------------------------------------------------
 // While a direct global->LDS load (global_load_lds) is in flight, the compiler makes every LDS access it knows of wait for
 // ALL outstanding vector memory operations, which defeats prefetching through LDS.  These accessors hide the DS

@@ -751,14 +751,6 @@ int dcb_slices(const bimamba2_params *p) {
 //    two-direction path;
 //  * the column sums over the four 16-lane groups come from one MFMA with a matrix of ones per column block.
 // ---------------------------------------------------------------------------------------------------------
-template <int N> __device__ __forceinline__ void wait_vmcnt() {
-    // at most N vector-memory operations of this wave outstanding; lgkmcnt / expcnt fields left at "no wait"
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
-typedef __attribute__((address_space(3))) void *lds_ptr_t;
-typedef const __attribute__((address_space(1))) void *gbl_ptr_t;
-
 // sum of v over the four lanes l%16, l%16+16, l%16+32, l%16+48, delivered to all of them: D = ones(16x4) * B where lane l
 // supplies B[k = l/16][n = l%16]
 __device__ __forceinline__ float lanegroup_sum_mfma(float v) {

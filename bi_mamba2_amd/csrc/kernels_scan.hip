@@ -31,7 +31,14 @@ constexpr int SCAN_WAVES = 8, SCAN_THREADS = 64 * SCAN_WAVES;
 // dstate % 64 == 0 and every operand is 16-byte aligned with strides that keep rows aligned: all guarded scalar
 // fallbacks compile away and loads become unconditional (rows past the end of the sequence are read from a valid
 // row and never stored).
-template <typename T, int QT, int NJ, bool BWD, bool FAST>
+//
+// NF > 0 (16-bit types, FAST, dstate = 32 * NF): CB is not read at all.  The 16 x 32 piece of CB (resp. CB^T) a wave needs
+// for a K step is recomputed with MFMAs from the C and B rows, arranged so that the product comes out in the A operand
+// layout: D[m][n] = sum_d Krow[k(m)][d] * Ownrow[n][d] with k(m) = k0 + 8*(m/4) + m%4 (+4 for the second product) leaves
+// lane (l%16 = row, l/16 = g) with columns k0 + 8g + 0..3 (resp. +4..7) of its row.  All waves of a workgroup read the
+// same 32 K rows per step, so they come from L1, where the CB rows were 256 KB of L2 traffic per workgroup.  The state
+// products use the raw rows as well and scale the accumulator instead of the operand.
+template <typename T, int QT, int NJ, bool BWD, bool FAST, int NF>
 __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimamba2_params p, int nc, int npt) {
     typedef Mma<T> M;
     constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
@@ -47,10 +54,11 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     // the operand images (xT and the two state tiles) and the per-wave epilogue staging patches are never live together
     __shared__ __attribute__((aligned(16))) char shared_u[XT_BYTES + ST_BYTES > STG_BYTES ? XT_BYTES + ST_BYTES : STG_BYTES];
     __shared__ float lo[QP], up[QP];              // decay exponents (times log2 e), see below
+    __shared__ float glo[QP], gup[QP];            // their column factors relative to the edge of the 16-block, see below
     __shared__ float red[SCAN_WAVES][PW];
     T *xT = reinterpret_cast<T *>(shared_u);
     T *sF = reinterpret_cast<T *>(shared_u + XT_BYTES), *sB = sF + PW * LDS_;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lr = lane & 15, lg = lane >> 4;
     // linear block id -> (pt, h, bc) with bc fastest: all heads of one (batch, chunk) share CB and C, and
     // consecutive ids are dealt round-robin to the 8 XCDs, so equal bc % 8 keeps them on one XCD's L2
@@ -71,6 +79,37 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
 #define TSTAMP(i)
 #endif
     TSTAMP(0)
+    // NF > 0: the K rows of part 2 (forward: B rows, mirror: C rows) travel straight into a ring of LDS slots, KRING - 1
+    // K steps (of 32 rows) ahead of their use: a global access takes microseconds when the memory system is busy.  Wave w brings rows 4w..4w+3 of the step: unit u = 32*w + lane (lane < 32) is row
+    // u/8, chunk position u%8, which holds the row's 16-byte chunk (u%8) ^ (row % 8).
+    constexpr int KRING = 4;                       // slots of the K-row image: requests run KRING - 1 steps ahead
+    __shared__ __attribute__((aligned(16))) T krl[NF > 0 ? KRING * 32 * 64 : 8];
+    const char *krbase = nullptr;                  // uniform: row 0 of the chunk in the K-row matrix
+    unsigned krs_bytes = 0;                        // its row stride (the launcher checks that 256 rows fit 32 bits)
+    if constexpr (NF > 0) {
+        if (BWD) { krs_bytes = (unsigned)p.C_sl * sizeof(T); krbase = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * p.C_sl + g * p.C_sg); }
+        else { krs_bytes = (unsigned)p.B_sl * sizeof(T); krbase = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * p.B_sl + g * p.B_sg); }
+    }
+    if constexpr (NF > 0) {
+        // keep the base in scalar registers (it is uniform, but that is not visible through the 64-bit arithmetic)
+        const uint64_t kb64 = reinterpret_cast<uint64_t>(krbase);
+        const uint32_t klo = __builtin_amdgcn_readfirstlane((uint32_t)kb64), khi = __builtin_amdgcn_readfirstlane((uint32_t)(kb64 >> 32));
+        krbase = reinterpret_cast<const char *>(((uint64_t)khi << 32) | klo);
+    }
+    auto kr_issue = [&](int step) {
+        if (lane < 32) {
+            int ln = lane;
+            asm volatile("" : "+v"(ln));           // recompute the few lane terms per call rather than keep them in registers
+            const int rowl = wave * 4 + (ln >> 3);
+            const unsigned off = (unsigned)min(step * 32 + rowl, limit - 1) * krs_bytes + (((ln & 7) ^ (rowl & 7)) * 16);
+            load16_to_lds(krbase + off, krl + (step % KRING) * (32 * 64) + wave * 256);
+        }
+    };
+    if constexpr (NF > 0) {
+#pragma unroll
+        for (int st = 0; st < KRING - 1; ++st)
+            if (st * 32 < limit) kr_issue(st);
+    }
     int rowi[QT];                                  // this lane's A-operand row in each row tile
 #pragma unroll
     for (int rt = 0; rt < QT; ++rt) rowi[rt] = (wave * QT + rt) * 16 + lr;
@@ -103,11 +142,17 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
 
     // forward: k<r uses lo[r]-lo[k] with lo = cs_f, k>r uses up[r]-up[k] with up = cs_b
     // mirror : k<r uses e^{cs_b[k]-cs_b[r]} -> lo = -cs_b;  k>r uses e^{cs_f[k]-cs_f[r]} -> up = -cs_f
+    // Away from the diagonal the factor separates: with m = lo at the last position of k's block of 16 (which lies
+    // between k and r), 2^{lo[r]-lo[k]} = 2^{lo[r]-m} * glo[k], glo[k] = 2^{m-lo[k]}, both factors <= 1 for A <= 0;
+    // likewise gup[k] = 2^{up[first of k's block] - up[k]}.  One exponential per lane and K step instead of one per element.
     for (int q = threadIdx.x; q < QP; q += SCAN_THREADS) {
-        const int qq = min(q, Q - 1);
+        const int qq = min(q, Q - 1), qe = min(q | 15, Q - 1), qs = min(q & ~15, Q - 1);
         const float f = csf[qq] * LOG2E, r = csb[qq] * LOG2E;
-        lo[q] = BWD ? -r : f;
-        up[q] = BWD ? -f : r;
+        const float l = BWD ? -r : f, u = BWD ? -f : r;
+        lo[q] = l;
+        up[q] = u;
+        glo[q] = __builtin_amdgcn_exp2f((BWD ? -csb[qe] : csf[qe]) * LOG2E - l);
+        gup[q] = __builtin_amdgcn_exp2f((BWD ? -csf[qs] : csb[qs]) * LOG2E - u);
     }
     // K operand of part 2, transposed into LDS
     const T *kp;
@@ -118,7 +163,15 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     if (BWD) stage_transposed<T, QP, PW, LDX, FAST>(xT, kp + p0, ks, limit, P - p0, [&](int k) { return k < limit ? 1.f : 0.f; });
     else stage_transposed<T, QP, PW, LDX, FAST>(xT, kp + p0, ks, limit, P - p0, [&](int k) { return k < limit ? dto[k] : 0.f; });
 
-    load_arows(0);
+    typename M::Frag own[QT][NF > 0 ? NF : 1];     // NF > 0: this lane's rows, 32 dstate columns per fragment
+    if constexpr (NF > 0) {
+#pragma unroll
+        for (int rt = 0; rt < QT; ++rt)
+#pragma unroll
+            for (int f = 0; f < NF; ++f) own[rt][f] = M::load(ap + (int64_t)min(rowi[rt], limit - 1) * as + f * KSTEP + lg * KPL);
+    } else {
+        load_arows(0);
+    }
     f32x4 acc[QT][NJ] = {};
     TSTAMP(1)
 
@@ -138,6 +191,41 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             rsf[rt] = ef;
             rsb[rt] = eb;
         }
+        if constexpr (NF > 0) {
+            // raw rows as the A operand; the row factors go onto the accumulators (rows 4*(l/16)+i of each tile).
+            // One direction after the other, to keep one set of temporaries.
+            static_assert(NF == 0 || NF * KSTEP == NW, "one round of state tiles");
+            tile_load_kcontig<T, float, PW, NW>(sF, stf, N, P - p0, N, Ident());
+            tile_load_kcontig<T, float, PW, NW>(sB, stb, N, P - p0, N, Ident());
+            __syncthreads();
+            TSTAMP(2)
+#pragma unroll
+            for (int dir = 0; dir < 2; ++dir) {
+                const T *st = dir ? sB : sF;
+                f32x4 tmp[QT][NJ] = {};
+#pragma unroll
+                for (int s = 0; s < NW / KSTEP; ++s) {
+                    typename M::Frag bfs[NJ];
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) bfs[j] = M::load(st + (j * 16 + lr) * LDS_ + s * KSTEP + lg * KPL);
+#pragma unroll
+                    for (int rt = 0; rt < QT; ++rt)
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) tmp[rt][j] = M::mma(own[rt][s], bfs[j], tmp[rt][j]);
+                }
+#pragma unroll
+                for (int rt = 0; rt < QT; ++rt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int r = (wave * QT + rt) * 16 + lg * 4 + i, rc = min(r, limit - 1);
+                        const float *cs = dir ? csb : csf;
+                        float e = BWD ? __expf(cs[dir ? 0 : Q - 1] - cs[rc]) : __expf(cs[rc]);
+                        if (r >= limit) e = 0.f;
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) acc[rt][j][i] = dir ? __builtin_fmaf(tmp[rt][j][i], e, acc[rt][j][i]) : tmp[rt][j][i] * e;
+                    }
+            }
+        } else
         for (int n0 = 0; n0 < N; n0 += NW) {
             if (n0) {
                 __syncthreads();
@@ -184,15 +272,13 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     const bool xvec = aligned16(xrow + p0, p.x_sl) && (P % VS == 0);
     const bool vec2 = need2 && aligned16(row2 + p0, s2) && (P % VS == 0);
     const bool ovec = (P % VS == 0);
-    float ex[1][NPASS][VS], e2[1][NPASS][VS];
-    auto load_vec = [&](const T *ptr, bool vec, int ncol, float (&v)[VS]) {
+    Vec16<T> ex[QT][NPASS], e2[QT][NPASS];         // kept as loaded; converted where they are used
+    auto load_vec = [&](const T *ptr, bool vec, int ncol, Vec16<T> &v) {
         if (FAST || (vec && ncol >= VS)) {
-            Vec16<T> raw = *reinterpret_cast<const Vec16<T> *>(ptr);
-#pragma unroll
-            for (int i = 0; i < VS; ++i) v[i] = to_f(raw.v[i]);
+            v = *reinterpret_cast<const Vec16<T> *>(ptr);
         } else {
 #pragma unroll
-            for (int i = 0; i < VS; ++i) v[i] = i < ncol ? to_f(ptr[i]) : 0.f;
+            for (int i = 0; i < VS; ++i) v.v[i] = i < ncol ? ptr[i] : from_f<T>(0.f);
         }
     };
     auto store_vec = [&](T *ptr, bool vec, int ncol, const float (&v)[VS]) {
@@ -207,8 +293,8 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                 if (i < ncol) ptr[i] = from_f<T>(v[i]);
         }
     };
-    auto epi_issue = [&](auto BUF, int rt) {
-        constexpr int B_ = decltype(BUF)::value;
+    auto epi_issue = [&](int rt) {
+        const int B_ = rt;
         const int r0 = (wave * QT + rt) * 16;
 #pragma unroll
         for (int ps = 0; ps < NPASS; ++ps) {
@@ -268,24 +354,24 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             typename M::Frag bf[NJ];
 #pragma unroll
             for (int j = 0; j < NJ; ++j) bf[j] = M::load(xT + xt_index<T, LDX>(j * 16 + lr, kb));
-            float lok[KPL], upk[KPL];
-#pragma unroll
-            for (int i = 0; i < KPL; ++i) { lok[i] = lo[kb + i]; upk[i] = up[kb + i]; }
+            // this lane's KPL columns lie in one block of 16
 #pragma unroll
             for (int rt = 0; rt < QT; ++rt) {
                 const int r = rowi[rt], r0 = (wave * QT + rt) * 16;
                 float v[KPL];
                 if (k0 + KSTEP - 1 < r0) {            // every k of this step is below every row of the tile
+                    const float rf = __builtin_amdgcn_exp2f(lor[rt] - lo[kb | 15]);
 #pragma unroll
-                    for (int i = 0; i < KPL; ++i) v[i] = cbv[B_][rt][i] * __builtin_amdgcn_exp2f(lor[rt] - lok[i]);
+                    for (int i = 0; i < KPL; ++i) v[i] = cbv[B_][rt][i] * rf * glo[kb + i];
                 } else if (k0 > r0 + 15) {            // every k above every row
+                    const float rf = __builtin_amdgcn_exp2f(upr[rt] - up[kb & ~15]);
 #pragma unroll
-                    for (int i = 0; i < KPL; ++i) v[i] = cbv[B_][rt][i] * __builtin_amdgcn_exp2f(upr[rt] - upk[i]);
+                    for (int i = 0; i < KPL; ++i) v[i] = cbv[B_][rt][i] * rf * gup[kb + i];
                 } else {
 #pragma unroll
                     for (int i = 0; i < KPL; ++i) {
                         const int k = kb + i;
-                        const float e = k < r ? lor[rt] - lok[i] : upr[rt] - upk[i];
+                        const float e = k < r ? lor[rt] - lo[k] : upr[rt] - up[k];
                         v[i] = cbv[B_][rt][i] * ((k == r) ? 2.f : __builtin_amdgcn_exp2f(e));
                     }
                 }
@@ -294,15 +380,127 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                 for (int j = 0; j < NJ; ++j) acc[rt][j] = M::mma(af, bf[j], acc[rt][j]);
             }
         };
-        for (int k0 = 0; k0 < limit; k0 += KSTEP) {
-            issue(B0(), k0);
-            process(B0(), k0);
+        if constexpr (NF > 0) {
+            static_assert(NF == 0 || (NF == 2 && KPL == 8 && KSTEP == 32), "K-row image: 32 rows of 64 elements per step");
+            // fragment (hh, f): K row krow + 4*hh of the step, 16-byte chunk lg + 4*f, stored at chunk ^ (row % 8); with
+            // krow % 8 = lr % 4 that is element kfb + 256*hh + 32*(f ^ hh) of the slot
+            const int kfb = (8 * (lr >> 2) + (lr & 3)) * 64 + (lg ^ (lr & 3)) * 8;
+            // x^T fragment j of step s (xt_index(16j + lr, 32s + 8lg)): lane part by the parity of j, the rest is uniform
+            static_assert(NF == 0 || NJ == 4, "fragment addresses below are written out for four column tiles");
+            const int xl0 = lr * LDX + 8 * (lg ^ (lr >> 3)), xl1 = lr * LDX + 8 * (lg ^ ((lr >> 3) + 2));
+            // While requests are in flight every LDS access goes through the raw accessors (the compiler would make an
+            // access it knows of wait for all of them), and the barrier is the bare instruction.
+            const unsigned krl_a = lds_addr(krl) + kfb * 2, xt_a = lds_addr(xT);
+            const unsigned lg32 = lg * 32;             // this lane's 8 columns inside a step of the float tables
+            const int nsteps = (limit + KSTEP - 1) / KSTEP;
+            typedef typename M::Frag Frag;
+            for (int step = 0; step < nsteps; ++step) {
+                const int k0 = step * KSTEP;
+                // this wave's request for the step has landed: one request per step, up to KRING - 2 newer ones
+                const int newer = min(KRING - 2, nsteps - 1 - step);
+                if (newer >= 2) wait_vmcnt<2>();
+                else if (newer == 1) wait_vmcnt<1>();
+                else wait_vmcnt<0>();
+                raw_lds_barrier();                     // ... and everybody else's; the slot of step - 1 is free again
+                if (step + KRING - 1 < nsteps) kr_issue(step + KRING - 1);
+                const unsigned slot = krl_a + (step % KRING) * (32 * 64 * 2);
+                // the CB tiles of both row tiles first; the K fragments are dead after that
+                f32x4 cb1[QT], cb2[QT];
+                {
+                    Frag kf00 = raw_lds_read_at<Frag, 0>(slot), kf01 = raw_lds_read_at<Frag, 64>(slot);
+                    Frag kf10 = raw_lds_read_at<Frag, 512 + 64>(slot), kf11 = raw_lds_read_at<Frag, 512>(slot);
+                    raw_lds_wait();
+                    raw_lds_use(kf00); raw_lds_use(kf01); raw_lds_use(kf10); raw_lds_use(kf11);
+#pragma unroll
+                    for (int rt = 0; rt < QT; ++rt) {
+                        cb1[rt] = M::mma(kf00, own[rt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                        cb2[rt] = M::mma(kf10, own[rt][0], f32x4{0.f, 0.f, 0.f, 0.f});
+                        cb1[rt] = M::mma(kf01, own[rt][1], cb1[rt]);
+                        cb2[rt] = M::mma(kf11, own[rt][1], cb2[rt]);
+                    }
+                }
+                // the wave's rows [wr0, wr0 + 16*QT) meet the step's columns [k0, k0 + 32) in one step only
+                const int wr0 = wave * QT * 16;
+                const int cls = (k0 + KSTEP - 1 < wr0) ? 0 : (k0 > wr0 + QT * 16 - 1) ? 1 : 2;   // below, above, across the diagonal
+                const int kb = k0 + lg * KPL;
+                // ---- A operands of both row tiles: CB times the decay factors
+                Frag af[QT];
+                if (cls != 2) {
+                    const unsigned ta = lds_addr(cls == 0 ? glo : gup) + k0 * 4 + lg32;
+                    f32x4 ga0 = raw_lds_read_at<f32x4, 0>(ta), ga1 = raw_lds_read_at<f32x4, 16>(ta);
+                    float mref = raw_lds_read_at<float, 0>(cls == 0 ? lds_addr(lo) + (kb | 15) * 4 : lds_addr(up) + (kb & ~15) * 4);
+                    raw_lds_wait();
+                    raw_lds_use(ga0); raw_lds_use(ga1); raw_lds_use(mref);
+#pragma unroll
+                    for (int rt = 0; rt < QT; ++rt) {
+                        const float rf = __builtin_amdgcn_exp2f((cls == 0 ? lor[rt] : upr[rt]) - mref);
+                        float v[KPL];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { v[i] = cb1[rt][i] * rf * ga0[i]; v[i + 4] = cb2[rt][i] * rf * ga1[i]; }
+                        af[rt] = M::pack(v);
+                    }
+                } else {
+                    // the one step across the diagonal: element by element
+                    const unsigned la = lds_addr(lo) + k0 * 4 + lg32, ua = lds_addr(up) + k0 * 4 + lg32;
+                    f32x4 l0 = raw_lds_read_at<f32x4, 0>(la), l1 = raw_lds_read_at<f32x4, 16>(la);
+                    f32x4 u0 = raw_lds_read_at<f32x4, 0>(ua), u1 = raw_lds_read_at<f32x4, 16>(ua);
+                    raw_lds_wait();
+                    raw_lds_use(l0); raw_lds_use(l1); raw_lds_use(u0); raw_lds_use(u1);
+#pragma unroll
+                    for (int rt = 0; rt < QT; ++rt) {
+                        const int r = (wave * QT + rt) * 16 + lr;
+                        float v[KPL];
+#pragma unroll
+                        for (int i = 0; i < KPL; ++i) {
+                            const int k = kb + i;
+                            const float lk = i < 4 ? l0[i & 3] : l1[i & 3], uk = i < 4 ? u0[i & 3] : u1[i & 3];
+                            const float e = k < r ? lor[rt] - lk : upr[rt] - uk;
+                            v[i] = (i < 4 ? cb1[rt][i & 3] : cb2[rt][i & 3]) * ((k == r) ? 2.f : __builtin_amdgcn_exp2f(e));
+                        }
+                        af[rt] = M::pack(v);
+                    }
+                }
+                // ---- the x product, two column tiles at a time
+                const unsigned xa = xt_a + 64 * step, xb = xt_a + 64 * (step ^ 1);
+                {
+                    Frag b0 = raw_lds_read_at<Frag, 0>(xa + 2 * xl0), b1 = raw_lds_read_at<Frag, 32 * LDX>(xa + 2 * xl1);
+                    raw_lds_wait();
+                    raw_lds_use(b0); raw_lds_use(b1);
+#pragma unroll
+                    for (int rt = 0; rt < QT; ++rt) {
+                        acc[rt][0] = M::mma(af[rt], b0, acc[rt][0]);
+                        acc[rt][1] = M::mma(af[rt], b1, acc[rt][1]);
+                    }
+                }
+                {
+                    Frag b2 = raw_lds_read_at<Frag, 64 * LDX>(xb + 2 * xl0), b3 = raw_lds_read_at<Frag, 96 * LDX>(xb + 2 * xl1);
+                    raw_lds_wait();
+                    raw_lds_use(b2); raw_lds_use(b3);
+#pragma unroll
+                    for (int rt = 0; rt < QT; ++rt) {
+                        acc[rt][2] = M::mma(af[rt], b2, acc[rt][2]);
+                        acc[rt][3] = M::mma(af[rt], b3, acc[rt][3]);
+                    }
+                }
+            }
+            wait_vmcnt<0>();
+            __syncthreads();
+        } else {
+            for (int k0 = 0; k0 < limit; k0 += KSTEP) {
+                issue(B0(), k0);
+                process(B0(), k0);
+            }
         }
     }
 #endif
 
     // ---- epilogue.  Each wave passes its 16-row accumulator tiles through a private LDS patch so that out, out_x,
     // dx are written (and x, z, dy were read) as 16-byte vectors along headdim ----
+    // the epilogue operands of all row tiles are requested before the barrier
+#pragma unroll
+    for (int rt = 0; rt < QT; ++rt) {
+        if ((wave * QT + rt) * 16 < limit) epi_issue(rt);
+    }
     TSTAMP(4)
     __syncthreads();   // every wave is done with xT: the operand images become the staging area
     TSTAMP(5)
@@ -310,8 +508,8 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     float dsum[VS];
 #pragma unroll
     for (int i = 0; i < VS; ++i) dsum[i] = 0.f;
-    auto epi_consume = [&](auto BUF, int rt) {
-        constexpr int B_ = decltype(BUF)::value;
+    auto epi_consume = [&](int rt) {
+        const int B_ = rt;
         const int r0 = (wave * QT + rt) * 16;
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
@@ -339,24 +537,24 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                     if (p.has_D) {
 #pragma unroll
                         for (int i = 0; i < VS; ++i)
-                            a[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : p.D[h]) * ex[B_][ps][i];
+                            a[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : p.D[h]) * to_f(ex[B_][ps].v[i]);
                     }
                     if (p.has_z) {
                         if (p.out_x) store_vec(reinterpret_cast<T *>(p.out_x) + orow, ovec, ncol, a);
 #pragma unroll
-                        for (int i = 0; i < VS; ++i) a[i] *= silu_f(e2[B_][ps][i]);
+                        for (int i = 0; i < VS; ++i) a[i] *= silu_f(to_f(e2[B_][ps].v[i]));
                     }
                     store_vec(reinterpret_cast<T *>(p.out) + orow, ovec, ncol, a);
                 } else {
                     const float dtr = dto[r];
                     float dxv[VS];
 #pragma unroll
-                    for (int i = 0; i < VS; ++i) { rsum += a[i] * ex[B_][ps][i]; dxv[i] = a[i] * dtr; }
+                    for (int i = 0; i < VS; ++i) { rsum += a[i] * to_f(ex[B_][ps].v[i]); dxv[i] = a[i] * dtr; }
                     if (p.has_D) {
 #pragma unroll
                         for (int i = 0; i < VS; ++i) {
-                            dxv[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : p.D[h]) * e2[B_][ps][i];
-                            dsum[i] += e2[B_][ps][i] * ex[B_][ps][i];
+                            dxv[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : p.D[h]) * to_f(e2[B_][ps].v[i]);
+                            dsum[i] += to_f(e2[B_][ps].v[i]) * to_f(ex[B_][ps].v[i]);
                         }
                     }
                     store_vec(reinterpret_cast<T *>(p.dx) + orow, ovec, ncol, dxv);
@@ -377,10 +575,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     };
 #pragma unroll
     for (int rt = 0; rt < QT; ++rt) {
-        if ((wave * QT + rt) * 16 < limit) {
-            epi_issue(B0(), rt);
-            epi_consume(B0(), rt);
-        }
+        if ((wave * QT + rt) * 16 < limit) epi_consume(rt);
     }
     TSTAMP(6)
     if (BWD && p.has_D) {
@@ -408,31 +603,57 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
 
 static inline bool al16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
-template <typename T, int NJMAX, bool BWD>
-static int launch_scan_t(const bimamba2_params *p) {
-    const int nc = nchunks(p);
-    const int P = p->headdim, Q = p->chunk_size, N = p->dstate;
-    constexpr int VS = 16 / (int)sizeof(T);
+static inline int scan_col_tile(const bimamba2_params *p) {
     // headdim tile: the widest the LDS image allows (64 columns for 16-bit types, 32 for float32)
-    const int pw = P <= 16 ? 16 : (P <= 32 || NJMAX == 2) ? 32 : 64;
-    const int npt = (P + pw - 1) / pw;
-    dim3 grid(p->batch * nc * p->nheads * npt);
-    hipStream_t s = reinterpret_cast<hipStream_t>(p->stream);
-    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % VS == 0 && b % VS == 0 && c % VS == 0; };
-    bool fast = Q % 32 == 0 && P % pw == 0 && N % 64 == 0 && al16(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
-    if (BWD) {
+    const int njmax = p->dtype == BIMAMBA2_F32 ? 2 : 4;
+    return p->headdim <= 16 ? 16 : (p->headdim <= 32 || njmax == 2) ? 32 : 64;
+}
+
+// whether the kernels without guarded fallbacks apply (vs = elements per 16 bytes)
+static bool scan_fast(const bimamba2_params *p, bool bwd, int pw, int vs) {
+    auto mult = [vs](int64_t a, int64_t b, int64_t c) { return a % vs == 0 && b % vs == 0 && c % vs == 0; };
+    bool fast = p->chunk_size % 32 == 0 && p->headdim % pw == 0 && p->dstate % 64 == 0 && al16(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
+    if (bwd) {
         fast = fast && al16(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al16(p->dx);
         fast = fast && (p->has_z ? al16(p->dout_x) : (al16(p->dout) && mult(p->dout_sb, p->dout_sl, p->dout_sh)));
     } else {
         fast = fast && al16(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg) && al16(p->out);
         if (p->has_z) fast = fast && al16(p->z) && mult(p->z_sb, p->z_sl, p->z_sh) && (!p->out_x || al16(p->out_x));
     }
-#define BM2_SCAN(QTV, NJV)                                                                                                     \
-    do {                                                                                                                       \
-        if (fast) hipLaunchKernelGGL((chunk_scan_kernel<T, QTV, NJV, BWD, true>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt); \
-        else hipLaunchKernelGGL((chunk_scan_kernel<T, QTV, NJV, BWD, false>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);     \
+    return fast;
+}
+
+bool scan_recomputes_cb(const bimamba2_params *p, bool bwd) {
+    if (p->dtype == BIMAMBA2_F32 || p->dstate != 64 || scan_col_tile(p) != 64) return false;
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
+    if (p->B_sl <= 0 || p->C_sl <= 0 || p->B_sl > (1 << 21) || p->C_sl > (1 << 21)) return false;   // 256 rows in 32-bit byte offsets
+    return scan_fast(p, bwd, 64, 8) && al16(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al16(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg);
+}
+
+template <typename T, int NJMAX, bool BWD>
+static int launch_scan_t(const bimamba2_params *p) {
+    const int nc = nchunks(p);
+    const int P = p->headdim, Q = p->chunk_size, N = p->dstate;
+    constexpr int VS = 16 / (int)sizeof(T);
+    const int pw = scan_col_tile(p);
+    const int npt = (P + pw - 1) / pw;
+    dim3 grid(p->batch * nc * p->nheads * npt);
+    hipStream_t s = reinterpret_cast<hipStream_t>(p->stream);
+    const bool fast = scan_fast(p, BWD, pw, VS);
+#define BM2_SCAN(QTV, NJV)                                                                                                        \
+    do {                                                                                                                          \
+        if (fast) hipLaunchKernelGGL((chunk_scan_kernel<T, QTV, NJV, BWD, true, 0>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt); \
+        else hipLaunchKernelGGL((chunk_scan_kernel<T, QTV, NJV, BWD, false, 0>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);     \
     } while (0)
     const int qt = Q <= 128 ? 1 : 2;             // 16-row tiles per wave (8 waves)
+    if constexpr (sizeof(T) == 2 && NJMAX == 4) {
+        if ((BWD ? p->CBT : p->CB) == nullptr) {        // the caller checked scan_recomputes_cb()
+            if (qt == 1) hipLaunchKernelGGL((chunk_scan_kernel<T, 1, 4, BWD, true, 2>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
+            else hipLaunchKernelGGL((chunk_scan_kernel<T, 2, 4, BWD, true, 2>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
+            return check_launch();
+        }
+    }
+    if ((BWD ? p->CBT : p->CB) == nullptr) return BIMAMBA2_EINVAL;
     if (pw == 16) { if (qt == 1) BM2_SCAN(1, 1); else BM2_SCAN(2, 1); }
     else if (pw == 32) { if (qt == 1) BM2_SCAN(1, 2); else BM2_SCAN(2, 2); }
     else { if (qt == 1) BM2_SCAN(1, NJMAX); else BM2_SCAN(2, NJMAX); }

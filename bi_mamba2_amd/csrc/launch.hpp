@@ -13,6 +13,8 @@ int launch_bmm_chunk_fwd(const bimamba2_params *p);
 int launch_chunk_state(const bimamba2_params *p, bool dstates);
 int launch_state_passing_fwd(const bimamba2_params *p);
 int launch_chunk_scan(const bimamba2_params *p, bool bwd);
+// true when that launch recomputes CB (bwd: CB^T) from the C and B rows instead of reading it
+bool scan_recomputes_cb(const bimamba2_params *p, bool bwd);
 
 int launch_bwd_dz(const bimamba2_params *p);
 int launch_state_passing_bwd(const bimamba2_params *p);

@@ -410,7 +410,7 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
     like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
     out, out_x and the final states are materialised as tensors (the rest lives in a workspace).
-    keep_for_bwd=True appends a tenth element: the tuple (dt_out, cs_f, cs_b, CB, CBT, states_f, states_b) that
+    keep_for_bwd=True appends a tenth element: the tuple (dt_out, cs_f, cs_b, states_f, states_b) that
     _mamba_chunk_scan_combined_bwd accepts as `saved` to skip its recomputation."""
     c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
     batch, seqlen, nheads, headdim = x.shape
@@ -425,8 +425,7 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
         sshape = (batch, c.nchunks, nheads, headdim, dstate)
         sf = c.new("states_f", sshape); sb = c.new("states_b", sshape)
     if keep_for_bwd:
-        cbshape = (batch, c.nchunks, ngroups, chunk_size, chunk_size)
-        saved = (dt_out, cs_f, cs_b, c.new("CB", cbshape), c.new("CBT", cbshape), sf, sb)
+        saved = (dt_out, cs_f, cs_b, sf, sb)
     c.workspace(False)
     c.run("bimamba2_fwd")
     res = (out, out_x, dt_out, cs_f, cs_b, sf, sb, ff, fb)
@@ -446,7 +445,7 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     batch, seqlen, nheads, headdim = x.shape
     c.set_dout(dout)
     if saved is not None:
-        for name, t in zip(("dt_out", "cs_f", "cs_b", "CB", "CBT", "states_f", "states_b"), saved):
+        for name, t in zip(("dt_out", "cs_f", "cs_b", "states_f", "states_b"), saved):
             c.put(name, t, torch.float32)
         c.p.fwd_saved = 1
     if z is not None:

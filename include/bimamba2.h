@@ -54,8 +54,8 @@ typedef struct bimamba2_params {
     int32_t dtype;          /* BIMAMBA2_* : x, z, Bm, Cm, out, out_x, dout and their gradients */
     int32_t dt_dtype;       /* BIMAMBA2_* : dt and ddt */
     int32_t has_D, D_has_hdim, has_z, has_dt_bias, dt_softplus;
-    int32_t fwd_saved;      /* bimamba2_bwd only: dt_out, cs_f, cs_b, CB, CBT, states_f, states_b hold what bimamba2_fwd
-                               left in them, so the backward pass does not recompute them */
+    int32_t fwd_saved;      /* bimamba2_bwd only: dt_out, cs_f, cs_b, states_f, states_b hold what bimamba2_fwd left in
+                               them, so the backward pass does not recompute them (CB is always recomputed) */
     int32_t reserved0;
     float dt_min, dt_max;
     /* element strides of the strided inputs (last dim contiguous) */
@@ -103,16 +103,24 @@ size_t bimamba2_params_size(void);
 /* bytes of workspace the composite entry points need (is_bwd = 0: forward, 1: backward) */
 size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd);
 
+/* 0 when the chunk-scan launch of this problem recomputes the CB tiles it needs from the C and B rows inside the
+ * kernel (16-bit dtype, dstate 64, headdim a multiple of 64, chunk_size a multiple of 32, 16-byte aligned
+ * operands), 1 when it reads them: CB for bimamba2_chunk_scan_fwd (is_bwd = 0), CBT for bimamba2_chunk_scan_bwd_dx
+ * (is_bwd = 1).  When it is 0 a caller of the single stages may pass that pointer as NULL (and skip the CBT buffer).
+ * Fuses _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208) into the scan for those shapes. */
+int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int is_bwd);
+
 /* Whole forward; replaces _mamba_chunk_scan_combined_fwd (src/ssd/bi/ssd_combined.py:297-331).
  * Needs: x dt A Bm Cm [D z dt_bias] out [out_x when has_z] [final_f final_b] workspace.  Intermediates given as
  * non-NULL pointers (dt_out cs_f cs_b CB CBT states_f states_b) are filled in place of workspace memory, so a
- * caller can keep them for the backward pass. */
+ * caller can keep them for the backward pass (CB and CBT are only computed when given or when the scan kernel
+ * reads them). */
 int bimamba2_fwd(const bimamba2_params *p);
 
 /* Whole backward; replaces _mamba_chunk_scan_combined_bwd (src/ssd/bi/ssd_combined.py:334-475).
  * Needs: the forward inputs, dout, out_x (pre-gate output, when has_z), dx ddt dA dB dC [dD dz ddt_bias],
  * workspace.  With fwd_saved = 0 it recomputes the forward intermediates as the reference does; with
- * fwd_saved = 1 it reads them from the seven pointers named at that flag. */
+ * fwd_saved = 1 it reads them from the five pointers named at that flag. */
 int bimamba2_bwd(const bimamba2_params *p);
 
 /* ---- single stages (each is also what the composites run) ------------------------------------------ */
@@ -128,8 +136,9 @@ int bimamba2_chunk_state_fwd(const bimamba2_params *p);
  * launch; optional final_f/final_b.  Replaces the two _state_passing_fwd calls
  * (src/ssd/bi/ssd_state_passing.py:190-207; src/ssd/bi/ssd_combined.py:324-327). */
 int bimamba2_state_passing_fwd(const bimamba2_params *p);
-/* CB, x, z, dt_out, cs_f, cs_b, Cm, states_f/b, D -> out, out_x.  Replaces _chunk_scan_fwd
- * (src/ssd/bi/ssd_chunk_scan.py:1638-1686). */
+/* CB, x, z, dt_out, cs_f, cs_b, Cm, Bm, states_f/b, D -> out, out_x.  Replaces _chunk_scan_fwd
+ * (src/ssd/bi/ssd_chunk_scan.py:1638-1686).  With CB = NULL, allowed when bimamba2_chunk_scan_reads_cb(p, 0) is 0,
+ * the kernel rebuilds the CB tiles from Cm and Bm; a CB that is given is read. */
 int bimamba2_chunk_scan_fwd(const bimamba2_params *p);
 
 /* z, out_x, dout -> dz, dout_x.  Replaces _chunk_scan_bwd_dz (src/ssd/bi/ssd_chunk_scan.py:1741-1798);
@@ -142,7 +151,8 @@ int bimamba2_chunk_scan_bwd_dstates(const bimamba2_params *p);
  * Replaces the two _state_passing_bwd calls (src/ssd/bi/ssd_state_passing.py:210-248). */
 int bimamba2_state_passing_bwd(const bimamba2_params *p);
 /* -> dx, ddt_direct, dD partials (reduced into dD).  Replaces _chunk_scan_chunk_state_bwd_dx
- * (src/ssd/bi/ssd_combined.py:235-294). */
+ * (src/ssd/bi/ssd_combined.py:235-294).  With CBT = NULL, allowed when bimamba2_chunk_scan_reads_cb(p, 1) is 0,
+ * the kernel rebuilds the tiles from Cm and Bm; a CBT that is given is read. */
 int bimamba2_chunk_scan_bwd_dx(const bimamba2_params *p);
 /* x, dstates_f/b, dt_out, cs, Bm -> dBs, v_f, v_b.  Replaces _chunk_state_bwd_db
  * (src/ssd/bi/ssd_chunk_state.py:836-894); v_* are its ddA_next terms before the scan. */
