@@ -64,6 +64,10 @@ E2E = [
     (2, 512, 8, 64, 1, 64, 256, torch.bfloat16, True, "h", True, True, (0.0, INF)),
     (1, 700, 4, 64, 2, 128, 256, torch.bfloat16, False, "h", True, True, (0.0, INF)),
     (2, 256, 4, 64, 4, 64, 128, torch.float16, True, "h", True, True, (0.0, INF)),
+    # shapes whose scan kernels rebuild CB themselves, with a ragged last chunk (44 valid rows), grouped heads,
+    # resp. two headdim tiles
+    (2, 300, 4, 64, 2, 64, 256, torch.bfloat16, False, "hp", True, True, (0.0, INF)),
+    (1, 200, 2, 128, 1, 64, 128, torch.float16, True, "h", True, True, (0.0, INF)),
 ]
 
 
