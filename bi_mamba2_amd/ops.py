@@ -134,9 +134,27 @@ class _Call:
         self.p.workspace_bytes = ws.numel()
 
     def run(self, entry):
+        if torch.cuda.current_device() == self.device.index:
+            self.p.stream = torch.cuda.current_stream().cuda_stream
+            _lib.call(entry, self.p)
+            return
         with torch.cuda.device(self.device):
             self.p.stream = torch.cuda.current_stream().cuda_stream
             _lib.call(entry, self.p)
+
+    # ---- reuse of the input half of a call (the autograd function builds it once for forward and backward) ----
+    def snapshot(self):
+        """The parameter block as bytes plus the small converted tensors it points at (A, D, dt_bias copies)."""
+        return bytes(self.p), [t for t in self.keep if t.numel() <= 1 << 16]
+
+    @classmethod
+    def from_snapshot(cls, snap, x, nchunks):
+        self = cls.__new__(cls)
+        self.p = Params.from_buffer_copy(snap[0])
+        self.keep = list(snap[1])
+        self.device, self.dtype, self.dt_dtype = x.device, x.dtype, None
+        self.nchunks = nchunks
+        return self
 
 
 def _check_chunk(chunk_size):
@@ -410,11 +428,13 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
     like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
     out, out_x and the final states are materialised as tensors (the rest lives in a workspace).
-    keep_for_bwd=True appends a tenth element: the tuple (dt_out, cs_f, cs_b, states_f, states_b) that
-    _mamba_chunk_scan_combined_bwd accepts as `saved` to skip its recomputation."""
+    keep_for_bwd=True appends a tenth element: the tuple (dt_out, cs_f, cs_b, states_f, states_b, snapshot) that
+    _mamba_chunk_scan_combined_bwd accepts as `saved` to skip its recomputation (snapshot: the input half of the
+    parameter block, reused when the backward pass gets the same tensors)."""
     c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
     batch, seqlen, nheads, headdim = x.shape
     ngroups, dstate = B.shape[2], B.shape[3]
+    snap = c.snapshot() if keep_for_bwd else None
     out = c.new("out", x.shape, x.dtype)
     out_x = c.new("out_x", x.shape, x.dtype) if z is not None else None
     ff = c.new("final_f", (batch, nheads, headdim, dstate)); fb = c.new("final_b", (batch, nheads, headdim, dstate))
@@ -425,7 +445,7 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
         sshape = (batch, c.nchunks, nheads, headdim, dstate)
         sf = c.new("states_f", sshape); sb = c.new("states_b", sshape)
     if keep_for_bwd:
-        saved = (dt_out, cs_f, cs_b, sf, sb)
+        saved = (dt_out, cs_f, cs_b, sf, sb, snap)
     c.workspace(False)
     c.run("bimamba2_fwd")
     res = (out, out_x, dt_out, cs_f, cs_b, sf, sb, ff, fb)
@@ -441,11 +461,21 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     assert dfinal_states is None, "final states are not supported in the backward pass"
     assert not recompute_output, "recompute_output is not supported"
     assert dout.shape == x.shape
-    c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
+    snap = saved[5] if saved is not None and len(saved) > 5 else None
+    c = None
+    if snap is not None:
+        # the forward's parameter block, if the tensors handed back by autograd are still the ones it describes
+        c = _Call.from_snapshot(snap, x, (x.shape[1] + chunk_size - 1) // chunk_size)
+        same = (c.p.x == x.data_ptr() and c.p.dt == dt.data_ptr() and c.p.Bm == B.data_ptr() and c.p.Cm == C.data_ptr()
+                and (z is None or c.p.z == z.data_ptr()) and x.is_cuda)
+        if not same:
+            c = None
+    if c is None:
+        c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
     batch, seqlen, nheads, headdim = x.shape
     c.set_dout(dout)
     if saved is not None:
-        for name, t in zip(("dt_out", "cs_f", "cs_b", "states_f", "states_b"), saved):
+        for name, t in zip(("dt_out", "cs_f", "cs_b", "states_f", "states_b"), saved[:5]):
             c.put(name, t, torch.float32)
         c.p.fwd_saved = 1
     if z is not None:
@@ -487,7 +517,8 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
         out, out_x, ff, fb = res[0], res[1], res[7], res[8]
         saved = res[9] if keep else ()
         ctx.n_saved = len(saved)
-        ctx.save_for_backward(out_x if z is not None else None, x, dt, A, B, C, D, z, dt_bias, *saved)
+        ctx.snap = saved[5] if keep else None
+        ctx.save_for_backward(out_x if z is not None else None, x, dt, A, B, C, D, z, dt_bias, *saved[:5])
         ctx.dt_softplus = dt_softplus
         ctx.chunk_size = chunk_size
         ctx.dt_limit = dt_limit
@@ -500,7 +531,7 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout, *args):
         out_x, x, dt, A, B, C, D, z, dt_bias = ctx.saved_tensors[:9]
-        saved = ctx.saved_tensors[9:] if ctx.n_saved else None
+        saved = tuple(ctx.saved_tensors[9:]) + (ctx.snap,) if ctx.n_saved else None
         assert not ctx.return_final_states, "final states are not currently supported in the bwd pass"
         dx, ddt, dA, dB, dC, dD, dz, ddt_bias = _mamba_chunk_scan_combined_bwd(
             dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
