@@ -33,6 +33,42 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// ---- row-major tiles as MFMA operands: LDS transpose reads ------------------------------------------------------
+// A tile of 16-bit elements lies in LDS as it lies in global memory, [k][n] with n contiguous (rows of 64 elements,
+// 128 bytes), brought there by direct loads.  Its 16-byte chunks are swizzled, chunk c of row k sits at position
+// c ^ (k % 8), which keeps the reads below off each other's banks.
+// ds_read_b64_tr_b16 works on groups of 16 lanes: lane s supplies the address of 4 consecutive elements and lane j
+// receives element j % 4 of the lanes j / 4, j / 4 + 4, j / 4 + 8, j / 4 + 12.  Pointing lane s at row k0 + s / 4,
+// columns n0 + 4 * (s % 4) .. + 3 therefore hands lane j the elements [k0 .. k0 + 3][n0 + j]: four consecutive k of
+// "its" column, which is what an MFMA operand holds.  Two such reads give the 8 k of one 16x16x32 operand.
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+// byte offset inside a swizzled [rows][64] 16-bit tile of the 4 elements (k, n .. n + 3), n a multiple of 4
+__device__ __forceinline__ int tile64_tr_offset(int k, int n) {
+    return k * 128 + ((((n >> 3) ^ (k & 7)) << 4) | ((n & 4) << 1));
+}
+// fragment of lane (lr = lane % 16, lg = lane / 16): k = k0 + 8 * lg .. + 7 of column n0 + lr
+template <typename Frag> __device__ __forceinline__ Frag tile64_tr_frag(const void *tile, int k0, int n0, int lr, int lg) {
+    typedef __attribute__((address_space(3))) i16x4 *lds_i16x4_ptr;
+    const char *t = reinterpret_cast<const char *>(tile);
+    const int k = k0 + 8 * lg + (lr >> 2), n = n0 + 4 * (lr & 3);
+    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(t + tile64_tr_offset(k, n)));
+    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr)(t + tile64_tr_offset(k + 4, n)));
+    const i16x8 f = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(Frag, f);
+}
+// Requests rows [0, nrows) x 64 elements of a row-major global tile into such an LDS image: the calling wave brings the
+// units wave, wave + nwaves, ... of 64 lanes x 16 bytes (8 rows each); rows >= rvalid read row rvalid - 1.
+template <typename T>
+__device__ __forceinline__ void tile64_request(T *tile, const T *src, int64_t row_stride, int nrows, int rvalid, int wave, int nwaves,
+                                               int lane) {
+    static_assert(sizeof(T) == 2, "16-bit tiles");
+    for (int u = wave; u < nrows / 8; u += nwaves) {
+        const int row = u * 8 + (lane >> 3);
+        load16_to_lds(src + (int64_t)min(row, rvalid - 1) * row_stride + (((lane & 7) ^ (row & 7)) << 3), tile + u * 512);
+    }
+}
+
 // ---- LDS accesses issued from inline assembly ---------------------------------------------------------------
 // While a direct global->LDS load (global_load_lds) is in flight, the compiler makes every LDS access it knows of wait for
 // ALL outstanding vector memory operations, which defeats prefetching through LDS.  These accessors hide the DS

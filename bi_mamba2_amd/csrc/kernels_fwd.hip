@@ -186,6 +186,93 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_kernel(const bimamba2_pa
         }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// The same for 16-bit types with headdim % 64 == 0, dstate % 64 == 0, chunk_size % 32 == 0 and aligned operands: both
+// tiles travel as they are from global memory into LDS (direct loads: no registers, nothing to wait for until all of
+// the chunk is under way), and the MFMA operands are read from the row-major images with LDS transpose reads.  The
+// weights go onto the x-side fragment, one scaled copy per direction; the B-side fragments serve both directions.
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, bool DSTATES>
+__global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bimamba2_params p, int nc) {
+    typedef Mma<T> M;
+    typedef typename M::Frag Frag;
+    static_assert(sizeof(T) == 2, "16-bit operands");
+    __shared__ __attribute__((aligned(16))) T xt[BIMAMBA2_MAX_CHUNK * 64];
+    __shared__ __attribute__((aligned(16))) T bt[BIMAMBA2_MAX_CHUNK * 64];
+    __shared__ __attribute__((aligned(16))) float wf[BIMAMBA2_MAX_CHUNK], wb[BIMAMBA2_MAX_CHUNK];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lr = lane & 15, lg = lane >> 4;
+    const int nt = blockIdx.x, pt = blockIdx.y;
+    const int h = blockIdx.z % p.nheads, bc = blockIdx.z / p.nheads, c = bc % nc, b = bc / nc;
+    const int g = h / (p.nheads / p.ngroups);
+    const int Q = p.chunk_size, N = p.dstate, P = p.headdim;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const T *xp;
+    int64_t xs;
+    if (DSTATES) {
+        const T *src = reinterpret_cast<const T *>(p.has_z ? p.dout_x : p.dout);
+        if (p.has_z) { xs = (int64_t)p.nheads * P; xp = src + ((int64_t)b * p.seqlen + (int64_t)c * Q) * xs + (int64_t)h * P; }
+        else { xs = p.dout_sl; xp = src + b * p.dout_sb + (int64_t)c * Q * xs + h * p.dout_sh; }
+    } else {
+        xs = p.x_sl;
+        xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * xs + h * p.x_sh;
+    }
+    const T *bp;
+    int64_t bs;
+    if (DSTATES) { bs = p.C_sl; bp = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * bs + g * p.C_sg; }
+    else { bs = p.B_sl; bp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * bs + g * p.B_sg; }
+    const int rows = (limit + 31) & ~31;                   // K steps of 32 positions
+    tile64_request(xt, xp + pt * 64, xs, rows, limit, wave, NTHREADS / 64, lane);
+    tile64_request(bt, bp + nt * 64, bs, rows, limit, wave, NTHREADS / 64, lane);
+    const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
+    for (int q = threadIdx.x; q < rows; q += NTHREADS) {
+        float f = 0.f, r = 0.f;
+        if (q < limit) {
+            if (DSTATES) {
+                f = __expf(p.cs_f[o + q]);
+                r = __expf(p.cs_b[o + q]);
+            } else {
+                const float d = p.dt_out[o + q];
+                f = __expf(p.cs_f[o + Q - 1] - p.cs_f[o + q]) * d;
+                r = __expf(p.cs_b[o] - p.cs_b[o + q]) * d;
+            }
+        }
+        wf[q] = f;
+        wb[q] = r;
+    }
+    __syncthreads();       // (the compiler drains this wave's requests before its first LDS access; the barrier covers the rest)
+    f32x4 accf[4] = {}, accb[4] = {};
+    for (int k0 = 0; k0 < rows; k0 += 32) {
+        const Frag a = tile64_tr_frag<Frag>(xt, k0, wave * 16, lr, lg);
+        const f32x4 f0 = *reinterpret_cast<const f32x4 *>(wf + k0 + 8 * lg), f1 = *reinterpret_cast<const f32x4 *>(wf + k0 + 8 * lg + 4);
+        const f32x4 r0 = *reinterpret_cast<const f32x4 *>(wb + k0 + 8 * lg), r1 = *reinterpret_cast<const f32x4 *>(wb + k0 + 8 * lg + 4);
+        float vf[8], vb[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float v = to_f(a[i]);
+            vf[i] = v * (i < 4 ? f0[i & 3] : f1[i & 3]);
+            vb[i] = v * (i < 4 ? r0[i & 3] : r1[i & 3]);
+        }
+        const Frag af = M::pack(vf), ab = M::pack(vb);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const Frag bfr = tile64_tr_frag<Frag>(bt, k0, j * 16, lr, lg);
+            accf[j] = M::mma(af, bfr, accf[j]);
+            accb[j] = M::mma(ab, bfr, accb[j]);
+        }
+    }
+    float *of = (DSTATES ? p.dstates_f : p.states_f) + (int64_t)blockIdx.z * P * N;
+    float *ob = (DSTATES ? p.dstates_b : p.states_b) + (int64_t)blockIdx.z * P * N;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int pp = pt * 64 + wave * 16 + lg * 4 + i, n = nt * 64 + j * 16 + lr;
+            of[(int64_t)pp * N + n] = accf[j][i];
+            ob[(int64_t)pp * N + n] = accb[j][i];
+        }
+}
+
 // =========================================================================================================
 // inter-chunk recurrences, both directions, in place:
 //   forward : prev_f[0] = 0, prev_f[c+1] = e^{tot_c} prev_f[c] + S_f[c]   (final_f = value after the last chunk)
@@ -292,6 +379,13 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates) {
         fast = fast && al(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
     }
     hipStream_t s = stream_of(p);
+    if constexpr (sizeof(T) == 2) {
+        if (fast && p->chunk_size % 32 == 0) {
+            if (dstates) hipLaunchKernelGGL((chunk_state_direct_kernel<T, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            else hipLaunchKernelGGL((chunk_state_direct_kernel<T, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            return check_launch();
+        }
+    }
     if (dstates) {
         if (fast) hipLaunchKernelGGL((chunk_state_kernel<T, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
         else hipLaunchKernelGGL((chunk_state_kernel<T, true, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
