@@ -36,16 +36,18 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // ---- row-major tiles as MFMA operands: LDS transpose reads ------------------------------------------------------
 // A tile of 16-bit elements lies in LDS as it lies in global memory, [k][n] with n contiguous (rows of 64 elements,
 // 128 bytes), brought there by direct loads.  Its 16-byte chunks are swizzled, chunk c of row k sits at position
-// c ^ (k % 8), which keeps the reads below off each other's banks.
+// c ^ tile64_swz(k), which keeps the reads below (4 rows x 32 bytes per 16 lanes, rows 8 apart for the next 16 lanes)
+// off each other's banks.
 // ds_read_b64_tr_b16 works on groups of 16 lanes: lane s supplies the address of 4 consecutive elements and lane j
 // receives element j % 4 of the lanes j / 4, j / 4 + 4, j / 4 + 8, j / 4 + 12.  Pointing lane s at row k0 + s / 4,
 // columns n0 + 4 * (s % 4) .. + 3 therefore hands lane j the elements [k0 .. k0 + 3][n0 + j]: four consecutive k of
 // "its" column, which is what an MFMA operand holds.  Two such reads give the 8 k of one 16x16x32 operand.
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef short i16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ int tile64_swz(int k) { return (k & 7) ^ ((k >> 1) & 4); }
 // byte offset inside a swizzled [rows][64] 16-bit tile of the 4 elements (k, n .. n + 3), n a multiple of 4
 __device__ __forceinline__ int tile64_tr_offset(int k, int n) {
-    return k * 128 + ((((n >> 3) ^ (k & 7)) << 4) | ((n & 4) << 1));
+    return k * 128 + ((((n >> 3) ^ tile64_swz(k)) << 4) | ((n & 4) << 1));
 }
 // fragment of lane (lr = lane % 16, lg = lane / 16): k = k0 + 8 * lg .. + 7 of column n0 + lr
 template <typename Frag> __device__ __forceinline__ Frag tile64_tr_frag(const void *tile, int k0, int n0, int lr, int lg) {
@@ -65,7 +67,7 @@ __device__ __forceinline__ void tile64_request(T *tile, const T *src, int64_t ro
     static_assert(sizeof(T) == 2, "16-bit tiles");
     for (int u = wave; u < nrows / 8; u += nwaves) {
         const int row = u * 8 + (lane >> 3);
-        load16_to_lds(src + (int64_t)min(row, rvalid - 1) * row_stride + (((lane & 7) ^ (row & 7)) << 3), tile + u * 512);
+        load16_to_lds(src + (int64_t)min(row, rvalid - 1) * row_stride + (((lane & 7) ^ tile64_swz(row)) << 3), tile + u * 512);
     }
 }
 
@@ -95,6 +97,13 @@ template <typename V, int OFF> __device__ __forceinline__ V raw_lds_read_at(unsi
     static_assert(OFF >= 0 && OFF < 65536, "DS offset field is 16 bits");
     if constexpr (sizeof(V) == 16) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
     else asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+// LDS transpose read (see tile64_tr_frag) in the same raw form
+template <int OFF> __device__ __forceinline__ i16x4 raw_lds_tr16_read_at(unsigned addr) {
+    i16x4 v;
+    static_assert(OFF >= 0 && OFF < 65536, "DS offset field is 16 bits");
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
     return v;
 }
 template <int OFF> __device__ __forceinline__ void raw_lds_write_at(unsigned addr, float v) {
