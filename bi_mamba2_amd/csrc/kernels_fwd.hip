@@ -405,8 +405,48 @@ int launch_chunk_state(const bimamba2_params *p, bool dstates) {
     }
 }
 
+// The same with 16-byte accesses and one direction per workgroup (blockIdx.z = 2 b + dir); the loads of 8 chunks go out
+// together, unconditionally (past the last chunk a valid chunk is read again and not used).  Needs P*N % 4 == 0 and
+// 16-byte aligned tensors.
+__global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const bimamba2_params p, int nc) {
+    const int PN = p.headdim * p.dstate;
+    const int e = (blockIdx.x * NTHREADS + threadIdx.x) * 4;
+    const int h = blockIdx.y, b = blockIdx.z >> 1, dir = blockIdx.z & 1;
+    if (e >= PN) return;
+    const int Q = p.chunk_size;
+    const float *cs = (dir == 0 ? p.cs_f : p.cs_b) + ((int64_t)b * p.nheads + h) * nc * Q + (dir == 0 ? Q - 1 : 0);
+    const int64_t cstride = (int64_t)p.nheads * PN;
+    float *st = (dir == 0 ? p.states_f : p.states_b) + ((int64_t)b * nc * p.nheads + h) * PN + e;
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < nc; s0 += 8) {
+        f32x4 v[8];
+        float d[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int si = min(s0 + i, nc - 1), c = dir == 0 ? si : nc - 1 - si;
+            v[i] = *reinterpret_cast<const f32x4 *>(st + c * cstride);
+            d[i] = cs[(int64_t)c * Q];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (s0 + i < nc) {
+                const int c = dir == 0 ? s0 + i : nc - 1 - (s0 + i);
+                *reinterpret_cast<f32x4 *>(st + c * cstride) = s;
+                s = __expf(d[i]) * s + v[i];
+            }
+    }
+    float *fin = dir == 0 ? p.final_f : p.final_b;
+    if (fin) *reinterpret_cast<f32x4 *>(fin + ((int64_t)b * p.nheads + h) * PN + e) = s;
+}
+
 int launch_state_passing_fwd(const bimamba2_params *p) {
     const int nc = nchunks(p), PN = p->headdim * p->dstate;
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->final_f) && al(p->final_b)) {
+        dim3 grid((PN / 4 + NTHREADS - 1) / NTHREADS, p->nheads, p->batch * 2);
+        hipLaunchKernelGGL(state_passing_fwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+        return check_launch();
+    }
     dim3 grid((PN + NTHREADS - 1) / NTHREADS, p->nheads, p->batch);
     hipLaunchKernelGGL(state_passing_fwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
     return check_launch();
