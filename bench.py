@@ -35,9 +35,10 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def stage_table(w, e, fused=(False, False)):
+def stage_table(w, e, fused=(False, False, False)):
     """Algorithmic flops and bytes per launch of every stage kernel (e = bytes per element of x/B/C/z).
-    fused[0] / fused[1]: the forward scan / the dx kernel rebuilds its CB tiles from C and B instead of reading them."""
+    fused[0] / [1] / [2]: the forward scan / the dx kernel / the dCB kernel rebuilds its CB tiles from C and B instead of
+    reading them."""
     B, L, H, P, G, N, Q = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate", "chunk_size"))
     nc = (L + Q - 1) // Q
     u, ug = B * nc * H, B * nc * G                 # (b, c, h) and (b, c, g) units
@@ -60,7 +61,9 @@ def stage_table(w, e, fused=(False, False)):
                                        3 * e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + scan_cb[1][1]),
         "bimamba2_chunk_state_bwd_db": (u * 4 * Q * P * N, e * T4 + e * T2 + 5 * 4 * T1 + 2 * st + 4 * T2),
         "bimamba2_chunk_scan_bwd_dc": (u * 4 * Q * P * N, e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + 4 * T2),
-        "bimamba2_chunk_scan_bwd_dcb": (u * 2 * Q * Q * P, 2 * e * T4 + 3 * 4 * T1 + 2 * cb + 4 * B * H * nc * ((Q + 63) // 64) ** 2 * 128),
+        "bimamba2_chunk_scan_bwd_dcb": (u * 2 * Q * Q * P + (ug * 2 * Q * Q * N if fused[2] else 0),
+                                        2 * e * T4 + 3 * 4 * T1 + (2 * e * T2 if fused[2] else cb) + 2 * cb
+                                        + 4 * B * H * nc * ((Q + 63) // 64) ** 2 * 128),
         "bimamba2_bmm_chunk_bwd": (ug * 4 * Q * Q * N, 4 * e * T2 + cb + 2 * 4 * T2),
         "bimamba2_chunk_cumsum_bwd": (0, 2 * 4 * B * L * H + 8 * 4 * T1),
     }
@@ -197,15 +200,18 @@ def main():
     c.run("bimamba2_fwd")
     c.run("bimamba2_bwd")
     torch.cuda.synchronize()
-    reads_cb = [_lib.load().bimamba2_chunk_scan_reads_cb(ctypes.byref(c.p), d) for d in (0, 1)]
-    table = stage_table(w, e, fused=(reads_cb[0] == 0, reads_cb[1] == 0))
+    reads_cb = [_lib.load().bimamba2_chunk_scan_reads_cb(ctypes.byref(c.p), d) for d in (0, 1, 2)]
+    table = stage_table(w, e, fused=tuple(r == 0 for r in reads_cb))
+    if not any(reads_cb):
+        del table["bimamba2_bmm_chunk_fwd"]     # not launched by the composites for this problem
     kernels = {}
     reps = max(10, args.steps)
     for entry, (flops, nbytes) in table.items():
         if entry == "bimamba2_chunk_scan_bwd_dz" and not has_z:
             continue
         # time the scan stages the way the composites launch them: without CB / CBT when the kernel rebuilds it
-        hidden = {"bimamba2_chunk_scan_fwd": ("CB", 0), "bimamba2_chunk_scan_bwd_dx": ("CBT", 1)}.get(entry)
+        hidden = {"bimamba2_chunk_scan_fwd": ("CB", 0), "bimamba2_chunk_scan_bwd_dx": ("CBT", 1),
+                  "bimamba2_chunk_scan_bwd_dcb": ("CB", 2)}.get(entry)
         kept = None
         if hidden and reads_cb[hidden[1]] == 0:
             kept = getattr(c.p, hidden[0])

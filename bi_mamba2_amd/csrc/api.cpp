@@ -64,7 +64,8 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     need_f(q->dt_out, bhcq);
     need_f(q->cs_f, bhcq);
     need_f(q->cs_b, bhcq);
-    if (is_bwd || !scan_recomputes_cb(q, false)) need_f(q->CB, cbn);
+    // CB: read by the forward scan and by the dCB kernel unless they rebuild it; CB^T: by the dx kernel, likewise
+    if (is_bwd ? !(scan_recomputes_cb(q, true) && dcb_recomputes_cb(q)) : !scan_recomputes_cb(q, false)) need_f(q->CB, cbn);
     need_f(q->states_f, stn);
     need_f(q->states_b, stn);
     if (is_bwd) {
@@ -119,9 +120,10 @@ size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd) {
     return carve(&q, is_bwd, nullptr);
 }
 
-int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int is_bwd) {
+int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which) {
     if (check_problem(p)) return 1;
-    return scan_recomputes_cb(p, is_bwd != 0) ? 0 : 1;
+    if (which == 2) return dcb_recomputes_cb(p) ? 0 : 1;
+    return scan_recomputes_cb(p, which != 0) ? 0 : 1;
 }
 
 int bimamba2_chunk_cumsum_fwd(const bimamba2_params *p) {
@@ -216,7 +218,8 @@ int bimamba2_chunk_scan_bwd_dc(const bimamba2_params *p) {
 
 int bimamba2_chunk_scan_bwd_dcb(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->x); REQUIRE(p->CB); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    REQUIRE(p->x); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (!p->CB && !(p->Cm && p->Bm && dcb_recomputes_cb(p))) return BIMAMBA2_EINVAL;   // without CB the kernel rebuilds it from Cm, Bm
     REQUIRE(p->dCB); REQUIRE(p->dCBT); REQUIRE(p->da_intra);
     if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
     return launch_bwd_dcb(p);
@@ -264,7 +267,9 @@ int bimamba2_bwd(const bimamba2_params *p) {
         TRY(bimamba2_chunk_state_fwd(&q));
         TRY(bimamba2_state_passing_fwd(&q));
     }
-    TRY(bimamba2_bmm_chunk_fwd(&q));               // CB for the dCB kernel, CB^T when the dx kernel reads it
+    const bool need_cbt = !scan_recomputes_cb(&q, true), need_cb = need_cbt || !dcb_recomputes_cb(&q);
+    if (need_cb) TRY(bimamba2_bmm_chunk_fwd(&q));  // CB for the dCB kernel, CB^T for the dx kernel, unless they rebuild it
+    else q.CB = nullptr;
     if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
     TRY(bimamba2_chunk_scan_bwd_dstates(&q));
     TRY(bimamba2_state_passing_bwd(&q));

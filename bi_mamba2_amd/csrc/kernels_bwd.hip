@@ -922,14 +922,31 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
         f32x4 acc[4] = {};
         issue(0);
         if (nit > 1) issue(1);
+        if (p.CB) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float *cbg = p.CB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+            for (int j = 0; j < 4; ++j) {
+                const float *cbg = p.CB + ((int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int t = t0 + trow + i, s = s0 + j * 16 + lr;
-                cbr[j][i] = (t < limit && s < limit) ? cbg[(int64_t)t * Q + s] : 0.f;
+                for (int i = 0; i < 4; ++i) {
+                    const int t = t0 + trow + i, s = s0 + j * 16 + lr;
+                    cbr[j][i] = (t < limit && s < limit) ? cbg[(int64_t)t * Q + s] : 0.f;
+                }
             }
+        } else {
+            // no CB given: the tile CB[t, s] = C_t . B_s is rebuilt here, once per workgroup; both operands are read from
+            // global memory in MFMA layout (dstate is contiguous) and the product lands in the layout of cbr
+            const T *crow = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + ((int64_t)c * Q + min(t0 + wave * 16 + lr, limit - 1)) * p.C_sl + g * p.C_sg + lg * 8;
+            const T *brow = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * p.B_sl + g * p.B_sg + lg * 8;
+            for (int n0 = 0; n0 < p.dstate; n0 += 32) {
+                const Frag cf = M::load(crow + n0);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) cbr[j] = M::mma(cf, M::load(brow + (int64_t)min(s0 + j * 16 + lr, limit - 1) * p.B_sl + n0), cbr[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (t0 + trow + i >= limit || s0 + j * 16 + lr >= limit) cbr[j][i] = 0.f;
         }
         // settle these register loads here: inside the loop a wait for them would drain the ring's requests as well
         wait_vmcnt<0>();
@@ -1162,6 +1179,17 @@ template <typename T> static void launch_dcb_ring(dim3 grid, const bimamba2_para
     if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((bwd_dcb_ring_kernel<T>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
 }
 
+// whether the dCB kernel can do without CB (it rebuilds its tile from the C and B rows): the 16-bit ring variant, dstate a
+// multiple of 32, 16-byte aligned row matrices
+bool dcb_recomputes_cb(const bimamba2_params *p) {
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
+    if (p->dtype == BIMAMBA2_F32 || p->headdim % 64 || p->chunk_size % 64 || p->dstate % 32) return false;
+    if (!(al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh))) return false;
+    if (!(p->has_z ? al(p->dout_x) : (al(p->dout) && mult(p->dout_sb, p->dout_sl, p->dout_sh)))) return false;
+    return al(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg);
+}
+
 template <typename T>
 static int launch_dcb_t(const bimamba2_params *p) {
     const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
@@ -1171,6 +1199,7 @@ static int launch_dcb_t(const bimamba2_params *p) {
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     bool fast = p->headdim % (sizeof(T) == 2 ? 64 : 16) == 0 && al(p->x) && p->x_sb % VS == 0 && p->x_sl % VS == 0 && p->x_sh % VS == 0;
     fast = fast && (p->has_z ? al(p->dout_x) : (al(p->dout) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && p->dout_sh % VS == 0));
+    if (!p->CB && !dcb_recomputes_cb(p)) return BIMAMBA2_EINVAL;
     if (fast && sizeof(T) == 2 && p->chunk_size % 64 == 0) launch_dcb_ring<T>(grid, p, nc, nqt);
     else if (fast) hipLaunchKernelGGL((bwd_dcb_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
     else hipLaunchKernelGGL((bwd_dcb_kernel<T, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);

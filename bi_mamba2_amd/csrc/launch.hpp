@@ -15,6 +15,8 @@ int launch_state_passing_fwd(const bimamba2_params *p);
 int launch_chunk_scan(const bimamba2_params *p, bool bwd);
 // true when that launch recomputes CB (bwd: CB^T) from the C and B rows instead of reading it
 bool scan_recomputes_cb(const bimamba2_params *p, bool bwd);
+// true when the dCB launch can rebuild its CB tiles from the C and B rows (then CB may be NULL)
+bool dcb_recomputes_cb(const bimamba2_params *p);
 
 int launch_bwd_dz(const bimamba2_params *p);
 int launch_state_passing_bwd(const bimamba2_params *p);

@@ -103,12 +103,14 @@ size_t bimamba2_params_size(void);
 /* bytes of workspace the composite entry points need (is_bwd = 0: forward, 1: backward) */
 size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd);
 
-/* 0 when the chunk-scan launch of this problem recomputes the CB tiles it needs from the C and B rows inside the
- * kernel (16-bit dtype, dstate 64, headdim a multiple of 64, chunk_size a multiple of 32, 16-byte aligned
- * operands), 1 when it reads them: CB for bimamba2_chunk_scan_fwd (is_bwd = 0), CBT for bimamba2_chunk_scan_bwd_dx
- * (is_bwd = 1).  When it is 0 a caller of the single stages may pass that pointer as NULL (and skip the CBT buffer).
- * Fuses _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208) into the scan for those shapes. */
-int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int is_bwd);
+/* Whether a kernel of this problem reads CB (1) or rebuilds the CB tiles it needs from the C and B rows with MFMAs (0):
+ *   which = 0: bimamba2_chunk_scan_fwd reads CB      (0 for 16-bit dtype, dstate 64, headdim % 64 == 0, chunk_size % 32 == 0)
+ *   which = 1: bimamba2_chunk_scan_bwd_dx reads CBT  (same conditions)
+ *   which = 2: bimamba2_chunk_scan_bwd_dcb reads CB  (0 for 16-bit dtype, dstate % 32 == 0, headdim % 64 == 0, chunk_size % 64 == 0)
+ * always with 16-byte aligned operands.  When it is 0 a caller of the single stages may pass that pointer as NULL; when
+ * all three are 0, bimamba2_bmm_chunk_fwd is not needed at all.  Fuses _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208)
+ * into its consumers for those shapes. */
+int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which);
 
 /* Whole forward; replaces _mamba_chunk_scan_combined_fwd (src/ssd/bi/ssd_combined.py:297-331).
  * Needs: x dt A Bm Cm [D z dt_bias] out [out_x when has_z] [final_f final_b] workspace.  Intermediates given as
@@ -161,7 +163,8 @@ int bimamba2_chunk_state_bwd_db(const bimamba2_params *p);
  * (src/ssd/bi/ssd_chunk_scan.py:1829-1877); u_* are its ddA_cumsum_prev terms. */
 int bimamba2_chunk_scan_bwd_dc(const bimamba2_params *p);
 /* x, dout, dt_out, cs, CB -> dCB, dCBT, da_intra.  Replaces _chunk_scan_bwd_dcb (src/ssd/bi/ssd_chunk_scan.py:1880-1909)
- * and _chunk_scan_bwd_ddAcs_stable_fwd/_bwd (src/ssd/bi/ssd_chunk_scan.py:2036-2098) in one pass. */
+ * and _chunk_scan_bwd_ddAcs_stable_fwd/_bwd (src/ssd/bi/ssd_chunk_scan.py:2036-2098) in one pass.  With CB = NULL,
+ * allowed when bimamba2_chunk_scan_reads_cb(p, 2) is 0, the kernel rebuilds its CB tiles from Cm and Bm. */
 int bimamba2_chunk_scan_bwd_dcb(const bimamba2_params *p);
 /* dCB, dCBT, Cm, Bm, dBs, dCs -> dB, dC.  Replaces the two _bmm_chunk_bwd calls (src/ssd/bi/ssd_bmm.py:211-262). */
 int bimamba2_bmm_chunk_bwd(const bimamba2_params *p);
