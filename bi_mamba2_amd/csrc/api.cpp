@@ -123,6 +123,7 @@ size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd) {
 int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which) {
     if (check_problem(p)) return 1;
     if (which == 2) return dcb_recomputes_cb(p) ? 0 : 1;
+    if (which == 3) return chunk_state_does_cumsum(p) ? 0 : 1;
     return scan_recomputes_cb(p, which != 0) ? 0 : 1;
 }
 
@@ -239,14 +240,24 @@ int bimamba2_chunk_cumsum_bwd(const bimamba2_params *p) {
     return launch_chunk_cumsum_bwd(p);
 }
 
+// chunk cumsum + chunk states: one launch where the chunk-state kernel does both, else the two stages
+static int forward_cumsum_and_states(const bimamba2_params *q) {
+    if (chunk_state_does_cumsum(q)) {
+        REQUIRE(q->dt); REQUIRE(q->A); REQUIRE(q->x); REQUIRE(q->Bm);
+        if (q->has_dt_bias) REQUIRE(q->dt_bias);
+        return launch_chunk_state(q, false, true);
+    }
+    TRY(bimamba2_chunk_cumsum_fwd(q));
+    return bimamba2_chunk_state_fwd(q);
+}
+
 int bimamba2_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     bimamba2_params q = *p;
     const size_t need = carve(&q, 0, p->workspace);
     if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
-    TRY(bimamba2_chunk_cumsum_fwd(&q));
+    TRY(forward_cumsum_and_states(&q));
     if (q.CB) TRY(bimamba2_bmm_chunk_fwd(&q));     // given by the caller, or carved because the scan kernel reads it
-    TRY(bimamba2_chunk_state_fwd(&q));
     TRY(bimamba2_state_passing_fwd(&q));
     if (scan_recomputes_cb(&q, false)) q.CB = nullptr;
     TRY(bimamba2_chunk_scan_fwd(&q));
@@ -263,8 +274,7 @@ int bimamba2_bwd(const bimamba2_params *p) {
         REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
     } else {
         // recompute the forward intermediates (the reference does the same, src/ssd/bi/ssd_combined.py:373-380)
-        TRY(bimamba2_chunk_cumsum_fwd(&q));
-        TRY(bimamba2_chunk_state_fwd(&q));
+        TRY(forward_cumsum_and_states(&q));
         TRY(bimamba2_state_passing_fwd(&q));
     }
     const bool need_cbt = !scan_recomputes_cb(&q, true), need_cb = need_cbt || !dcb_recomputes_cb(&q);

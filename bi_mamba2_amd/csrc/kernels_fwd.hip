@@ -192,7 +192,10 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_kernel(const bimamba2_pa
 // the chunk is under way), and the MFMA operands are read from the row-major images with LDS transpose reads.  The
 // weights go onto the x-side fragment, one scaled copy per direction; the B-side fragments serve both directions.
 // ---------------------------------------------------------------------------------------------------------
-template <typename T, bool DSTATES>
+// CUMSUM (states only): the workgroup also does the work of chunk_cumsum_fwd_kernel for its (b, c, h) - wave 0 transforms
+// dt and scans it while the tiles are under way - and the first tile's workgroup writes dt_out, cs_f, cs_b for the later
+// kernels: one launch less in front of the forward pass.
+template <typename T, bool DSTATES, bool CUMSUM>
 __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bimamba2_params p, int nc) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
@@ -225,6 +228,51 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     tile64_request(xt, xp + pt * 64, xs, rows, limit, wave, NTHREADS / 64, lane);
     tile64_request(bt, bp + nt * 64, bs, rows, limit, wave, NTHREADS / 64, lane);
     const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
+    if constexpr (CUMSUM && !DSTATES) {
+        __shared__ float dts[BIMAMBA2_MAX_CHUNK], csfs[BIMAMBA2_MAX_CHUNK], csbs[BIMAMBA2_MAX_CHUNK];
+        if (wave == 0) {
+            const float A = p.A[h];
+            const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
+            const int64_t dto = b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
+            float v[4], a[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int q = lane * 4 + e;
+                const int64_t at = dto + (int64_t)min(q, limit - 1) * p.dt_sl;
+                float d = p.dt_dtype == BIMAMBA2_F32 ? reinterpret_cast<const float *>(p.dt)[at]
+                        : p.dt_dtype == BIMAMBA2_BF16 ? to_f(reinterpret_cast<const bf16_t *>(p.dt)[at])
+                                                      : to_f(reinterpret_cast<const f16_t *>(p.dt)[at]);
+                d += bias;
+                if (p.dt_softplus) d = d > 20.f ? d : log1pf(expf(d));
+                d = fminf(fmaxf(d, p.dt_min), p.dt_max);
+                if (q >= limit) d = 0.f;
+                v[e] = d;
+                a[e] = d * A;
+            }
+            float pf[4], sb[4];
+            pf[0] = a[0]; pf[1] = pf[0] + a[1]; pf[2] = pf[1] + a[2]; pf[3] = pf[2] + a[3];
+            sb[3] = a[3]; sb[2] = sb[3] + a[2]; sb[1] = sb[2] + a[1]; sb[0] = sb[1] + a[0];
+            const float tot = pf[3];
+            const float before = wave_incl_prefix(tot, lane) - tot, after = wave_incl_suffix(tot, lane) - tot;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int q = lane * 4 + e;
+                dts[q] = v[e];
+                csfs[q] = before + pf[e];
+                csbs[q] = after + sb[e];
+                if (q < Q && nt == 0 && pt == 0) {
+                    p.dt_out[o + q] = v[e];
+                    p.cs_f[o + q] = before + pf[e];
+                    p.cs_b[o + q] = after + sb[e];
+                }
+            }
+        }
+        __syncthreads();
+        for (int q = threadIdx.x; q < rows; q += NTHREADS) {
+            wf[q] = q < limit ? __expf(csfs[Q - 1] - csfs[q]) * dts[q] : 0.f;
+            wb[q] = q < limit ? __expf(csbs[0] - csbs[q]) * dts[q] : 0.f;
+        }
+    } else
     for (int q = threadIdx.x; q < rows; q += NTHREADS) {
         float f = 0.f, r = 0.f;
         if (q < limit) {
@@ -365,7 +413,7 @@ int launch_bmm_chunk_fwd(const bimamba2_params *p) {
 }
 
 template <typename T>
-static int launch_chunk_state_t(const bimamba2_params *p, bool dstates) {
+static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cumsum) {
     const int nc = nchunks(p);
     dim3 grid((p->dstate + 63) / 64, (p->headdim + 63) / 64, p->batch * nc * p->nheads);
     constexpr int VS = 16 / (int)sizeof(T);
@@ -381,11 +429,13 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates) {
     hipStream_t s = stream_of(p);
     if constexpr (sizeof(T) == 2) {
         if (fast && p->chunk_size % 32 == 0) {
-            if (dstates) hipLaunchKernelGGL((chunk_state_direct_kernel<T, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
-            else hipLaunchKernelGGL((chunk_state_direct_kernel<T, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            if (dstates) hipLaunchKernelGGL((chunk_state_direct_kernel<T, true, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            else if (cumsum) hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            else hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
             return check_launch();
         }
     }
+    if (cumsum) return BIMAMBA2_EINVAL;      // the caller checked chunk_state_does_cumsum()
     if (dstates) {
         if (fast) hipLaunchKernelGGL((chunk_state_kernel<T, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
         else hipLaunchKernelGGL((chunk_state_kernel<T, true, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
@@ -396,13 +446,22 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates) {
     return check_launch();
 }
 
-int launch_chunk_state(const bimamba2_params *p, bool dstates) {
+int launch_chunk_state(const bimamba2_params *p, bool dstates, bool cumsum) {
     switch (p->dtype) {
-        case BIMAMBA2_F32: return launch_chunk_state_t<float>(p, dstates);
-        case BIMAMBA2_BF16: return launch_chunk_state_t<bf16_t>(p, dstates);
-        case BIMAMBA2_F16: return launch_chunk_state_t<f16_t>(p, dstates);
+        case BIMAMBA2_F32: return launch_chunk_state_t<float>(p, dstates, cumsum);
+        case BIMAMBA2_BF16: return launch_chunk_state_t<bf16_t>(p, dstates, cumsum);
+        case BIMAMBA2_F16: return launch_chunk_state_t<f16_t>(p, dstates, cumsum);
         default: return BIMAMBA2_EUNSUPPORTED;
     }
+}
+
+// whether launch_chunk_state(p, false, true) exists for this problem: the chunk-state launch that also does the chunk
+// cumsum (16-bit dtype, headdim and dstate multiples of 64, chunk_size a multiple of 32, aligned x and B)
+bool chunk_state_does_cumsum(const bimamba2_params *p) {
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
+    return p->dtype != BIMAMBA2_F32 && p->headdim % 64 == 0 && p->dstate % 64 == 0 && p->chunk_size % 32 == 0 && al(p->Bm) &&
+           mult(p->B_sb, p->B_sl, p->B_sg) && al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
 }
 
 // The same with 16-byte accesses and one direction per workgroup (blockIdx.z = 2 b + dir); the loads of 8 chunks go out

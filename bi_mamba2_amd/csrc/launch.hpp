@@ -10,7 +10,8 @@ static inline int check_launch() { return hipGetLastError() == hipSuccess ? BIMA
 
 int launch_chunk_cumsum_fwd(const bimamba2_params *p);
 int launch_bmm_chunk_fwd(const bimamba2_params *p);
-int launch_chunk_state(const bimamba2_params *p, bool dstates);
+int launch_chunk_state(const bimamba2_params *p, bool dstates, bool cumsum = false);   // cumsum: also does the chunk cumsum
+bool chunk_state_does_cumsum(const bimamba2_params *p);
 int launch_state_passing_fwd(const bimamba2_params *p);
 int launch_chunk_scan(const bimamba2_params *p, bool bwd);
 // true when that launch recomputes CB (bwd: CB^T) from the C and B rows instead of reading it

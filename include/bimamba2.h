@@ -107,8 +107,10 @@ size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd);
  *   which = 0: bimamba2_chunk_scan_fwd reads CB      (0 for 16-bit dtype, dstate 64, headdim % 64 == 0, chunk_size % 32 == 0)
  *   which = 1: bimamba2_chunk_scan_bwd_dx reads CBT  (same conditions)
  *   which = 2: bimamba2_chunk_scan_bwd_dcb reads CB  (0 for 16-bit dtype, dstate % 32 == 0, headdim % 64 == 0, chunk_size % 64 == 0)
+ *   which = 3: (not about CB) 1 when bimamba2_fwd launches bimamba2_chunk_cumsum_fwd on its own, 0 when its chunk-state
+ *              launch does the cumsum as well (16-bit dtype, headdim and dstate multiples of 64, chunk_size % 32 == 0)
  * always with 16-byte aligned operands.  When it is 0 a caller of the single stages may pass that pointer as NULL; when
- * all three are 0, bimamba2_bmm_chunk_fwd is not needed at all.  Fuses _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208)
+ * the first three are 0, bimamba2_bmm_chunk_fwd is not needed at all.  Fuses _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208)
  * into its consumers for those shapes. */
 int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which);
 
