@@ -196,7 +196,7 @@ def main():
     c.new("ddA_chunk_f", (w["batch"], w["nheads"], nc, nsplit)); c.new("ddA_chunk_b", (w["batch"], w["nheads"], nc, nsplit))
     slices = (w["nheads"] // w["ngroups"] + 3) // 4
     c.new("dBs", (slices,) + tuple(inp["B"].shape)); c.new("dCs", (slices,) + tuple(inp["B"].shape))
-    c.new("red", (max(w["batch"] * nc * w["nheads"] * w["headdim"], 2 * w["batch"] * nc * w["nheads"]),))
+    c.new("red", (w["batch"] * nc * w["nheads"] * w["headdim"] + 2 * w["batch"] * nc * w["nheads"],))
     c.run("bimamba2_fwd")
     c.run("bimamba2_bwd")
     torch.cuda.synchronize()

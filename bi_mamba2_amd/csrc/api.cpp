@@ -89,8 +89,8 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
         const size_t bn = slices * q->batch * q->seqlen * q->ngroups * q->dstate;
         need_f(q->dBs, bn);
         need_f(q->dCs, bn);
-        const size_t red = std::max((size_t)q->batch * nc * q->nheads * q->headdim, (size_t)2 * q->batch * nc * q->nheads);
-        need_f(q->red, red);
+        // partial sums of dD, then those of dA and ddt_bias (the composite reduces all three in one launch at the end)
+        need_f(q->red, (size_t)q->batch * nc * q->nheads * q->headdim + (size_t)2 * q->batch * nc * q->nheads);
     }
     return (cv.off + 255) & ~size_t(255);
 }
@@ -283,16 +283,34 @@ int bimamba2_bwd(const bimamba2_params *p) {
     if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
     TRY(bimamba2_chunk_scan_bwd_dstates(&q));
     TRY(bimamba2_state_passing_bwd(&q));
+    ReduceJobs jobs;
     {
+        // as bimamba2_chunk_scan_bwd_dx, with the reduction of the dD partial sums left for the end
         bimamba2_params qx = q;
         if (scan_recomputes_cb(&q, true)) qx.CBT = nullptr;
-        TRY(bimamba2_chunk_scan_bwd_dx(&qx));
+        REQUIRE(qx.dx); REQUIRE(qx.ddt_direct);
+        if (qx.has_D) { REQUIRE(qx.D); REQUIRE(qx.dD); }
+        const int nc = nchunks(&q);
+        if (q.headdim > (q.dtype == BIMAMBA2_F32 ? 32 : 64))
+            TRY(launch_fill(q.ddt_direct, (size_t)q.batch * q.nheads * nc * q.chunk_size, 0.f, stream_of(&q)));
+        TRY(launch_chunk_scan(&qx, true));
+        if (q.has_D) {
+            if (q.D_has_hdim) jobs.job[jobs.n++] = ReduceJob{q.red, q.dD, q.batch * nc, q.nheads * q.headdim, 1};
+            else jobs.job[jobs.n++] = ReduceJob{q.red, q.dD, q.batch * nc, q.nheads, q.headdim};
+        }
     }
     TRY(bimamba2_chunk_state_bwd_db(&q));
     TRY(bimamba2_chunk_scan_bwd_dc(&q));
     TRY(bimamba2_chunk_scan_bwd_dcb(&q));
     TRY(bimamba2_bmm_chunk_bwd(&q));
-    TRY(bimamba2_chunk_cumsum_bwd(&q));
+    {
+        // as bimamba2_chunk_cumsum_bwd, its partial sums behind those of dD
+        bimamba2_params qc = q;
+        qc.red = q.red + (size_t)q.batch * nchunks(&q) * q.nheads * q.headdim;
+        REQUIRE(q.ddt); REQUIRE(q.dA);
+        TRY(launch_chunk_cumsum_bwd(&qc, &jobs));
+    }
+    TRY(launch_reduce_jobs(jobs, stream_of(&q)));
     return BIMAMBA2_OK;
 }
 

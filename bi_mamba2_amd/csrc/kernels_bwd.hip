@@ -47,6 +47,31 @@ int launch_reduce(const float *in, float *out, int ni, int nj, int nk, hipStream
     return check_launch();
 }
 
+// several such reductions in one launch (the backward pass ends with three small ones)
+__global__ __launch_bounds__(NTHREADS) void reduce_jobs_kernel(ReduceJobs jobs) {
+    __shared__ float red[4];
+    int j = blockIdx.x, k = 0;
+    while (k + 1 < jobs.n && j >= jobs.job[k].nj) { j -= jobs.job[k].nj; ++k; }
+    const ReduceJob jb = jobs.job[k];
+    float s = 0.f;
+    const int total = jb.ni * jb.nk;
+    for (int t = threadIdx.x; t < total; t += NTHREADS) {
+        const int i = t / jb.nk, kk = t - i * jb.nk;
+        s += jb.in[((int64_t)i * jb.nj + j) * jb.nk + kk];
+    }
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) jb.out[j] = red[0] + red[1] + red[2] + red[3];
+}
+int launch_reduce_jobs(const ReduceJobs &jobs, hipStream_t stream) {
+    int blocks = 0;
+    for (int k = 0; k < jobs.n; ++k) blocks += jobs.job[k].nj;
+    if (blocks == 0) return BIMAMBA2_OK;
+    hipLaunchKernelGGL(reduce_jobs_kernel, dim3(blocks), dim3(NTHREADS), 0, stream, jobs);
+    return check_launch();
+}
+
 // =========================================================================================================
 // dz = dout * out_x * sigmoid(z) (1 + z (1 - sigmoid(z)));  dout_x = dout * z * sigmoid(z)
 // =========================================================================================================
@@ -1465,7 +1490,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
     }
 }
 
-int launch_chunk_cumsum_bwd(const bimamba2_params *p) {
+int launch_chunk_cumsum_bwd(const bimamba2_params *p, ReduceJobs *defer) {
     const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
     const int PN = p->headdim * p->dstate;
     const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS);
@@ -1479,6 +1504,12 @@ int launch_chunk_cumsum_bwd(const bimamba2_params *p) {
     int rc = check_launch();
     if (rc) return rc;
     const int ni = p->batch * nc;
+    if (defer) {
+        // the caller runs these together with its other reductions
+        defer->job[defer->n++] = ReduceJob{p->red, p->dA, ni, p->nheads, 1};
+        if (p->has_dt_bias && p->ddt_bias) defer->job[defer->n++] = ReduceJob{p->red + (int64_t)ni * p->nheads, p->ddt_bias, ni, p->nheads, 1};
+        return BIMAMBA2_OK;
+    }
     rc = launch_reduce(p->red, p->dA, ni, p->nheads, 1, stream_of(p));
     if (rc) return rc;
     if (p->has_dt_bias && p->ddt_bias) rc = launch_reduce(p->red + (int64_t)ni * p->nheads, p->ddt_bias, ni, p->nheads, 1, stream_of(p));

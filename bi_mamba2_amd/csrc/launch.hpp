@@ -25,7 +25,12 @@ int launch_bwd_dbdc(const bimamba2_params *p, bool is_db);
 int launch_bwd_dcb(const bimamba2_params *p);
 int dcb_slices(const bimamba2_params *p);   // head slices whose dCB partial sums the kernel keeps apart
 int launch_bmm_chunk_bwd(const bimamba2_params *p);
-int launch_chunk_cumsum_bwd(const bimamba2_params *p);
+// out[j] = sum_i sum_k in[(i*nj + j)*nk + k]
+struct ReduceJob { const float *in; float *out; int ni, nj, nk; };
+struct ReduceJobs { ReduceJob job[4]; int n = 0; };
+int launch_reduce_jobs(const ReduceJobs &jobs, hipStream_t stream);
+// defer != NULL: the final reductions of dA and ddt_bias are appended to *defer instead of being launched
+int launch_chunk_cumsum_bwd(const bimamba2_params *p, ReduceJobs *defer = nullptr);
 int launch_fill(float *ptr, size_t n, float value, hipStream_t stream);
 // out[j] = sum_{i<ni} sum_{k<nk} in[(i*nj + j)*nk + k]
 int launch_reduce(const float *in, float *out, int ni, int nj, int nk, hipStream_t stream);
