@@ -28,10 +28,11 @@ WORKLOAD = dict(batch=4, seqlen=2048, nheads=32, headdim=64, ngroups=1, dstate=6
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
 # size); None until measured for the kernel in question.  Source: the summaries under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "bimamba2_chunk_scan_bwd_dcb": 264.5e6, "bimamba2_chunk_scan_bwd_dc": 203.1e6, "bimamba2_chunk_state_bwd_db": 202.1e6,
-    "bimamba2_chunk_scan_fwd": 235.7e6, "bimamba2_chunk_scan_bwd_dx": 191.4e6, "bimamba2_chunk_scan_bwd_dz": 167.9e6,
-    "bimamba2_state_passing_bwd": 101.9e6, "bimamba2_bmm_chunk_bwd": 63.7e6, "bimamba2_chunk_state_fwd": 78.4e6,
-    "bimamba2_chunk_scan_bwd_dstates": 78.4e6, "bimamba2_state_passing_fwd": 70.6e6,
+    "bimamba2_chunk_scan_bwd_dcb": 104.1e6, "bimamba2_chunk_scan_bwd_dc": 90.0e6, "bimamba2_chunk_state_bwd_db": 90.0e6,
+    "bimamba2_chunk_scan_fwd": 213.6e6, "bimamba2_chunk_scan_bwd_dx": 174.7e6, "bimamba2_chunk_scan_bwd_dz": 167.9e6,
+    "bimamba2_state_passing_bwd": 101.9e6, "bimamba2_bmm_chunk_bwd": 61.0e6, "bimamba2_chunk_state_fwd": 78.1e6,
+    "bimamba2_chunk_scan_bwd_dstates": 78.1e6, "bimamba2_state_passing_fwd": 69.5e6, "bimamba2_chunk_cumsum_bwd": 24.3e6,
+    "bimamba2_bmm_chunk_fwd": 23.1e6,
 }
 
 
