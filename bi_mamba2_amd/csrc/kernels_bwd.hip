@@ -1375,44 +1375,61 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
     const int Q = p.chunk_size, H = p.nheads;
     const int limit = min(Q, p.seqlen - c * Q);
     const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
-    float vf[4], vb[4], uf[4], ub[4], di[4];
+    // Every load of the kernel goes out here, unconditionally and from clamped (valid) addresses, before anything is
+    // used: a load that is waited for costs microseconds, and conditional loads get serialised by the compiler.
+    float vf[4], vb[4], uf[4], ub[4], di[4], dtr[4], ddr[4];
+    const DT *dt = reinterpret_cast<const DT *>(p.dt) + b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const int q = lane * 4 + e;
-        const bool ok = q < limit;
-        vf[e] = ok ? p.v_f[o + q] : 0.f;
-        vb[e] = ok ? p.v_b[o + q] : 0.f;
-        uf[e] = ok ? p.u_f[o + q] : 0.f;
-        ub[e] = ok ? p.u_b[o + q] : 0.f;
+        const int qc = min(lane * 4 + e, limit - 1);
+        vf[e] = p.v_f[o + qc];
+        vb[e] = p.v_b[o + qc];
+        uf[e] = p.u_f[o + qc];
+        ub[e] = p.u_b[o + qc];
+        ddr[e] = p.ddt_direct[o + qc];
+        dtr[e] = to_f(dt[(int64_t)qc * p.dt_sl]);
+    }
+    const float A = p.A[h];
+    const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
+    float chunk_term = 0.f;
+    for (int s = 0; s < nsplit; ++s)
+        chunk_term += p.ddA_chunk_f[(((int64_t)b * H + h) * nc + c) * nsplit + s] + p.ddA_chunk_b[(((int64_t)b * H + h) * nc + c) * nsplit + s];
+    // within-chunk part from the per-tile vectors of the dCB kernel; tile I = lane / 16 holds this lane's positions.
+    // Four tiles per side at most (Q <= 256): tile indices past nqt are clamped for the loads and masked afterwards.
+    const int I = lane >> 4, i0 = (lane & 15) * 4, Ic = min(I, nqt - 1);
+    const float *tv = p.da_intra + (o / Q) * nqt * nqt * DCB_VEC;
+    float4 colv[4], rowv[4], tot[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const int ac = min(a, nqt - 1);
+        colv[a] = *reinterpret_cast<const float4 *>(tv + (ac * nqt + Ic) * DCB_VEC + i0);          // [0] of tile (a, I)
+        rowv[a] = *reinterpret_cast<const float4 *>(tv + (Ic * nqt + ac) * DCB_VEC + 64 + i0);     // [1] of tile (I, a)
+#pragma unroll
+        for (int bq = 0; bq < 4; ++bq) tot[a][bq] = *reinterpret_cast<const float4 *>(tv + (ac * nqt + min(bq, nqt - 1)) * DCB_VEC + i0);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (lane * 4 + e >= limit) vf[e] = vb[e] = uf[e] = ub[e] = 0.f;
         di[e] = 0.f;
     }
-    // within-chunk part from the per-tile vectors of bwd_dcb_kernel; tile I = lane / 16 holds this lane's positions
     {
-        const int I = lane >> 4, i0 = (lane & 15) * 4;
         if (I < nqt) {
-            const float *tv = p.da_intra + (o / Q) * nqt * nqt * DCB_VEC;
-            auto vec = [&](int tile, int which, float (&r)[4], bool add) {
-                const float4 v = *reinterpret_cast<const float4 *>(tv + tile * DCB_VEC + which * 64 + i0);
-                if (add) { r[0] += v.x; r[1] += v.y; r[2] += v.z; r[3] += v.w; }
-                else { r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w; }
-            };
+            auto add = [](float (&r)[4], const float4 &v) { r[0] += v.x; r[1] += v.y; r[2] += v.z; r[3] += v.w; };
             // the diagonal tile's difference vectors join the exclusive scans: cwf gets cw_f - rw_f, cwb gets cw_b - rw_b
-            float cwf[4], cwb[4], rwf[4] = {0.f, 0.f, 0.f, 0.f}, rwb[4] = {0.f, 0.f, 0.f, 0.f};
-            vec(I * nqt + I, 0, cwf, false);
-            vec(I * nqt + I, 1, cwb, false);
+            float cwf[4] = {0.f, 0.f, 0.f, 0.f}, cwb[4] = {0.f, 0.f, 0.f, 0.f}, rwf[4] = {0.f, 0.f, 0.f, 0.f}, rwb[4] = {0.f, 0.f, 0.f, 0.f};
             float between = 0.f;
-            for (int a = 0; a < nqt; ++a) {
-                if (a > I) { vec(a * nqt + I, 0, cwf, true); vec(I * nqt + a, 1, rwb, true); }
-                if (a < I) { vec(I * nqt + a, 1, rwf, true); vec(a * nqt + I, 0, cwb, true); }
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                if (a < nqt) {
+                    if (a == I) { add(cwf, colv[a]); add(cwb, rowv[a]); }
+                    if (a > I) { add(cwf, colv[a]); add(rwb, rowv[a]); }
+                    if (a < I) { add(rwf, rowv[a]); add(cwb, colv[a]); }
+                    // tiles with this tile strictly between their row tile and column tile add their total
+#pragma unroll
+                    for (int bq = 0; bq < 4; ++bq)
+                        if (bq < nqt && ((bq < I && I < a) || (a < I && I < bq))) between += tot[a][bq].x + tot[a][bq].y + tot[a][bq].z + tot[a][bq].w;
+                }
             }
-            // tiles with this tile strictly between their row tile and column tile add their total
-            for (int a = 0; a < nqt; ++a)
-                for (int bq = 0; bq < nqt; ++bq)
-                    if ((bq < I && I < a) || (a < I && I < bq)) {
-                        float t4[4];
-                        vec(a * nqt + bq, 0, t4, false);
-                        between += t4[0] + t4[1] + t4[2] + t4[3];
-                    }
             between = row16_sum(between);
             // forward: exclusive prefix of cwf + inclusive suffix of rwf; reverse: inclusive prefix of rwb + exclusive suffix of cwb
             const float t_cwf = cwf[0] + cwf[1] + cwf[2] + cwf[3], t_rwb = rwb[0] + rwb[1] + rwb[2] + rwb[3];
@@ -1433,9 +1450,6 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
             }
         }
     }
-    float chunk_term = 0.f;
-    for (int s = 0; s < nsplit; ++s)
-        chunk_term += p.ddA_chunk_f[(((int64_t)b * H + h) * nc + c) * nsplit + s] + p.ddA_chunk_b[(((int64_t)b * H + h) * nc + c) * nsplit + s];
     // lane totals and cross-lane scans
     const float tvf = vf[0] + vf[1] + vf[2] + vf[3], tvb = vb[0] + vb[1] + vb[2] + vb[3];
     const float tuf = uf[0] + uf[1] + uf[2] + uf[3], tub = ub[0] + ub[1] + ub[2] + ub[3];
@@ -1460,21 +1474,18 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
             ex_vb += vb[e];
         }
     }
-    const float A = p.A[h];
-    const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
-    const DT *dt = reinterpret_cast<const DT *>(p.dt) + b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
     DT *ddt = reinterpret_cast<DT *>(p.ddt);
     float sA = 0.f, sb = 0.f;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int q = lane * 4 + e;
         if (q < limit) {
-            const float pre = to_f(dt[(int64_t)q * p.dt_sl]) + bias;
+            const float pre = dtr[e] + bias;
             float d = pre;
             if (p.dt_softplus) d = d > 20.f ? d : log1pf(expf(d));
             const bool clamped = d < p.dt_min || d > p.dt_max;
             d = fminf(fmaxf(d, p.dt_min), p.dt_max);
-            float g = da[e] * A + p.ddt_direct[o + q];
+            float g = da[e] * A + ddr[e];
             if (clamped) g = 0.f;
             if (p.dt_softplus && pre <= 20.f) g *= 1.f / (1.f + expf(-pre));
             ddt[((int64_t)b * p.seqlen + (int64_t)c * Q + q) * H + h] = from_f<DT>(g);
