@@ -237,14 +237,16 @@ def _state_passing_fwd(states_f, states_b, dA_cumsum_f, dA_cumsum_b, return_fina
     return pf, pb, ff, fb
 
 
-def _chunk_scan_fwd(CB, x, dt, dA_cumsum_f, dA_cumsum_b, C, states_f, states_b, D=None, z=None):
-    """-> out, out_x (out_x is None without z)."""
+def _chunk_scan_fwd(CB, x, dt, dA_cumsum_f, dA_cumsum_b, C, states_f, states_b, D=None, z=None, B=None):
+    """-> out, out_x (out_x is None without z).  CB may be None when B is given and the problem is one whose scan
+    kernel rebuilds CB from C and B (bimamba2_chunk_scan_reads_cb == 0); anything else raises ValueError."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape
     _, _, ngroups, dstate = C.shape
     assert nheads % ngroups == 0
     assert C.shape == (batch, seqlen, ngroups, dstate)
-    assert CB.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    assert CB is None or CB.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    assert CB is not None or B is not None, "without CB the kernel needs B to rebuild it"
     if z is not None:
         assert z.shape == x.shape
     if D is not None:
@@ -253,6 +255,8 @@ def _chunk_scan_fwd(CB, x, dt, dA_cumsum_f, dA_cumsum_b, C, states_f, states_b, 
     assert states_f.shape == (batch, nchunks, nheads, headdim, dstate) and states_b.shape == states_f.shape
     c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, x.dtype, x.device)
     c.set_x(x); c.set_C(C); c.set_z(z); c.set_D(D)
+    if CB is None:
+        c.set_B(B)
     c.put("CB", CB, torch.float32); c.put("dt_out", dt, torch.float32)
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     c.put("states_f", states_f, torch.float32); c.put("states_b", states_b, torch.float32)
@@ -303,18 +307,25 @@ def _state_passing_bwd(states_f, states_b, dA_cumsum_f, dA_cumsum_b, dstates_f, 
     return gf, gb, af.sum(-1), ab.sum(-1)
 
 
-def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum_f, dA_cumsum_b, B, CB, dout, dstates_f, dstates_b, D=None, dx=None):
-    """-> dx, ddt_direct (batch, nheads, nchunks, chunk_size) float32, dD."""
+def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum_f, dA_cumsum_b, B, CB, dout, dstates_f, dstates_b, D=None, dx=None,
+                                   C=None):
+    """-> dx, ddt_direct (batch, nheads, nchunks, chunk_size) float32, dD.  CB may be None when C is given and the
+    kernel rebuilds it (see _chunk_scan_fwd)."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape
     _, _, ngroups, dstate = B.shape
     assert nheads % ngroups == 0
-    assert CB.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    assert CB is None or CB.shape == (batch, nchunks, ngroups, chunk_size, chunk_size)
+    assert CB is not None or C is not None, "without CB the kernel needs C to rebuild it"
     assert dout.shape == x.shape
     assert dstates_f.shape == (batch, nchunks, nheads, headdim, dstate) and dstates_b.shape == dstates_f.shape
     c = _Call(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size, x.dtype, x.device)
     c.set_x(x); c.set_B(B); c.set_dout(dout); c.set_D(D)
-    c.put("CBT", CB.transpose(-1, -2).contiguous(), torch.float32); c.put("dt_out", dt, torch.float32)
+    if CB is None:
+        c.set_C(C)
+    else:
+        c.put("CBT", CB.transpose(-1, -2).contiguous(), torch.float32)
+    c.put("dt_out", dt, torch.float32)
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     c.put("dstates_f", dstates_f, torch.float32); c.put("dstates_b", dstates_b, torch.float32)
     dx = c.put("dx", dx) if dx is not None else c.new("dx", x.shape, x.dtype)
@@ -361,14 +372,18 @@ def _chunk_scan_bwd_dC(states_f, states_b, dA_cumsum_f, dA_cumsum_b, dout, C=Non
     return dCs, uf, ub
 
 
-def _chunk_scan_bwd_dcb(x, dt, dA_cumsum_f, dA_cumsum_b, dout, CB, ngroups=1):
+def _chunk_scan_bwd_dcb(x, dt, dA_cumsum_f, dA_cumsum_b, dout, CB, ngroups=1, B=None, C=None):
     """-> dCB (batch, nchunks, ngroups, Q, Q) float32 and the per-tile vectors (batch, nheads, nchunks, tiles, 2, 64)
     from which chunk_cumsum_bwd assembles the within-chunk part of d(dt*A) (the reference's ddA_f + ddA_b of
-    its two "stable" kernels): column / row sums of off-diagonal 64x64 tiles, full contribution of diagonal ones."""
+    its two "stable" kernels): column / row sums of off-diagonal 64x64 tiles, full contribution of diagonal ones.
+    CB may be None when B and C are given and the kernel rebuilds its CB tiles (see _chunk_scan_fwd)."""
     batch, seqlen, nheads, headdim = x.shape
     _, _, nchunks, chunk_size = dt.shape
-    c = _Call(batch, seqlen, nheads, headdim, ngroups, 1, chunk_size, x.dtype, x.device)
+    assert CB is not None or (B is not None and C is not None), "without CB the kernel needs B and C to rebuild it"
+    c = _Call(batch, seqlen, nheads, headdim, ngroups, 1 if CB is not None else B.shape[-1], chunk_size, x.dtype, x.device)
     c.set_x(x); c.set_dout(dout)
+    if CB is None:
+        c.set_B(B); c.set_C(C)
     c.put("CB", CB, torch.float32); c.put("dt_out", dt, torch.float32)
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     nsl = max(1, min(4, nheads // ngroups // 32))      # head slices, added up in place by the kernel launcher

@@ -116,3 +116,38 @@ def test_forward_strided_inputs(ops):
                                           C.unflatten(-1, (G, N)), Q, D=d["D"], dt_bias=d["dt_bias"], dt_softplus=True)
     ref = O.bimamba2_quadratic(r["x"], r["dt"], r["A"], r["B"], r["C"], D=r["D"], dt_bias=r["dt_bias"], dt_softplus=True)[0]
     assert_close(out, ref, torch.float32, "out")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_stages_rebuild_cb_when_it_is_not_given(ops, dtype):
+    """The scan, dx and dCB stages called without CB (the way the composites call them at such shapes) agree with the
+    same stages reading the CB of the bmm stage.  Ragged last chunk (44 rows), two head groups."""
+    b, L, H, P, G, N, Q = 2, 300, 4, 64, 2, 64, 256
+    inp = make_case(b, L, H, P, G, N, dtype, with_z=True)
+    d = to_dev(inp)
+    csf, csb, dt_out = ops._chunk_cumsum_fwd(d["dt"], d["A"], Q, dt_bias=d["dt_bias"], dt_softplus=True)
+    CB = ops._bmm_chunk_fwd(d["C"], d["B"], Q)
+    sf, sb = ops._chunk_state_fwd(d["B"], d["x"], dt_out, csf, csb)
+    pf, pb, _, _ = ops._state_passing_fwd(sf, sb, csf, csb)
+    out1, outx1 = ops._chunk_scan_fwd(CB, d["x"], dt_out, csf, csb, d["C"], pf, pb, D=d["D"], z=d["z"])
+    out2, outx2 = ops._chunk_scan_fwd(None, d["x"], dt_out, csf, csb, d["C"], pf, pb, D=d["D"], z=d["z"], B=d["B"])
+    assert_close(outx2, outx1.double().cpu(), dtype, "out_x without CB")
+    assert_close(out2, out1.double().cpu(), dtype, "out without CB")
+    g = torch.Generator().manual_seed(11)
+    dout = torch.randn(d["x"].shape, generator=g).to(dtype).cuda()
+    dsf = torch.randn(pf.shape, generator=g).cuda() * 0.1
+    dsb = torch.randn(pf.shape, generator=g).cuda() * 0.1
+    dx1, ddt1, dD1 = ops._chunk_scan_chunk_state_bwd_dx(d["x"], dt_out, csf, csb, d["B"], CB, dout, dsf, dsb, D=d["D"])
+    dx2, ddt2, dD2 = ops._chunk_scan_chunk_state_bwd_dx(d["x"], dt_out, csf, csb, d["B"], None, dout, dsf, dsb, D=d["D"], C=d["C"])
+    assert_close(dx2, dx1.double().cpu(), dtype, "dx without CB")
+    # positions past the end of the sequence are not written by either path
+    valid = (torch.arange(ddt1.shape[2])[:, None] * Q + torch.arange(Q)[None, :] < L).to(ddt1.device)
+    assert_close(torch.where(valid, ddt2, 0.0), torch.where(valid, ddt1, 0.0).double().cpu(), dtype, "ddt_direct without CB")
+    assert_close(dD2, dD1.double().cpu(), dtype, "dD without CB")
+    dCB1, da1 = ops._chunk_scan_bwd_dcb(d["x"], dt_out, csf, csb, dout, CB, ngroups=G)
+    dCB2, da2 = ops._chunk_scan_bwd_dcb(d["x"], dt_out, csf, csb, dout, None, ngroups=G, B=d["B"], C=d["C"])
+    assert_close(dCB2, dCB1.double().cpu(), dtype, "dCB without CB")
+    assert_close(da2, da1.double().cpu(), dtype, "da_intra without CB")
+    # shapes whose kernels cannot rebuild CB refuse a missing CB instead of reading a null pointer
+    with pytest.raises(ValueError):
+        ops._chunk_scan_fwd(None, d["x"].float(), dt_out, csf, csb, d["C"].float(), pf, pb, B=d["B"].float())
