@@ -70,6 +70,46 @@ def stage_table(w, e, fused=(False, False, False)):
     }
 
 
+def rmsnorm_line(w, dtype, dev, reps):
+    """The layer's gated RMS norm at the workload's size (rows = batch * seqlen, cols = nheads * headdim): launch
+    durations of the forward and the backward entry point and their algorithmic HBM rates."""
+    import torch
+    from bi_mamba2_amd import layernorm_gated as LN
+    from bi_mamba2_amd._lib import load as _lib_load
+    rows, cols = w["batch"] * w["seqlen"], w["nheads"] * w["headdim"]
+    x = torch.randn(rows, cols, device=dev).to(dtype)
+    z = torch.randn(rows, cols, device=dev).to(dtype)
+    dy = torch.randn(rows, cols, device=dev).to(dtype)
+    wt = torch.ones(cols, device=dev)
+    e = x.element_size()
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(reps):
+            fn()
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) * 1e3 / reps
+
+    # one parameter block per direction, buffers allocated once: the loops below time launches, not the host wrapper
+    out, rstd = LN._layer_norm_fwd(x, wt, None, 1e-5, z=z)
+    pf = LN._params(x, z, wt, None, 1e-5, None, True)
+    pf.out, pf.out_rs, pf.rstd = out.data_ptr(), out.stride(0), rstd.data_ptr()
+    pb = LN._params(x, z, wt, None, 1e-5, None, True)
+    dx, dz, dw = torch.empty_like(x), torch.empty_like(x), torch.empty(cols, device=dev)
+    pb.dout, pb.dout_rs, pb.rstd = dy.data_ptr(), dy.stride(0), rstd.data_ptr()
+    pb.dx, pb.dx_rs, pb.dz, pb.dz_rs, pb.dweight = dx.data_ptr(), dx.stride(0), dz.data_ptr(), dz.stride(0), dw.data_ptr()
+    ws = torch.empty(max(int(_lib_load().bimamba2_rmsnorm_gated_workspace_bytes(ctypes.byref(pb))), 1), device=dev, dtype=torch.uint8)
+    pb.workspace, pb.workspace_bytes = ws.data_ptr(), ws.numel()
+    t_f = timed(lambda: LN._call("bimamba2_rmsnorm_gated_fwd", pf, x.device))
+    t_b = timed(lambda: LN._call("bimamba2_rmsnorm_gated_bwd", pb, x.device))
+    return {"rows": rows, "cols": cols, "fwd_us": round(t_f, 2), "bwd_us": round(t_b, 2),
+            "fwd_GBs": round(3 * e * rows * cols / t_f / 1e3, 1), "bwd_GBs": round(5 * e * rows * cols / t_b / 1e3, 1)}
+
+
 def whole_op_bytes(w, e, has_z):
     B, L, H, P, G, N = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate"))
     T4, T2, T1 = B * L * H * P, B * L * G * N, B * L * H
@@ -281,6 +321,7 @@ def main():
                      "sum_kernel_us": round(sum(k["us"] for k in kernels.values()), 1),
                      "measured_copy_GBs": round(copy_gbs, 1)},
         "kernels": kernels,
+        "gated_rmsnorm": rmsnorm_line(w, dtype, dev, max(10, args.steps)),
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w)

@@ -43,10 +43,23 @@ ENTRY_POINTS = (
     "bimamba2_chunk_scan_bwd_dx", "bimamba2_chunk_state_bwd_db", "bimamba2_chunk_scan_bwd_dc",
     "bimamba2_chunk_scan_bwd_dcb", "bimamba2_bmm_chunk_bwd", "bimamba2_chunk_cumsum_bwd",
 )
+NORM_ENTRY_POINTS = ("bimamba2_rmsnorm_gated_fwd", "bimamba2_rmsnorm_gated_bwd")
 ALL_SYMBOLS = ENTRY_POINTS + ("bimamba2_strerror", "bimamba2_version", "bimamba2_params_size",
-                              "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb")
+                              "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb", "bimamba2_norm_params_size",
+                              "bimamba2_rmsnorm_gated_workspace_bytes") + NORM_ENTRY_POINTS
 
 _lib = None
+
+
+class NormParams(ctypes.Structure):
+    """Mirror of ``struct bimamba2_norm_params`` (gated RMSNorm)."""
+    _fields_ = (
+        [("rows", _i64), ("cols", _i32), ("group_size", _i32), ("dtype", _i32), ("has_z", _i32), ("has_bias", _i32),
+         ("norm_before_gate", _i32), ("eps", _f32), ("reserved0", _i32)]
+        + [(n, _i64) for n in ("x_rs", "z_rs", "out_rs", "dout_rs", "dx_rs", "dz_rs")]
+        + [(n, _vp) for n in ("x", "z", "weight", "bias", "out", "rstd", "dout", "dx", "dz", "dweight", "dbias", "workspace")]
+        + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
+    )
 
 
 def load():
@@ -73,6 +86,15 @@ def load():
         raise RuntimeError("bimamba2_params layout mismatch between the library and its Python mirror")
     lib.bimamba2_workspace_bytes.argtypes = [ctypes.POINTER(Params), ctypes.c_int]
     lib.bimamba2_workspace_bytes.restype = ctypes.c_size_t
+    for name in NORM_ENTRY_POINTS:
+        fn = getattr(lib, name)
+        fn.argtypes = [ctypes.POINTER(NormParams)]
+        fn.restype = ctypes.c_int
+    lib.bimamba2_norm_params_size.restype = ctypes.c_size_t
+    if lib.bimamba2_norm_params_size() != ctypes.sizeof(NormParams):
+        raise RuntimeError("bimamba2_norm_params layout mismatch between the library and its Python mirror")
+    lib.bimamba2_rmsnorm_gated_workspace_bytes.argtypes = [ctypes.POINTER(NormParams)]
+    lib.bimamba2_rmsnorm_gated_workspace_bytes.restype = ctypes.c_size_t
     _lib = lib
     return lib
 

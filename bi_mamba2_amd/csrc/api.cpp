@@ -314,4 +314,36 @@ int bimamba2_bwd(const bimamba2_params *p) {
     return BIMAMBA2_OK;
 }
 
+size_t bimamba2_norm_params_size(void) { return sizeof(bimamba2_norm_params); }
+
+static int check_norm(const bimamba2_norm_params *p) {
+    if (!p) return BIMAMBA2_EINVAL;
+    if (p->rows < 0 || p->cols <= 0 || p->group_size <= 0 || p->cols % p->group_size) return BIMAMBA2_EINVAL;
+    if (p->dtype != BIMAMBA2_F32 && p->dtype != BIMAMBA2_BF16 && p->dtype != BIMAMBA2_F16) return BIMAMBA2_EUNSUPPORTED;
+    if (p->group_size > 8192) return BIMAMBA2_EUNSUPPORTED;
+    if (!p->x || !p->weight || (p->has_z && !p->z) || (p->has_bias && !p->bias)) return BIMAMBA2_EINVAL;
+    return BIMAMBA2_OK;
+}
+
+size_t bimamba2_rmsnorm_gated_workspace_bytes(const bimamba2_norm_params *p) {
+    if (check_norm(p)) return 0;
+    return norm_workspace_bytes(p);
+}
+
+int bimamba2_rmsnorm_gated_fwd(const bimamba2_norm_params *p) {
+    TRY(check_norm(p));
+    REQUIRE(p->out);
+    if (p->rows == 0) return BIMAMBA2_OK;
+    return launch_rmsnorm_gated(p, false);
+}
+
+int bimamba2_rmsnorm_gated_bwd(const bimamba2_norm_params *p) {
+    TRY(check_norm(p));
+    REQUIRE(p->dout); REQUIRE(p->rstd); REQUIRE(p->dx); REQUIRE(p->dweight);
+    if (p->has_z) REQUIRE(p->dz);
+    if (p->has_bias) REQUIRE(p->dbias);
+    if (!p->workspace || p->workspace_bytes < norm_workspace_bytes(p)) return BIMAMBA2_EWORKSPACE;
+    return launch_rmsnorm_gated(p, true);
+}
+
 }  // extern "C"

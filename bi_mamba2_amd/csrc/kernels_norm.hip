@@ -1,0 +1,343 @@
+// Gated RMSNorm for gfx950, forward and backward (the step right after the bidirectional SSD operator in the BiMamba2
+// layer):   xg = x            (norm_before_gate)   or  x * silu(z)
+//           y  = xg * rstd * weight (+ bias),  rstd = 1 / sqrt(mean_group(xg^2) + eps)
+//           out = y * silu(z) (norm_before_gate)   or  y
+// Math of rms_norm_ref (src/ssd/bi/layernorm_gated.py:18-39 of the reference); replaces its kernels
+// _layer_norm_fwd_1pass_kernel (:45-105) and _layer_norm_bwd_kernel (:155-268) for the RMS case.
+//
+// Pure HBM traffic: one wave owns one (row, group); lane l owns the 8-element pieces l, l + 64, ... of the group (16-byte
+// accesses when the rows allow it).  Forward keeps the group in registers between the two passes.  Backward re-reads it
+// (from cache) for its second pass and keeps only the weight-gradient partial sums in registers: a workgroup's four
+// waves stay on one group and walk over rows, each wave writes one partial row of dweight / dbias, and a fixed-order
+// reduction adds them up (no atomics).
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace bm2 {
+
+static inline hipStream_t stream_of(const bimamba2_norm_params *p) { return reinterpret_cast<hipStream_t>(p->stream); }
+
+// 8 consecutive elements as float; zero past `ncol` valid ones
+template <typename T> __device__ __forceinline__ void load8(const T *ptr, bool vec, int ncol, float (&v)[8]) {
+    if (vec && ncol >= 8) {
+        if constexpr (sizeof(T) == 2) {
+            const Vec16<T> raw = *reinterpret_cast<const Vec16<T> *>(ptr);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = to_f(raw.v[i]);
+        } else {
+            const f32x4 a = *reinterpret_cast<const f32x4 *>(ptr), b = *reinterpret_cast<const f32x4 *>(ptr + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[i + 4] = b[i]; }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = i < ncol ? to_f(ptr[i]) : 0.f;
+    }
+}
+template <typename T> __device__ __forceinline__ void store8(T *ptr, bool vec, int ncol, const float (&v)[8]) {
+    if (vec && ncol >= 8) {
+        if constexpr (sizeof(T) == 2) {
+            Vec16<T> o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o.v[i] = from_f<T>(v[i]);
+            *reinterpret_cast<Vec16<T> *>(ptr) = o;
+        } else {
+            *reinterpret_cast<f32x4 *>(ptr) = f32x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4 *>(ptr + 4) = f32x4{v[4], v[5], v[6], v[7]};
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (i < ncol) ptr[i] = from_f<T>(v[i]);
+    }
+}
+
+template <typename T, int NCH>
+__global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_fwd_kernel(const bimamba2_norm_params p, bool vec, bool wvec) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ngroups = p.cols / p.group_size, gs = p.group_size;
+    const int64_t item = (int64_t)blockIdx.x * 4 + wave;
+    if (item >= (int64_t)p.rows * ngroups) return;
+    const int g = (int)(item % ngroups);
+    const int64_t row = item / ngroups;
+    const T *x = reinterpret_cast<const T *>(p.x) + row * p.x_rs + g * gs;
+    const T *z = p.has_z ? reinterpret_cast<const T *>(p.z) + row * p.z_rs + g * gs : nullptr;
+    T *out = reinterpret_cast<T *>(p.out) + row * p.out_rs + g * gs;
+    const float *w = p.weight + g * gs, *bias = p.has_bias ? p.bias + g * gs : nullptr;
+    const bool gate_first = p.has_z && !p.norm_before_gate;
+    // both operands are requested before anything is reduced; z is kept as loaded between the passes
+    float xv[NCH][8];
+    T zk[NCH][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int c = (k * 64 + lane) * 8;
+        load8(x + c, vec, gs - c, xv[k]);
+        if (p.has_z) {
+            float zv[8];
+            load8(z + c, vec, gs - c, zv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (gate_first) xv[k][i] *= silu_f(zv[i]);
+                else zk[k][i] = from_f<T>(zv[i]);      // exact: zv came from a T
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < NCH; ++k)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += xv[k][i] * xv[k][i];
+    ss = wave_sum(ss);
+    const float rstd = 1.f / sqrtf(ss / gs + p.eps);
+    if (lane == 0 && p.rstd) p.rstd[item] = rstd;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int c = (k * 64 + lane) * 8;
+        if (c >= gs) continue;
+        float wv[8], yv[8];
+        load8(w + c, wvec, gs - c, wv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) yv[i] = xv[k][i] * rstd * wv[i];
+        if (bias) {
+            float bv[8];
+            load8(bias + c, wvec, gs - c, bv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) yv[i] += bv[i];
+        }
+        if (p.has_z && p.norm_before_gate) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) yv[i] *= silu_f(to_f(zk[k][i]));
+        }
+        store8(out + c, vec, gs - c, yv);
+    }
+}
+
+// d silu(z) / dz
+__device__ __forceinline__ float dsilu_f(float z) {
+    const float s = sigmoid_f(z);
+    return s * (1.f + z * (1.f - s));
+}
+
+// grid (row blocks, groups); wave w of workgroup bx handles rows bx*4 + w, + 4*gridDim.x, ...
+template <typename T, int NCH, bool HAS_BIAS>
+__global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimamba2_norm_params p, bool vec, bool wvec, float *part_w,
+                                                                     float *part_b) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ngroups = p.cols / p.group_size, gs = p.group_size;
+    const int g = blockIdx.y;
+    const float *w = p.weight + g * gs, *bias = HAS_BIAS ? p.bias + g * gs : nullptr;
+    const bool gate_first = p.has_z && !p.norm_before_gate, gate_last = p.has_z && p.norm_before_gate;
+    float dw[NCH][8], db[HAS_BIAS ? NCH : 1][8];
+#pragma unroll
+    for (int k = 0; k < NCH; ++k)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            dw[k][i] = 0.f;
+            if (HAS_BIAS) db[k][i] = 0.f;
+        }
+    for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < p.rows; row += (int64_t)gridDim.x * 4) {
+        const T *x = reinterpret_cast<const T *>(p.x) + row * p.x_rs + g * gs;
+        const T *z = p.has_z ? reinterpret_cast<const T *>(p.z) + row * p.z_rs + g * gs : nullptr;
+        const T *dout = reinterpret_cast<const T *>(p.dout) + row * p.dout_rs + g * gs;
+        T *dx = reinterpret_cast<T *>(p.dx) + row * p.dx_rs + g * gs;
+        T *dz = p.has_z ? reinterpret_cast<T *>(p.dz) + row * p.dz_rs + g * gs : nullptr;
+        const float rstd = p.rstd[row * ngroups + g];
+        // Per element: xhat = xg * rstd, wdy = weight * dy' (dy' = dy * silu(z) when the gate comes last), and for a gate
+        // that comes first sl = silu(z), g2 = x * dsilu(z).  Groups of up to 2048 columns keep them in registers between
+        // the two passes; wider ones read the row again (from cache) and recompute.
+        constexpr bool HOLD = NCH <= 4;
+        float xh[HOLD ? NCH : 1][8], wd[HOLD ? NCH : 1][8], sl[HOLD ? NCH : 1][8], g2[HOLD ? NCH : 1][8];
+        auto element = [&](int k, int c, bool first, float (&xhat)[8], float (&wdy)[8], float (&slv)[8], float (&g2v)[8]) {
+            float xv[8], dy[8], zv[8], wv[8], bv[8], dzv[8];
+            load8(x + c, vec, gs - c, xv);
+            load8(dout + c, vec, gs - c, dy);
+            load8(w + c, wvec, gs - c, wv);
+            if (HAS_BIAS && first) load8(bias + c, wvec, gs - c, bv);
+            if (p.has_z) load8(z + c, vec, gs - c, zv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float sg = 0.f, si = 1.f, ds = 0.f;
+                if (p.has_z) {
+                    sg = sigmoid_f(zv[i]);
+                    si = zv[i] * sg;
+                    ds = sg * (1.f + zv[i] * (1.f - sg));
+                }
+                slv[i] = si;
+                g2v[i] = xv[i] * ds;
+                xhat[i] = (gate_first ? xv[i] * si : xv[i]) * rstd;
+                if (gate_last) {
+                    dzv[i] = dy[i] * (xhat[i] * wv[i] + (HAS_BIAS && first ? bv[i] : 0.f)) * ds;
+                    dy[i] *= si;
+                }
+                wdy[i] = wv[i] * dy[i];
+                if (first) {
+                    dw[k][i] += dy[i] * xhat[i];
+                    if (HAS_BIAS) db[k][i] += dy[i];
+                }
+            }
+            if (gate_last && first) store8(dz + c, vec, gs - c, dzv);
+        };
+        // pass 1: c1 = mean(xhat * wdy), weight / bias gradients, and dz when the gate comes last
+        float c1 = 0.f;
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) {
+            const int c = (k * 64 + lane) * 8;
+            if (c >= gs) continue;
+            float xhat[8], wdy[8], slv[8], g2v[8];
+            element(k, c, true, xhat, wdy, slv, g2v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                c1 += xhat[i] * wdy[i];
+                if (HOLD) { xh[k][i] = xhat[i]; wd[k][i] = wdy[i]; sl[k][i] = slv[i]; g2[k][i] = g2v[i]; }
+            }
+        }
+        c1 = wave_sum(c1) / gs;
+        // pass 2: dx, and dz when the gate comes first
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) {
+            const int c = (k * 64 + lane) * 8;
+            if (c >= gs) continue;
+            float xhat[8], wdy[8], slv[8], g2v[8], dxv[8], dzv[8];
+            if (HOLD) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { xhat[i] = xh[k][i]; wdy[i] = wd[k][i]; slv[i] = sl[k][i]; g2v[i] = g2[k][i]; }
+            } else {
+                element(k, c, false, xhat, wdy, slv, g2v);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float dxg = (wdy[i] - xhat[i] * c1) * rstd;
+                dxv[i] = gate_first ? dxg * slv[i] : dxg;
+                dzv[i] = dxg * g2v[i];
+            }
+            store8(dx + c, vec, gs - c, dxv);
+            if (gate_first) store8(dz + c, vec, gs - c, dzv);
+        }
+    }
+    if constexpr (NCH <= 8) {
+        // the four waves add their sums in LDS (fixed order): one partial row per workgroup
+        __shared__ float red[3][NCH * 512];
+        for (int pass = 0; pass < (HAS_BIAS ? 2 : 1); ++pass) {
+            if (pass) __syncthreads();
+            if (wave > 0) {
+#pragma unroll
+                for (int k = 0; k < NCH; ++k)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) red[wave - 1][(k * 64 + lane) * 8 + i] = pass ? db[HAS_BIAS ? k : 0][i] : dw[k][i];
+            }
+            __syncthreads();
+            if (wave == 0) {
+                const int64_t prow = (int64_t)blockIdx.x * p.cols + g * gs;
+#pragma unroll
+                for (int k = 0; k < NCH; ++k) {
+                    const int c = (k * 64 + lane) * 8;
+                    if (c >= gs) continue;
+                    float v[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[i] = (pass ? db[HAS_BIAS ? k : 0][i] : dw[k][i]) + red[0][c + i] + red[1][c + i] + red[2][c + i];
+                    store8((pass ? part_b : part_w) + prow + c, false, gs - c, v);
+                }
+            }
+        }
+    } else {
+        // this wave's partial sums: row (blockIdx.x * 4 + wave) of the (gridDim.x * 4, cols) partial arrays
+        const int64_t prow = ((int64_t)blockIdx.x * 4 + wave) * p.cols + g * gs;
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) {
+            const int c = (k * 64 + lane) * 8;
+            if (c >= gs) continue;
+            store8(part_w + prow + c, false, gs - c, dw[k]);
+            if (HAS_BIAS) store8(part_b + prow + c, false, gs - c, db[k]);
+        }
+    }
+}
+
+// workgroups along the rows, and partial rows of dweight / dbias they leave (one per workgroup up to groups of 4096
+// columns, one per wave above)
+static int norm_row_blocks(const bimamba2_norm_params *p) { return (int)std::min<int64_t>((p->rows + 3) / 4, p->group_size <= 4096 ? 1024 : 256); }
+static int norm_partial_rows(const bimamba2_norm_params *p) { return norm_row_blocks(p) * (p->group_size <= 4096 ? 1 : 4); }
+
+size_t norm_workspace_bytes(const bimamba2_norm_params *p) {
+    return (size_t)norm_partial_rows(p) * p->cols * sizeof(float) * (p->has_bias ? 2 : 1);
+}
+
+// out[j] = sum_i in[i * nj + j] for many columns j: 16 columns x 16 row slices per workgroup, the slices added in a fixed
+// order; blockIdx.y selects one of up to two (in, out) pairs
+__global__ __launch_bounds__(NTHREADS) void colsum_kernel(const float *in0, float *out0, const float *in1, float *out1, int ni, int nj) {
+    __shared__ float red[16][17];
+    const float *in = blockIdx.y ? in1 : in0;
+    float *out = blockIdx.y ? out1 : out0;
+    const int jl = threadIdx.x & 15, sl = threadIdx.x >> 4, j = blockIdx.x * 16 + jl;
+    float s = 0.f;
+    if (j < nj) {
+        int i = sl;
+        for (; i + 48 < ni; i += 64) {
+            const float a = in[(int64_t)i * nj + j], b = in[(int64_t)(i + 16) * nj + j], c = in[(int64_t)(i + 32) * nj + j],
+                        d = in[(int64_t)(i + 48) * nj + j];
+            s += (a + b) + (c + d);
+        }
+        for (; i < ni; i += 16) s += in[(int64_t)i * nj + j];
+    }
+    red[sl][jl] = s;
+    __syncthreads();
+    if (sl == 0 && j < nj) {
+        float t = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) t += red[q][jl];
+        out[j] = t;
+    }
+}
+
+static bool norm_vec_ok(const bimamba2_norm_params *p, bool bwd, int elem) {
+    const int vs = 16 / elem;
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    bool ok = p->group_size % 8 == 0 && al(p->x) && p->x_rs % vs == 0 && (!p->has_z || (al(p->z) && p->z_rs % vs == 0));
+    if (!bwd) return ok && al(p->out) && p->out_rs % vs == 0;
+    return ok && al(p->dout) && p->dout_rs % vs == 0 && al(p->dx) && p->dx_rs % vs == 0 && (!p->has_z || (al(p->dz) && p->dz_rs % vs == 0));
+}
+
+template <typename T, int NCH>
+static int launch_norm_nch(const bimamba2_norm_params *p, bool bwd) {
+    const bool vec = norm_vec_ok(p, bwd, (int)sizeof(T));
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    const bool wvec = p->group_size % 4 == 0 && al(p->weight) && (!p->has_bias || al(p->bias));
+    if (!bwd) {
+        const int64_t items = (int64_t)p->rows * (p->cols / p->group_size);
+        hipLaunchKernelGGL((rmsnorm_gated_fwd_kernel<T, NCH>), dim3((unsigned)((items + 3) / 4)), dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec);
+        return check_launch();
+    }
+    const int nb = norm_row_blocks(p);
+    float *part_w = reinterpret_cast<float *>(p->workspace);
+    const int npr = norm_partial_rows(p);
+    float *part_b = p->has_bias ? part_w + (size_t)npr * p->cols : nullptr;
+    const dim3 grid(nb, p->cols / p->group_size);
+    if (p->has_bias) hipLaunchKernelGGL((rmsnorm_gated_bwd_kernel<T, NCH, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+    else hipLaunchKernelGGL((rmsnorm_gated_bwd_kernel<T, NCH, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+    int rc = check_launch();
+    if (rc) return rc;
+    hipLaunchKernelGGL(colsum_kernel, dim3((p->cols + 15) / 16, p->has_bias ? 2 : 1), dim3(NTHREADS), 0, stream_of(p), part_w, p->dweight,
+                       part_b, p->dbias, npr, p->cols);
+    return check_launch();
+}
+
+template <typename T>
+static int launch_norm_t(const bimamba2_norm_params *p, bool bwd) {
+    const int nch = (p->group_size + 511) / 512;
+    if (nch <= 1) return launch_norm_nch<T, 1>(p, bwd);
+    if (nch <= 2) return launch_norm_nch<T, 2>(p, bwd);
+    if (nch <= 4) return launch_norm_nch<T, 4>(p, bwd);
+    if (nch <= 8) return launch_norm_nch<T, 8>(p, bwd);
+    if (nch <= 16) return launch_norm_nch<T, 16>(p, bwd);
+    return BIMAMBA2_EUNSUPPORTED;
+}
+
+int launch_rmsnorm_gated(const bimamba2_norm_params *p, bool bwd) {
+    switch (p->dtype) {
+        case BIMAMBA2_F32: return launch_norm_t<float>(p, bwd);
+        case BIMAMBA2_BF16: return launch_norm_t<bf16_t>(p, bwd);
+        case BIMAMBA2_F16: return launch_norm_t<f16_t>(p, bwd);
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+}
+
+}  // namespace bm2

@@ -35,4 +35,8 @@ int launch_fill(float *ptr, size_t n, float value, hipStream_t stream);
 // out[j] = sum_{i<ni} sum_{k<nk} in[(i*nj + j)*nk + k]
 int launch_reduce(const float *in, float *out, int ni, int nj, int nk, hipStream_t stream);
 
+// gated RMSNorm (kernels_norm.hip)
+int launch_rmsnorm_gated(const bimamba2_norm_params *p, bool bwd);
+size_t norm_workspace_bytes(const bimamba2_norm_params *p);
+
 }  // namespace bm2

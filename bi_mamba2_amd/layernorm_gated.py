@@ -1,0 +1,148 @@
+"""Gated RMSNorm on the HIP kernels, with the reference's names (src/ssd/bi/layernorm_gated.py of Hprairie/Bi-Mamba2):
+``rmsnorm_fn`` (:383-384 there), the ``RMSNorm`` module (:415-437) and the autograd function behind them
+(``LayerNormFn``, :333-376, with is_rms_norm=True).
+
+    xg  = x                    if norm_before_gate else x * silu(z)
+    y   = xg / sqrt(mean_group(xg^2) + eps) * weight (+ bias)
+    out = y * silu(z)          if norm_before_gate else y
+
+There is no CPU or PyTorch fallback: CPU tensors raise, a missing library raises.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from .ops import _DT, _require_gpu
+
+
+def _rows(t, name):
+    _require_gpu(t, name)
+    t2 = t.reshape(-1, t.shape[-1])
+    if t2.stride(-1) != 1:
+        t2 = t2.contiguous()
+    return t2
+
+
+def _call(entry, p, device):
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        p.stream = torch.cuda.current_stream().cuda_stream
+        rc = getattr(lib, entry)(ctypes.byref(p))
+    if rc != 0:
+        msg = lib.bimamba2_strerror(rc).decode()
+        raise (ValueError if rc in (-1, -2) else RuntimeError)(f"{entry}: {msg} (code {rc})")
+
+
+def _params(x2, z2, weight, bias, eps, group_size, norm_before_gate):
+    if x2.dtype not in _DT:
+        raise ValueError(f"unsupported dtype {x2.dtype} (need float32, bfloat16 or float16)")
+    p = _lib.NormParams()
+    p.rows, p.cols = x2.shape
+    p.group_size = group_size if group_size is not None else x2.shape[1]
+    p.dtype = _DT[x2.dtype]
+    p.has_z, p.has_bias, p.norm_before_gate = int(z2 is not None), int(bias is not None), int(bool(norm_before_gate))
+    p.eps = float(eps)
+    p.x, p.x_rs = x2.data_ptr(), x2.stride(0)
+    if z2 is not None:
+        p.z, p.z_rs = z2.data_ptr(), z2.stride(0)
+    p.weight = weight.data_ptr()
+    if bias is not None:
+        p.bias = bias.data_ptr()
+    return p
+
+
+def _layer_norm_fwd(x, weight, bias, eps, z=None, group_size=None, norm_before_gate=True):
+    """x, z: (rows, cols) with unit stride along cols; weight, bias: (cols,) float32.  -> out, rstd (rows, ngroups)."""
+    rows, cols = x.shape
+    gs = group_size if group_size is not None else cols
+    assert cols % gs == 0
+    assert weight.shape == (cols,) and (bias is None or bias.shape == (cols,))
+    assert z is None or z.shape == x.shape
+    p = _params(x, z, weight, bias, eps, group_size, norm_before_gate)
+    out = torch.empty((rows, cols), device=x.device, dtype=x.dtype)
+    rstd = torch.empty((rows, cols // gs), device=x.device, dtype=torch.float32)
+    p.out, p.out_rs, p.rstd = out.data_ptr(), out.stride(0), rstd.data_ptr()
+    _call("bimamba2_rmsnorm_gated_fwd", p, x.device)
+    return out, rstd
+
+
+def _layer_norm_bwd(dy, x, weight, bias, eps, rstd, z=None, group_size=None, norm_before_gate=True):
+    """-> dx, dweight (float32), dbias (float32 or None), dz (or None)."""
+    p = _params(x, z, weight, bias, eps, group_size, norm_before_gate)
+    dx = torch.empty_like(x, memory_format=torch.contiguous_format)
+    dz = torch.empty_like(x, memory_format=torch.contiguous_format) if z is not None else None
+    dw = torch.empty((x.shape[1],), device=x.device, dtype=torch.float32)
+    db = torch.empty_like(dw) if bias is not None else None
+    p.dout, p.dout_rs, p.rstd = dy.data_ptr(), dy.stride(0), rstd.data_ptr()
+    p.dx, p.dx_rs, p.dweight = dx.data_ptr(), dx.stride(0), dw.data_ptr()
+    if dz is not None:
+        p.dz, p.dz_rs = dz.data_ptr(), dz.stride(0)
+    if db is not None:
+        p.dbias = db.data_ptr()
+    n = _lib.load().bimamba2_rmsnorm_gated_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty(max(int(n), 1), device=x.device, dtype=torch.uint8)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    _call("bimamba2_rmsnorm_gated_bwd", p, x.device)
+    return dx, dw, db, dz
+
+
+class LayerNormFn(torch.autograd.Function):
+    """RMS case of the reference's function of the same name (is_rms_norm is always True here)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True, is_rms_norm=True):
+        assert is_rms_norm, "only the RMS norm is built on the HIP kernels"
+        shape = x.shape
+        x2 = _rows(x, "x")
+        z2 = _rows(z, "z") if z is not None else None
+        if z2 is not None:
+            assert z.shape == shape
+            if z2.dtype != x2.dtype:
+                z2 = z2.to(x2.dtype)
+        w32 = weight.detach().float().contiguous()
+        b32 = bias.detach().float().contiguous() if bias is not None else None
+        _require_gpu(w32, "weight")
+        out, rstd = _layer_norm_fwd(x2, w32, b32, eps, z=z2, group_size=group_size, norm_before_gate=norm_before_gate)
+        ctx.save_for_backward(x2, w32, b32, rstd, z2)
+        ctx.shape, ctx.eps, ctx.group_size, ctx.norm_before_gate = shape, eps, group_size, norm_before_gate
+        ctx.wdtype = weight.dtype
+        ctx.bdtype = bias.dtype if bias is not None else None
+        ctx.zdtype = z.dtype if z is not None else None
+        return out.reshape(shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, w32, b32, rstd, z2 = ctx.saved_tensors
+        dy2 = _rows(dy, "dy")
+        if dy2.dtype != x2.dtype:
+            dy2 = dy2.to(x2.dtype)
+        dx, dw, db, dz = _layer_norm_bwd(dy2, x2, w32, b32, ctx.eps, rstd, z=z2, group_size=ctx.group_size,
+                                         norm_before_gate=ctx.norm_before_gate)
+        return (dx.reshape(ctx.shape), dw.to(ctx.wdtype), db.to(ctx.bdtype) if db is not None else None,
+                dz.reshape(ctx.shape).to(ctx.zdtype) if dz is not None else None, None, None, None, None)
+
+
+def rmsnorm_fn(x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True):
+    return LayerNormFn.apply(x, weight, bias, z, eps, group_size, norm_before_gate, True)
+
+
+class RMSNorm(torch.nn.Module):
+    """Same constructor, parameters and forward as the reference's module (no bias parameter)."""
+
+    def __init__(self, hidden_size, eps=1e-5, group_size=None, norm_before_gate=True, device=None, dtype=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = torch.nn.Parameter(torch.empty(hidden_size, device=device, dtype=dtype))
+        self.register_parameter("bias", None)
+        self.group_size = group_size
+        self.norm_before_gate = norm_before_gate
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        torch.nn.init.ones_(self.weight)
+
+    def forward(self, x, z=None):
+        """norm(x) * silu(z) if norm_before_gate, else norm(x * silu(z)); plain norm without z."""
+        return rmsnorm_fn(x, self.weight, self.bias, z=z, eps=self.eps, group_size=self.group_size,
+                          norm_before_gate=self.norm_before_gate)

@@ -4,7 +4,7 @@ Same constructor keywords, parameter names/shapes (so state_dicts interchange) a
 reference layer (src/ssd/modules.py:17-187): in_proj -> split [z | xBC | dt] -> softplus(dt + dt_bias) ->
 non-causal depthwise conv1d + SiLU -> split x, B, C -> bidirectional SSD with D -> gated RMSNorm(y, z) ->
 out_proj.  Parameters are created in the reference's order, so a seeded construction draws the same values.
-The projections, the convolution and the norm are ordinary torch ops; the SSD is the HIP operator.
+The projections and the convolution are ordinary torch ops; the SSD and the gated RMS norm are the HIP operators.
 """
 import math
 
@@ -12,36 +12,12 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from .layernorm_gated import RMSNorm
 from .ops import bimamba_chunk_scan_combined
 
 
-class RMSNormGated(nn.Module):
-    """RMSNorm over the last dim with an optional silu(z) gate, norm first then gate by default (the math of
-    the reference's ``rms_norm_ref``, src/ssd/bi/layernorm_gated.py:18-39), computed in float32."""
-
-    def __init__(self, hidden_size, eps=1e-5, group_size=None, norm_before_gate=True, device=None, dtype=None):
-        super().__init__()
-        self.eps = eps
-        self.weight = nn.Parameter(torch.ones(hidden_size, device=device, dtype=dtype))
-        self.register_parameter("bias", None)
-        self.group_size = group_size
-        self.norm_before_gate = norm_before_gate
-
-    def forward(self, x, z=None):
-        dtype = x.dtype
-        xf = x.float()
-        zf = z.float() if z is not None else None
-        if zf is not None and not self.norm_before_gate:
-            xf = xf * F.silu(zf)
-        if self.group_size is None:
-            y = xf * torch.rsqrt(xf.square().mean(-1, keepdim=True) + self.eps)
-        else:
-            xg = xf.unflatten(-1, (-1, self.group_size))
-            y = (xg * torch.rsqrt(xg.square().mean(-1, keepdim=True) + self.eps)).flatten(-2)
-        y = y * self.weight.float()
-        if zf is not None and self.norm_before_gate:
-            y = y * F.silu(zf)
-        return y.to(dtype)
+# the gated RMS norm of the layer runs on the HIP kernels (bi_mamba2_amd/layernorm_gated.py)
+RMSNormGated = RMSNorm
 
 
 class BiMamba2(nn.Module):

@@ -175,6 +175,40 @@ int bimamba2_bmm_chunk_bwd(const bimamba2_params *p);
  * scans (src/ssd/bi/ssd_combined.py:456-466) and _chunk_cumsum_bwd (src/ssd/bi/ssd_chunk_state.py:727-761). */
 int bimamba2_chunk_cumsum_bwd(const bimamba2_params *p);
 
+/* ---- gated RMSNorm (the step after the operator in the BiMamba2 layer) -------------------------------------
+ *   xg = x (norm_before_gate) or x * silu(z);  y = xg * rstd * weight (+ bias), rstd = 1/sqrt(mean_group(xg^2) + eps);
+ *   out = y * silu(z) (norm_before_gate) or y.
+ * Rows of `cols` elements (last dim contiguous, row strides in elements), groups of `group_size` consecutive columns
+ * (group_size divides cols, <= 8192).  Replaces rmsnorm_fn / RMSNorm of the reference, i.e. _layer_norm_fwd
+ * (src/ssd/bi/layernorm_gated.py:108-152, kernel :45-105) and _layer_norm_bwd (:271-330, kernel :155-268) with
+ * is_rms_norm = True; math of rms_norm_ref (:18-39). */
+typedef struct bimamba2_norm_params {
+    int64_t rows;
+    int32_t cols, group_size;
+    int32_t dtype;              /* BIMAMBA2_*: x, z, out, dout, dx, dz */
+    int32_t has_z, has_bias, norm_before_gate;
+    float eps;
+    int32_t reserved0;
+    int64_t x_rs, z_rs, out_rs, dout_rs, dx_rs, dz_rs;
+    const void *x, *z;
+    const float *weight, *bias; /* (cols,) float32 */
+    void *out;                  /* forward */
+    float *rstd;                /* (rows, cols / group_size) float32: written by the forward (optional there), read by the backward */
+    const void *dout;           /* backward */
+    void *dx, *dz;
+    float *dweight, *dbias;     /* (cols,) float32 */
+    void *workspace;            /* backward only: bimamba2_rmsnorm_gated_workspace_bytes() */
+    size_t workspace_bytes;
+    void *stream;               /* hipStream_t */
+} bimamba2_norm_params;
+
+size_t bimamba2_norm_params_size(void);
+size_t bimamba2_rmsnorm_gated_workspace_bytes(const bimamba2_norm_params *p);
+/* x [z] weight [bias] -> out, rstd */
+int bimamba2_rmsnorm_gated_fwd(const bimamba2_norm_params *p);
+/* x [z] weight [bias] rstd dout -> dx [dz] dweight [dbias] */
+int bimamba2_rmsnorm_gated_bwd(const bimamba2_norm_params *p);
+
 #ifdef __cplusplus
 }
 #endif

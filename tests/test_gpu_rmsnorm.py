@@ -1,0 +1,68 @@
+"""GPU parity of the gated RMS norm (forward and backward, through the C ABI) against the float64 oracle."""
+import pytest
+import torch
+
+from oracle.rmsnorm_oracle import rms_norm_gated
+from tests.helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # shape, group_size, z, bias, norm_before_gate, dtype
+    ((2, 37, 256), None, True, False, True, torch.float32),      # the BiMamba2 layer's configuration
+    ((2, 37, 256), None, True, False, False, torch.float32),
+    ((3, 5, 192), 64, True, True, True, torch.float32),          # groups + bias
+    ((3, 5, 192), 64, False, False, True, torch.float32),        # no gate
+    ((4, 100), None, True, False, True, torch.float32),          # width not a multiple of 8: scalar accesses
+    ((2, 64, 2048), None, True, False, True, torch.bfloat16),    # the benchmark layer's width
+    ((2, 64, 2048), 512, True, True, False, torch.bfloat16),
+    ((8, 4096), None, True, False, True, torch.float16),
+    ((3, 8192), None, False, False, True, torch.bfloat16),       # the widest supported group
+    ((600, 2, 128), None, True, True, True, torch.float32),      # more rows than partial-sum slots
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_rmsnorm_gated_forward_backward(case):
+    from bi_mamba2_amd.layernorm_gated import rmsnorm_fn
+    shape, gs, with_z, with_b, before, dtype = case
+    g = torch.Generator().manual_seed(3)
+    n = shape[-1]
+    x = torch.randn(shape, generator=g).to(dtype)
+    z = torch.randn(shape, generator=g).to(dtype) if with_z else None
+    w = (1.0 + 0.3 * torch.randn(n, generator=g)).float()
+    b = (0.2 * torch.randn(n, generator=g)).float() if with_b else None
+    dy = torch.randn(shape, generator=g).to(dtype)
+    leaves = [t.cuda().requires_grad_(True) if t is not None else None for t in (x, w, b, z)]
+    out = rmsnorm_fn(leaves[0], leaves[1], leaves[2], z=leaves[3], eps=1e-5, group_size=gs, norm_before_gate=before)
+    assert out.dtype == dtype and out.shape == tuple(shape)
+    out.backward(dy.cuda())
+    ref_leaves = [t.double().requires_grad_(True) if t is not None else None for t in (x, w, b, z)]
+    ref = rms_norm_gated(ref_leaves[0], ref_leaves[1], ref_leaves[2], ref_leaves[3], eps=1e-5, group_size=gs, norm_before_gate=before)
+    ref.backward(dy.double())
+    assert_close(out, ref.detach(), dtype, "out")
+    for got, r, name in zip(leaves, ref_leaves, ("dx", "dweight", "dbias", "dz")):
+        if r is not None:
+            assert_close(got.grad, r.grad, dtype, name)
+
+
+def test_rmsnorm_strided_rows_and_module():
+    """Rows that are views into a wider projection output (as in the layer), and the module with its parameter."""
+    from bi_mamba2_amd.layernorm_gated import RMSNorm
+    g = torch.Generator().manual_seed(5)
+    wide = torch.randn(2, 33, 3 * 128, generator=g).cuda()
+    x, z = wide[..., :128], wide[..., 256:]
+    m = RMSNorm(128, eps=1e-5, norm_before_gate=True, device="cuda")
+    with torch.no_grad():
+        m.weight.copy_(1.0 + 0.1 * torch.randn(128, generator=g))
+    out = m(x, z)
+    ref = rms_norm_gated(x.double().cpu(), m.weight.detach().double().cpu(), None, z.double().cpu(), eps=1e-5)
+    assert_close(out, ref, torch.float32, "out (strided)")
+
+
+def test_rmsnorm_refuses_cpu_tensors_and_bad_groups():
+    from bi_mamba2_amd.layernorm_gated import rmsnorm_fn
+    with pytest.raises(RuntimeError):
+        rmsnorm_fn(torch.randn(4, 64), torch.ones(64), None)
+    with pytest.raises((ValueError, AssertionError)):
+        rmsnorm_fn(torch.randn(4, 64).cuda(), torch.ones(64).cuda(), None, group_size=48)
