@@ -403,8 +403,10 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_p
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    // unconditional loads from clamped addresses (conditional ones are waited for one by one), masked after
                     const int n = nt * 64 + j * 16 + lr;
-                    creg[nt][q][j][i] = (r0 + tl[q][i] < limit && n < N) ? to_f(cbp[(int64_t)tl[q][i] * cbs + n]) : 0.f;
+                    const float v = to_f(cbp[(int64_t)min(tl[q][i], limit - 1 - r0) * cbs + min(n, N - 1)]);
+                    creg[nt][q][j][i] = (r0 + tl[q][i] < limit && n < N) ? v : 0.f;
                 }
     f32x4 tot[NT][QT][4] = {};
 
