@@ -234,15 +234,25 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
             const float A = p.A[h];
             const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
             const int64_t dto = b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
-            float v[4], a[4];
+            float v[4], a[4], raw[4];
+            int64_t at[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) at[e] = dto + (int64_t)min(lane * 4 + e, limit - 1) * p.dt_sl;
+            // one branch on the type around all four loads, so that they go out together
+            if (p.dt_dtype == BIMAMBA2_F32) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) raw[e] = reinterpret_cast<const float *>(p.dt)[at[e]];
+            } else if (p.dt_dtype == BIMAMBA2_BF16) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) raw[e] = to_f(reinterpret_cast<const bf16_t *>(p.dt)[at[e]]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) raw[e] = to_f(reinterpret_cast<const f16_t *>(p.dt)[at[e]]);
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int q = lane * 4 + e;
-                const int64_t at = dto + (int64_t)min(q, limit - 1) * p.dt_sl;
-                float d = p.dt_dtype == BIMAMBA2_F32 ? reinterpret_cast<const float *>(p.dt)[at]
-                        : p.dt_dtype == BIMAMBA2_BF16 ? to_f(reinterpret_cast<const bf16_t *>(p.dt)[at])
-                                                      : to_f(reinterpret_cast<const f16_t *>(p.dt)[at]);
-                d += bias;
+                float d = raw[e] + bias;
                 if (p.dt_softplus) d = d > 20.f ? d : log1pf(expf(d));
                 d = fminf(fmaxf(d, p.dt_min), p.dt_max);
                 if (q >= limit) d = 0.f;
