@@ -195,8 +195,28 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             // raw rows as the A operand; the row factors go onto the accumulators (rows 4*(l/16)+i of each tile).
             // One direction after the other, to keep one set of temporaries.
             static_assert(NF == 0 || NF * KSTEP == NW, "one round of state tiles");
-            tile_load_kcontig<T, float, PW, NW>(sF, stf, N, P - p0, N, Ident());
-            tile_load_kcontig<T, float, PW, NW>(sB, stb, N, P - p0, N, Ident());
+            // full 64 x 64 float tiles (the launcher checked it): every 16-byte load of both tiles goes out
+            // before the first one is converted
+            {
+                constexpr int PER = PW * NW / 4 / SCAN_THREADS;
+                float4 rawf[PER], rawb[PER];
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
+                    const int idx = threadIdx.x + i * SCAN_THREADS;
+                    rawf[i] = *reinterpret_cast<const float4 *>(stf + idx * 4);
+                    rawb[i] = *reinterpret_cast<const float4 *>(stb + idx * 4);
+                }
+                struct alignas(sizeof(T) * 4) Out { T v[4]; };
+#pragma unroll
+                for (int i = 0; i < PER; ++i) {
+                    const int idx = threadIdx.x + i * SCAN_THREADS, r = idx / (NW / 4), k0 = (idx % (NW / 4)) * 4;
+                    Out of, ob;
+                    of.v[0] = from_f<T>(rawf[i].x); of.v[1] = from_f<T>(rawf[i].y); of.v[2] = from_f<T>(rawf[i].z); of.v[3] = from_f<T>(rawf[i].w);
+                    ob.v[0] = from_f<T>(rawb[i].x); ob.v[1] = from_f<T>(rawb[i].y); ob.v[2] = from_f<T>(rawb[i].z); ob.v[3] = from_f<T>(rawb[i].w);
+                    *reinterpret_cast<Out *>(sF + r * LDS_ + k0) = of;
+                    *reinterpret_cast<Out *>(sB + r * LDS_ + k0) = ob;
+                }
+            }
             __syncthreads();
             TSTAMP(2)
 #pragma unroll
@@ -627,6 +647,7 @@ bool scan_recomputes_cb(const bimamba2_params *p, bool bwd) {
     if (p->dtype == BIMAMBA2_F32 || p->dstate != 64 || scan_col_tile(p) != 64) return false;
     auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
     if (p->B_sl <= 0 || p->C_sl <= 0 || p->B_sl > (1 << 21) || p->C_sl > (1 << 21)) return false;   // 256 rows in 32-bit byte offsets
+    if (!(bwd ? al16(p->dstates_f) && al16(p->dstates_b) : al16(p->states_f) && al16(p->states_b))) return false;
     return scan_fast(p, bwd, 64, 8) && al16(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al16(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg);
 }
 
