@@ -1255,7 +1255,9 @@ int launch_bwd_dcb(const bimamba2_params *p) {
 // One workgroup: 64 rows x 64 dstate columns of one (b, c, g).  The K operand (C or B rows of the chunk) is staged
 // transposed in LDS once; the A operand is read from the float32 dCB / dCBT rows straight into MFMA operand layout.
 // =========================================================================================================
-template <typename T, int QP>
+// FAST (16-bit types, chunk_size == QP, dstate a multiple of 64, aligned operands, at most 8 slices): every global load
+// of a thread (its dCB row pieces, the slices it adds, the K operand) is requested before the first one is used.
+template <typename T, int QP, bool FAST>
 __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_params p, int nc, int nslices) {
     typedef Mma<T> M;
     constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
@@ -1273,9 +1275,77 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
     int64_t os;
     if (which == 0) { os = p.C_sl; op = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * os + g * p.C_sg + nt * 64; }
     else { os = p.B_sl; op = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * os + g * p.B_sg + nt * 64; }
+    const float *arow = (which == 0 ? p.dCBT : p.dCB) + (int64_t)bcg * Q * Q + (int64_t)min(r0 + wave * 16 + lr, Q - 1) * Q;
+    const float *res = which == 0 ? p.dBs : p.dCs;
+    T *out = reinterpret_cast<T *>(which == 0 ? p.dB : p.dC);
+    const int64_t slice = (int64_t)p.batch * p.seqlen * p.ngroups * N;
+    constexpr int VS = 16 / (int)sizeof(T), SLD = 64 + 4;
+    __shared__ __attribute__((aligned(16))) float stg[64 * SLD];
+    if constexpr (FAST) {
+        constexpr int NS = QP / KSTEP, NIT = 64 * (64 / VS) / NTHREADS, MAXSL = 8;
+        float4 raw[NS][2];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            raw[s][0] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL);
+            raw[s][1] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL + 4);
+        }
+        float4 sv[NIT][MAXSL][2];
+        int64_t oa[NIT];
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int id = threadIdx.x + it * NTHREADS;
+            const int rl = id / (64 / VS), cc = (id % (64 / VS)) * VS;
+            const int r = min(r0 + rl, limit - 1);
+            oa[it] = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + nt * 64 + cc;
+#pragma unroll
+            for (int sl = 0; sl < MAXSL; ++sl) {
+                const float *q = res + oa[it] + (int64_t)min(sl, nslices - 1) * slice;
+                sv[it][sl][0] = *reinterpret_cast<const float4 *>(q);
+                sv[it][sl][1] = *reinterpret_cast<const float4 *>(q + 4);
+            }
+        }
+        stage_transposed<T, QP, 64, LDX, true>(kT, op, os, limit, 64, [&](int k) { return k < limit ? 1.f : 0.f; });
+        __syncthreads();
+        f32x4 acc[4] = {};
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            if (s * KSTEP < limit) {
+                float v[KPL] = {raw[s][0].x, raw[s][0].y, raw[s][0].z, raw[s][0].w, raw[s][1].x, raw[s][1].y, raw[s][1].z, raw[s][1].w};
+                const typename M::Frag af = M::pack(v);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = M::mma(af, M::load(kT + xt_index<T, LDX>(j * 16 + lr, s * KSTEP + lg * KPL)), acc[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) stg[(wave * 16 + lg * 4 + i) * SLD + j * 16 + lr] = acc[j][i];
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int id = threadIdx.x + it * NTHREADS;
+            const int rl = id / (64 / VS), cc = (id % (64 / VS)) * VS;
+            float v[VS];
+#pragma unroll
+            for (int i = 0; i < VS; ++i) v[i] = stg[rl * SLD + cc + i];
+#pragma unroll
+            for (int sl = 0; sl < MAXSL; ++sl) {
+                if (sl < nslices) {
+                    v[0] += sv[it][sl][0].x; v[1] += sv[it][sl][0].y; v[2] += sv[it][sl][0].z; v[3] += sv[it][sl][0].w;
+                    v[4] += sv[it][sl][1].x; v[5] += sv[it][sl][1].y; v[6] += sv[it][sl][1].z; v[7] += sv[it][sl][1].w;
+                }
+            }
+            if (r0 + rl < limit) {
+                Vec16<T> ov;
+#pragma unroll
+                for (int i = 0; i < VS; ++i) ov.v[i] = from_f<T>(v[i]);
+                *reinterpret_cast<Vec16<T> *>(out + oa[it]) = ov;
+            }
+        }
+        return;
+    }
     stage_transposed<T, QP, 64, LDX, false>(kT, op, os, limit, N - nt * 64, [&](int k) { return 1.f; });
     __syncthreads();
-    const float *arow = (which == 0 ? p.dCBT : p.dCB) + (int64_t)bcg * Q * Q + (int64_t)min(r0 + wave * 16 + lr, Q - 1) * Q;
     const bool cvec = Q % 4 == 0;
     f32x4 acc[4] = {};
     for (int k0 = 0; k0 < limit; k0 += KSTEP) {
@@ -1299,13 +1369,8 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = M::mma(af, M::load(kT + xt_index<T, LDX>(j * 16 + lr, kb)), acc[j]);
     }
-    const float *res = which == 0 ? p.dBs : p.dCs;
-    T *out = reinterpret_cast<T *>(which == 0 ? p.dB : p.dC);
-    const int64_t slice = (int64_t)p.batch * p.seqlen * p.ngroups * N;
     // pass the tile through LDS so that the slices are read and the result is written
     // as 16-byte vectors along dstate
-    constexpr int VS = 16 / (int)sizeof(T), SLD = 64 + 4;
-    __shared__ __attribute__((aligned(16))) float stg[64 * SLD];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -1345,11 +1410,24 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
 
 template <typename T>
 static int launch_bmm_bwd_t(const bimamba2_params *p) {
-    const int nc = nchunks(p), Q = p->chunk_size;
+    const int nc = nchunks(p), Q = p->chunk_size, nsl = dbdc_slices(p);
     dim3 grid((p->dstate + 63) / 64, (Q + 63) / 64, p->batch * nc * p->ngroups * 2);
-    if (Q <= 64) hipLaunchKernelGGL((bmm_chunk_bwd_kernel<T, 64>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p));
-    else if (Q <= 128) hipLaunchKernelGGL((bmm_chunk_bwd_kernel<T, 128>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p));
-    else hipLaunchKernelGGL((bmm_chunk_bwd_kernel<T, 256>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, dbdc_slices(p));
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
+    const bool fast = sizeof(T) == 2 && (Q == 64 || Q == 128 || Q == 256) && p->dstate % 64 == 0 && nsl <= 8 && al(p->Bm) && al(p->Cm)
+                      && mult(p->B_sb, p->B_sl, p->B_sg) && mult(p->C_sb, p->C_sl, p->C_sg) && al(p->dCB) && al(p->dCBT) && al(p->dBs)
+                      && al(p->dCs) && al(p->dB) && al(p->dC);
+#define BM2_BMMB(QPV)                                                                                                              \
+    do {                                                                                                                       \
+        if constexpr (sizeof(T) == 2) {                                                                                        \
+            if (fast) { hipLaunchKernelGGL((bmm_chunk_bwd_kernel<T, QPV, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl); break; } \
+        }                                                                                                                      \
+        hipLaunchKernelGGL((bmm_chunk_bwd_kernel<T, QPV, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl);          \
+    } while (0)
+    if (Q <= 64) BM2_BMMB(64);
+    else if (Q <= 128) BM2_BMMB(128);
+    else BM2_BMMB(256);
+#undef BM2_BMMB
     return check_launch();
 }
 
