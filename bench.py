@@ -200,10 +200,20 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / n
 
+    def causal_step():
+        out = ops.causal_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"],
+                                             w["chunk_size"], D=leaves["D"], z=leaves["z"], dt_bias=leaves["dt_bias"],
+                                             dt_softplus=True)
+        torch.autograd.grad(out, grad_inputs, dout)
+
     for _ in range(args.warmup):
         step()
     t_step = timed(step, args.steps)
     t_fwd = timed(fwd_only, args.steps)
+    # the single-direction comparator: the same kernels with the reverse direction left out, same shape, same run
+    for _ in range(args.warmup):
+        causal_step()
+    t_causal = timed(causal_step, args.steps)
     tokens = w["batch"] * w["seqlen"]
     fwd_b, bwd_b = whole_op_bytes(w, e, has_z)
 
@@ -320,6 +330,10 @@ def main():
                      "fwd_hbm_frac": fwd_b / t_fwd / (HBM_PEAK_GBS * 1e9),
                      "sum_kernel_us": round(sum(k["us"] for k in kernels.values()), 1),
                      "measured_copy_GBs": round(copy_gbs, 1)},
+        "causal_comparator": {"ms_per_step": t_causal * 1e3, "Mtokens_s": tokens / t_causal / 1e6,
+                              "bidirectional_over_causal": t_step / t_causal,
+                              "what": "single-direction SSD (y = SS(x) + D x, z gate) forward + backward from the same "
+                                      "kernels with the reverse direction compiled out, same shape and dtypes"},
         "kernels": kernels,
         "gated_rmsnorm": rmsnorm_line(w, dtype, dev, max(10, args.steps)),
     }

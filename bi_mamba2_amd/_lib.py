@@ -20,7 +20,7 @@ class Params(ctypes.Structure):
     _fields_ = (
         [(n, _i32) for n in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate", "chunk_size",
                              "dtype", "dt_dtype", "has_D", "D_has_hdim", "has_z", "has_dt_bias", "dt_softplus",
-                             "fwd_saved", "reserved0")]
+                             "fwd_saved", "causal")]
         + [("dt_min", _f32), ("dt_max", _f32)]
         + [(n, _i64) for n in ("x_sb", "x_sl", "x_sh", "z_sb", "z_sl", "z_sh", "dout_sb", "dout_sl", "dout_sh",
                                "B_sb", "B_sl", "B_sg", "C_sb", "C_sl", "C_sg", "dt_sb", "dt_sl", "dt_sh")]

@@ -253,6 +253,7 @@ static int forward_cumsum_and_states(const bimamba2_params *q) {
 
 int bimamba2_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
+    if (p->causal && p->final_b) return BIMAMBA2_EINVAL;
     bimamba2_params q = *p;
     const size_t need = carve(&q, 0, p->workspace);
     if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;

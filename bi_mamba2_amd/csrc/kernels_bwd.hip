@@ -194,10 +194,10 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_kernel(const bimam
 // flight before the first of them is used: the recurrence is a chain over the chunks, and a global access that has to be
 // waited for at every link costs microseconds.  Needs P*N % 4 == 0 and 16-byte aligned tensors.
 constexpr int SP_CH = 8;
-__global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const bimamba2_params p, int nc, int nsplit) {
+__global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const bimamba2_params p, int nc, int nsplit, int ndir) {
     __shared__ float red[SP_CH][4];
     const int PN = p.headdim * p.dstate;
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z >> 1, dir = blockIdx.z & 1;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z / ndir, dir = blockIdx.z % ndir;   // ndir = 1: forward direction only
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int Q = p.chunk_size;
     const float *cs = (dir == 0 ? p.cs_f : p.cs_b) + ((int64_t)b * p.nheads + h) * nc * Q + (dir == 0 ? Q - 1 : 0);
@@ -250,11 +250,13 @@ int launch_state_passing_bwd(const bimamba2_params *p) {
     const int nc = nchunks(p), PN = p->headdim * p->dstate;
     const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS);
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    const int ndir = p->causal ? 1 : 2;
     if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->dstates_f) && al(p->dstates_b)) {
-        dim3 grid(nsplit, p->nheads, p->batch * 2);
-        hipLaunchKernelGGL(state_passing_bwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit);
+        dim3 grid(nsplit, p->nheads, p->batch * ndir);
+        hipLaunchKernelGGL(state_passing_bwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit, ndir);
         return check_launch();
     }
+    if (p->causal) return BIMAMBA2_EUNSUPPORTED;
     dim3 grid(nsplit, p->nheads, p->batch);
     hipLaunchKernelGGL(state_passing_bwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit);
     return check_launch();
@@ -280,7 +282,8 @@ constexpr int DBDC_WAVES = 8, DBDC_THREADS = 64 * DBDC_WAVES;
 // each state once.  Global memory latency is hidden by software pipelining over "steps" (head, dstate tile, headdim
 // chunk): the state blocks and A fragments of step s+1 are requested into registers before step s is multiplied, and
 // only then written to the LDS image.
-template <typename T, int NT, int QT, bool IS_DB, bool FAST>
+// UNI: the forward direction's state only (single-direction comparator).
+template <typename T, int NT, int QT, bool IS_DB, bool FAST, bool UNI = false>
 __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_params p, int nc) {
     typedef Mma<T> M;
     constexpr int KPL = M::KPL, KSTEP = M::KSTEP, KC = 64, NKS = KC / KSTEP;
@@ -319,7 +322,7 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_p
     auto request = [&](int step) __attribute__((always_inline)) {
         const int hh = hh0 + step / per_head, rem = step % per_head, nt = rem / nkc, kc = rem % nkc;
         const int h = g * hpg + hh;
-        if (stile < 2) {
+        if (stile < (UNI ? 1 : 2)) {
             const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * N;
             const float *st = (IS_DB ? (stile ? p.dstates_b : p.dstates_f) : (stile ? p.states_b : p.states_f)) + so;
 #pragma unroll
@@ -353,7 +356,7 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_p
     };
     // stage 2: the requested state block goes, transposed, into the LDS image (r = n, k = p)
     auto commit = [&](int buf) __attribute__((always_inline)) {
-        if (stile < 2) {
+        if (stile < (UNI ? 1 : 2)) {
             T *dst = stile ? sB[buf] : sF[buf];
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
@@ -380,10 +383,10 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_p
             if (IS_DB) {
                 const float d = p.dt_out[o + r];
                 f = d * __expf(p.cs_f[o + Q - 1] - p.cs_f[o + r]);
-                rv = d * __expf(p.cs_b[o] - p.cs_b[o + r]);
+                rv = UNI ? 0.f : d * __expf(p.cs_b[o] - p.cs_b[o + r]);
             } else {
                 f = __expf(p.cs_f[o + r]);
-                rv = __expf(p.cs_b[o + r]);
+                rv = UNI ? 0.f : __expf(p.cs_b[o + r]);
             }
         }
         sfs[hh][rl] = f;
@@ -440,11 +443,11 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_p
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const typename M::Frag bff = M::load(sF[buf] + xt_index<T, LDX>(j * 16 + lr, kq));
-                        const typename M::Frag bfb = M::load(sB[buf] + xt_index<T, LDX>(j * 16 + lr, kq));
+                        const typename M::Frag bfb = UNI ? bff : M::load(sB[buf] + xt_index<T, LDX>(j * 16 + lr, kq));
 #pragma unroll
                         for (int q = 0; q < QT; ++q) {
                             tf[q][j] = M::mma(afc[q][ks], bff, tf[q][j]);
-                            tb[q][j] = M::mma(afc[q][ks], bfb, tb[q][j]);
+                            if (!UNI) tb[q][j] = M::mma(afc[q][ks], bfb, tb[q][j]);
                         }
                     }
                 }
@@ -470,7 +473,7 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_p
                 const float a = row16_sum(uf[q][i]) * sfs[hh - hh0][tl[q][i]], bb = row16_sum(ub[q][i]) * sbs[hh - hh0][tl[q][i]];
                 if (lr == 0 && r0 + tl[q][i] < Q) {
                     of[o + r0 + tl[q][i]] = a;
-                    ob[o + r0 + tl[q][i]] = bb;
+                    if (!UNI) ob[o + r0 + tl[q][i]] = bb;
                 }
             }
     }
@@ -506,6 +509,16 @@ static int launch_dbdc_t(const bimamba2_params *p) {
         if (fast) hipLaunchKernelGGL((bwd_dbdc_kernel<T, NTV, QTV, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc); \
         else hipLaunchKernelGGL((bwd_dbdc_kernel<T, NTV, QTV, IS_DB, false>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);     \
     } while (0)
+    if (p->causal) {
+        if constexpr (sizeof(T) == 2) {
+            if (fast && nt == 1) {
+                if (qt == 2) hipLaunchKernelGGL((bwd_dbdc_kernel<T, 1, 2, IS_DB, true, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
+                else hipLaunchKernelGGL((bwd_dbdc_kernel<T, 1, 1, IS_DB, true, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
+                return check_launch();
+            }
+        }
+        return BIMAMBA2_EUNSUPPORTED;
+    }
     if (nt == 1 && qt == 2) BM2_DBDC(1, 2);
     else if (nt == 1) BM2_DBDC(1, 1);
     else if (nt == 2) BM2_DBDC(2, 1);
@@ -860,7 +873,8 @@ constexpr int DCB_PART_B = 10 * 64 * 4;
 #define TSR(k)
 #endif
 
-template <typename T>
+// UNI: the single-direction operator - tiles above the diagonal are empty, tiles on it keep the forward half.
+template <typename T, bool UNI = false>
 __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_params p, int nc, int nqt) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
@@ -883,7 +897,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
     const int Q = p.chunk_size, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
     const int limit = min(Q, p.seqlen - c * Q);
     const int t0 = tt * 64, s0 = st * 64;
-    const bool live = t0 < limit && s0 < limit;
+    const bool live = t0 < limit && s0 < limit && !(UNI && st > tt);
     const int trow = wave * 16 + lg * 4;                       // first of this lane's four accumulator rows
     f32x4 cbr[4] = {}, dcb[4] = {};
     const int hps = (hpg + gridDim.z - 1) / gridDim.z;
@@ -1086,7 +1100,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         if (j < wave) { sep_block(j, Ef, dts[j] * __expf(mf - cfs[j]), colF[j], rpf); }
-                        else if (j > wave) { colF[j] = 0.f; sep_block(j, Eb, dts[j] * __expf(mb - cbs[j]), colB[j], rpb); }
+                        else if (j > wave) { colF[j] = 0.f; if (!UNI) sep_block(j, Eb, dts[j] * __expf(mb - cbs[j]), colB[j], rpb); }
                         else {
                             // the block on the diagonal: both directions, masked element by element
                             float ca = 0.f, cb2 = 0.f;
@@ -1095,7 +1109,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
                                 const int ti = lg * 4 + i;     // row and column (lr) inside the block
                                 const float gv = acc[j][i] * dts[j];
                                 const float f = (lr <= ti) ? gv * __expf(cft_[i] - cfs[j]) : 0.f;
-                                const float r = (lr >= ti) ? gv * __expf(cbt_[i] - cbs[j]) : 0.f;
+                                const float r = (!UNI && lr >= ti) ? gv * __expf(cbt_[i] - cbs[j]) : 0.f;
                                 dcb[j][i] += f + r;
                                 const float wf = (lr < ti) ? f * cbr[j][i] : 0.f;
                                 const float wb = (lr > ti) ? r * cbr[j][i] : 0.f;
@@ -1203,7 +1217,10 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
 }
 
 template <typename T> static void launch_dcb_ring(dim3 grid, const bimamba2_params *p, int nc, int nqt) {
-    if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((bwd_dcb_ring_kernel<T>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
+    if constexpr (sizeof(T) == 2) {
+        if (p->causal) hipLaunchKernelGGL((bwd_dcb_ring_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
+        else hipLaunchKernelGGL((bwd_dcb_ring_kernel<T>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
+    }
 }
 
 // whether the dCB kernel can do without CB (it rebuilds its tile from the C and B rows): the 16-bit ring variant, dstate a
@@ -1227,6 +1244,7 @@ static int launch_dcb_t(const bimamba2_params *p) {
     bool fast = p->headdim % (sizeof(T) == 2 ? 64 : 16) == 0 && al(p->x) && p->x_sb % VS == 0 && p->x_sl % VS == 0 && p->x_sh % VS == 0;
     fast = fast && (p->has_z ? al(p->dout_x) : (al(p->dout) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && p->dout_sh % VS == 0));
     if (!p->CB && !dcb_recomputes_cb(p)) return BIMAMBA2_EINVAL;
+    if (p->causal && !(fast && sizeof(T) == 2 && p->chunk_size % 64 == 0)) return BIMAMBA2_EUNSUPPORTED;
     if (fast && sizeof(T) == 2 && p->chunk_size % 64 == 0) launch_dcb_ring<T>(grid, p, nc, nqt);
     else if (fast) hipLaunchKernelGGL((bwd_dcb_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
     else hipLaunchKernelGGL((bwd_dcb_kernel<T, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
@@ -1469,11 +1487,18 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
         ddr[e] = p.ddt_direct[o + qc];
         dtr[e] = to_f(dt[(int64_t)qc * p.dt_sl]);
     }
+    if (p.causal) {                   // single-direction operator: nothing wrote the reverse direction's terms
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vb[e] = ub[e] = 0.f;
+    }
     const float A = p.A[h];
     const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
     float chunk_term = 0.f;
     for (int s = 0; s < nsplit; ++s)
-        chunk_term += p.ddA_chunk_f[(((int64_t)b * H + h) * nc + c) * nsplit + s] + p.ddA_chunk_b[(((int64_t)b * H + h) * nc + c) * nsplit + s];
+    {
+        const float cf = p.ddA_chunk_f[(((int64_t)b * H + h) * nc + c) * nsplit + s], cr = p.ddA_chunk_b[(((int64_t)b * H + h) * nc + c) * nsplit + s];
+        chunk_term += cf + (p.causal ? 0.f : cr);
+    }
     // within-chunk part from the per-tile vectors of the dCB kernel; tile I = lane / 16 holds this lane's positions.
     // Four tiles per side at most (Q <= 256): tile indices past nqt are clamped for the loads and masked afterwards.
     const int I = lane >> 4, i0 = (lane & 15) * 4, Ic = min(I, nqt - 1);

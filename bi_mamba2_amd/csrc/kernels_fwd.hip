@@ -195,7 +195,8 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_kernel(const bimamba2_pa
 // CUMSUM (states only): the workgroup also does the work of chunk_cumsum_fwd_kernel for its (b, c, h) - wave 0 transforms
 // dt and scans it while the tiles are under way - and the first tile's workgroup writes dt_out, cs_f, cs_b for the later
 // kernels: one launch less in front of the forward pass.
-template <typename T, bool DSTATES, bool CUMSUM>
+// UNI: forward direction only (single-direction comparator).
+template <typename T, bool DSTATES, bool CUMSUM, bool UNI = false>
 __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bimamba2_params p, int nc) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
@@ -316,7 +317,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
         for (int j = 0; j < 4; ++j) {
             const Frag bfr = tile64_tr_frag<Frag>(bt, k0, j * 16, lr, lg);
             accf[j] = M::mma(af, bfr, accf[j]);
-            accb[j] = M::mma(ab, bfr, accb[j]);
+            if (!UNI) accb[j] = M::mma(ab, bfr, accb[j]);
         }
     }
     float *of = (DSTATES ? p.dstates_f : p.states_f) + (int64_t)blockIdx.z * P * N;
@@ -327,7 +328,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
         for (int i = 0; i < 4; ++i) {
             const int pp = pt * 64 + wave * 16 + lg * 4 + i, n = nt * 64 + j * 16 + lr;
             of[(int64_t)pp * N + n] = accf[j][i];
-            ob[(int64_t)pp * N + n] = accb[j][i];
+            if (!UNI) ob[(int64_t)pp * N + n] = accb[j][i];
         }
 }
 
@@ -438,6 +439,12 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cum
     }
     hipStream_t s = stream_of(p);
     if constexpr (sizeof(T) == 2) {
+        if (fast && p->chunk_size % 32 == 0 && p->causal) {
+            if (dstates) hipLaunchKernelGGL((chunk_state_direct_kernel<T, true, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            else if (cumsum) hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            else hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            return check_launch();
+        }
         if (fast && p->chunk_size % 32 == 0) {
             if (dstates) hipLaunchKernelGGL((chunk_state_direct_kernel<T, true, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
             else if (cumsum) hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
@@ -445,6 +452,7 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cum
             return check_launch();
         }
     }
+    if (p->causal) return BIMAMBA2_EUNSUPPORTED;
     if (cumsum) return BIMAMBA2_EINVAL;      // the caller checked chunk_state_does_cumsum()
     if (dstates) {
         if (fast) hipLaunchKernelGGL((chunk_state_kernel<T, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
@@ -477,10 +485,11 @@ bool chunk_state_does_cumsum(const bimamba2_params *p) {
 // The same with 16-byte accesses and one direction per workgroup (blockIdx.z = 2 b + dir); the loads of 8 chunks go out
 // together, unconditionally (past the last chunk a valid chunk is read again and not used).  Needs P*N % 4 == 0 and
 // 16-byte aligned tensors.
-__global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const bimamba2_params p, int nc) {
+// ndir = 1: the forward recurrence only (blockIdx.z = b).
+__global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const bimamba2_params p, int nc, int ndir) {
     const int PN = p.headdim * p.dstate;
     const int e = (blockIdx.x * NTHREADS + threadIdx.x) * 4;
-    const int h = blockIdx.y, b = blockIdx.z >> 1, dir = blockIdx.z & 1;
+    const int h = blockIdx.y, b = blockIdx.z / ndir, dir = blockIdx.z % ndir;
     if (e >= PN) return;
     const int Q = p.chunk_size;
     const float *cs = (dir == 0 ? p.cs_f : p.cs_b) + ((int64_t)b * p.nheads + h) * nc * Q + (dir == 0 ? Q - 1 : 0);
@@ -511,11 +520,13 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const b
 int launch_state_passing_fwd(const bimamba2_params *p) {
     const int nc = nchunks(p), PN = p->headdim * p->dstate;
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    const int ndir = p->causal ? 1 : 2;
     if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->final_f) && al(p->final_b)) {
-        dim3 grid((PN / 4 + NTHREADS - 1) / NTHREADS, p->nheads, p->batch * 2);
-        hipLaunchKernelGGL(state_passing_fwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+        dim3 grid((PN / 4 + NTHREADS - 1) / NTHREADS, p->nheads, p->batch * ndir);
+        hipLaunchKernelGGL(state_passing_fwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, ndir);
         return check_launch();
     }
+    if (p->causal) return BIMAMBA2_EUNSUPPORTED;
     dim3 grid((PN + NTHREADS - 1) / NTHREADS, p->nheads, p->batch);
     hipLaunchKernelGGL(state_passing_fwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
     return check_launch();

@@ -38,7 +38,9 @@ constexpr int SCAN_WAVES = 8, SCAN_THREADS = 64 * SCAN_WAVES;
 // lane (l%16 = row, l/16 = g) with columns k0 + 8g + 0..3 (resp. +4..7) of its row.  All waves of a workgroup read the
 // same 32 K rows per step, so they come from L1, where the CB rows were 256 KB of L2 traffic per workgroup.  The state
 // products use the raw rows as well and scale the accumulator instead of the operand.
-template <typename T, int QT, int NJ, bool BWD, bool FAST, int NF>
+// UNI (with NF > 0 only): the single-direction (causal) operator - the reverse direction's state product, the K steps on
+// the far side of the diagonal and the far half of the diagonal step are left out.
+template <typename T, int QT, int NJ, bool BWD, bool FAST, int NF, bool UNI = false>
 __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimamba2_params p, int nc, int npt) {
     typedef Mma<T> M;
     constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
@@ -204,7 +206,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                 for (int i = 0; i < PER; ++i) {
                     const int idx = threadIdx.x + i * SCAN_THREADS;
                     rawf[i] = *reinterpret_cast<const float4 *>(stf + idx * 4);
-                    rawb[i] = *reinterpret_cast<const float4 *>(stb + idx * 4);
+                    rawb[i] = UNI ? rawf[i] : *reinterpret_cast<const float4 *>(stb + idx * 4);
                 }
                 struct alignas(sizeof(T) * 4) Out { T v[4]; };
 #pragma unroll
@@ -220,7 +222,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             __syncthreads();
             TSTAMP(2)
 #pragma unroll
-            for (int dir = 0; dir < 2; ++dir) {
+            for (int dir = 0; dir < (UNI ? 1 : 2); ++dir) {
                 const T *st = dir ? sB : sF;
                 f32x4 tmp[QT][NJ] = {};
 #pragma unroll
@@ -423,6 +425,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                 else wait_vmcnt<0>();
                 raw_lds_barrier();                     // ... and everybody else's; the slot of step - 1 is free again
                 if (step + KRING - 1 < nsteps) kr_issue(step + KRING - 1);
+                if (UNI && (BWD ? k0 + KSTEP - 1 < wave * QT * 16 : k0 > wave * QT * 16 + QT * 16 - 1)) continue;   // far side of the diagonal
                 const unsigned slot = krl_a + (step % KRING) * (32 * 64 * 2);
                 // the CB tiles of both row tiles first; the K fragments are dead after that
                 f32x4 cb1[QT], cb2[QT];
@@ -475,7 +478,9 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                             const int k = kb + i;
                             const float lk = i < 4 ? l0[i & 3] : l1[i & 3], uk = i < 4 ? u0[i & 3] : u1[i & 3];
                             const float e = k < r ? lor[rt] - lk : upr[rt] - uk;
-                            v[i] = (i < 4 ? cb1[rt][i & 3] : cb2[rt][i & 3]) * ((k == r) ? 2.f : __builtin_amdgcn_exp2f(e));
+                            float w = (k == r) ? (UNI ? 1.f : 2.f) : __builtin_amdgcn_exp2f(e);
+                            if (UNI && (BWD ? k < r : k > r)) w = 0.f;
+                            v[i] = (i < 4 ? cb1[rt][i & 3] : cb2[rt][i & 3]) * w;
                         }
                         af[rt] = M::pack(v);
                     }
@@ -668,12 +673,19 @@ static int launch_scan_t(const bimamba2_params *p) {
     } while (0)
     const int qt = Q <= 128 ? 1 : 2;             // 16-row tiles per wave (8 waves)
     if constexpr (sizeof(T) == 2 && NJMAX == 4) {
+        if (p->causal) {                                // single-direction comparator: the fused kernels only
+            if (!scan_recomputes_cb(p, BWD)) return BIMAMBA2_EUNSUPPORTED;
+            if (qt == 1) hipLaunchKernelGGL((chunk_scan_kernel<T, 1, 4, BWD, true, 2, true>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
+            else hipLaunchKernelGGL((chunk_scan_kernel<T, 2, 4, BWD, true, 2, true>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
+            return check_launch();
+        }
         if ((BWD ? p->CBT : p->CB) == nullptr) {        // the caller checked scan_recomputes_cb()
             if (qt == 1) hipLaunchKernelGGL((chunk_scan_kernel<T, 1, 4, BWD, true, 2>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
             else hipLaunchKernelGGL((chunk_scan_kernel<T, 2, 4, BWD, true, 2>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
             return check_launch();
         }
     }
+    if (p->causal) return BIMAMBA2_EUNSUPPORTED;
     if ((BWD ? p->CBT : p->CB) == nullptr) return BIMAMBA2_EINVAL;
     if (pw == 16) { if (qt == 1) BM2_SCAN(1, 1); else BM2_SCAN(2, 1); }
     else if (pw == 32) { if (qt == 1) BM2_SCAN(1, 2); else BM2_SCAN(2, 2); }

@@ -439,20 +439,24 @@ def _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit):
 
 
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
-                                   dt_limit=(0.0, _INF), return_intermediates=True, keep_for_bwd=False):
+                                   dt_limit=(0.0, _INF), return_intermediates=True, keep_for_bwd=False, causal=False):
     """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
     like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
     out, out_x and the final states are materialised as tensors (the rest lives in a workspace).
     keep_for_bwd=True appends a tenth element: the tuple (dt_out, cs_f, cs_b, states_f, states_b, snapshot) that
     _mamba_chunk_scan_combined_bwd accepts as `saved` to skip its recomputation (snapshot: the input half of the
-    parameter block, reused when the backward pass gets the same tensors)."""
+    parameter block, reused when the backward pass gets the same tensors).
+    causal=True runs the single-direction operator (see causal_chunk_scan_combined): no reverse states, final_states_b
+    is None."""
     c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
+    c.p.causal = 1 if causal else 0
     batch, seqlen, nheads, headdim = x.shape
     ngroups, dstate = B.shape[2], B.shape[3]
     snap = c.snapshot() if keep_for_bwd else None
     out = c.new("out", x.shape, x.dtype)
     out_x = c.new("out_x", x.shape, x.dtype) if z is not None else None
-    ff = c.new("final_f", (batch, nheads, headdim, dstate)); fb = c.new("final_b", (batch, nheads, headdim, dstate))
+    ff = c.new("final_f", (batch, nheads, headdim, dstate))
+    fb = None if causal else c.new("final_b", (batch, nheads, headdim, dstate))
     dt_out = cs_f = cs_b = sf = sb = None
     saved = None
     if return_intermediates or keep_for_bwd:
@@ -469,7 +473,8 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
 
 def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
                                    dfinal_states=None, dt_softplus=False, dt_limit=(0.0, _INF),
-                                   dx=None, ddt=None, dB=None, dC=None, dz=None, recompute_output=False, saved=None):
+                                   dx=None, ddt=None, dB=None, dC=None, dz=None, recompute_output=False, saved=None,
+                                   causal=False):
     """Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias).  `out` must be the pre-gate output out_x when z is
     given (it is what the autograd function saves); it is not read otherwise.  `saved` is the tuple the forward
     returns with keep_for_bwd=True; without it the forward intermediates are recomputed, as in the reference."""
@@ -487,6 +492,7 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
             c = None
     if c is None:
         c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
+    c.p.causal = 1 if causal else 0
     batch, seqlen, nheads, headdim = x.shape
     c.set_dout(dout)
     if saved is not None:
@@ -576,3 +582,39 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
     """
     return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
                                           return_final_states)
+
+
+class CausalChunkScanCombinedFn(torch.autograd.Function):
+    """The single-direction operator  y = SS(x) + D*x  (gated by silu(z)) from the same kernels with the reverse
+    direction left out: the comparator the bidirectional pass is timed against.  It exists for the shapes whose scan
+    kernels rebuild C.B^T themselves (16-bit x/B/C, headdim a multiple of 64, dstate 64, chunk_size a multiple of 64,
+    16-byte aligned rows); other shapes raise.  The math is the reference's causal path
+    (src/ssd/uni/ssd_combined.py:621-659 there)."""
+
+    @staticmethod
+    def forward(ctx, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False, dt_limit=(0.0, _INF)):
+        keep = any(t is not None and t.requires_grad for t in (x, dt, A, B, C, D, z, dt_bias))
+        res = _mamba_chunk_scan_combined_fwd(
+            x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit,
+            return_intermediates=False, keep_for_bwd=keep, causal=True)
+        saved = res[9] if keep else ()
+        ctx.n_saved = len(saved)
+        ctx.snap = saved[5] if keep else None
+        ctx.save_for_backward(res[1] if z is not None else None, x, dt, A, B, C, D, z, dt_bias, *saved[:5])
+        ctx.dt_softplus, ctx.chunk_size, ctx.dt_limit = dt_softplus, chunk_size, dt_limit
+        return res[0]
+
+    @staticmethod
+    def backward(ctx, dout):
+        out_x, x, dt, A, B, C, D, z, dt_bias = ctx.saved_tensors[:9]
+        saved = tuple(ctx.saved_tensors[9:]) + (ctx.snap,) if ctx.n_saved else None
+        dx, ddt, dA, dB, dC, dD, dz, ddt_bias = _mamba_chunk_scan_combined_bwd(
+            dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
+            dt_limit=ctx.dt_limit, saved=saved, causal=True)
+        return dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, None, None
+
+
+def causal_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
+                               dt_limit=(0.0, _INF)):
+    """Single-direction (causal) SSD with the arguments of bimamba_chunk_scan_combined; see CausalChunkScanCombinedFn."""
+    return CausalChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)

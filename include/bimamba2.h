@@ -56,7 +56,12 @@ typedef struct bimamba2_params {
     int32_t has_D, D_has_hdim, has_z, has_dt_bias, dt_softplus;
     int32_t fwd_saved;      /* bimamba2_bwd only: dt_out, cs_f, cs_b, states_f, states_b hold what bimamba2_fwd left in
                                them, so the backward pass does not recompute them (CB is always recomputed) */
-    int32_t reserved0;
+    int32_t causal;         /* 0: the bidirectional operator.  1: the single-direction (causal) operator built from the same
+                               kernels with the reverse direction left out - the comparator the bidirectional pass is
+                               timed against.  Every entry point follows it, but only for the shapes whose scan
+                               kernels rebuild CB (bimamba2_chunk_scan_reads_cb() == 0): BIMAMBA2_EUNSUPPORTED otherwise.
+                               The reverse direction's buffers (states_b, dstates_b, u_b, v_b, ddA_chunk_b) are neither
+                               written nor used; final_b must be NULL. */
     float dt_min, dt_max;
     /* element strides of the strided inputs (last dim contiguous) */
     int64_t x_sb, x_sl, x_sh;

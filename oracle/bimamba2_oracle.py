@@ -163,6 +163,16 @@ def bimamba2_naive_chunked(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=N
     return out, out_x, final_f, final_b
 
 
+def ssd_causal(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False, dt_limit=(0.0, float("inf"))):
+    """The single-direction operator y = SS(x) + D*x (gated by silu(z)): one causal pass of the naive path above (math of
+    the reference's ssd_chunk_scan_combined_ref, src/ssd/uni/ssd_combined.py:621-659).  Returns (out, out_x, final).
+    It is what the causal comparator of the HIP path is checked against."""
+    dtp = dt_transform(dt, dt_bias, dt_softplus, dt_limit)
+    y, final = ssd_causal_chunked(x, dtp, A, B, C, chunk_size)
+    out, out_x = _finish(y, x, D, z)
+    return out, out_x, final
+
+
 # --------------------------------------------------------------------------------------------------------
 # per-stage restatements of the chunked bidirectional algorithm (layouts of the reference stage wrappers)
 # --------------------------------------------------------------------------------------------------------
@@ -286,6 +296,8 @@ def bimamba2_grads(dout, x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softpl
         out = bimamba2_quadratic(*leaves[:5], **kw)[0]
     elif form == "sequential":
         out = bimamba2_sequential(*leaves[:5], **kw)[0]
+    elif form == "causal":
+        out = ssd_causal(*leaves[:5], chunk_size, **kw)[0]
     else:
         out = bimamba2_naive_chunked(*leaves[:5], chunk_size, **kw)[0]
     present = [l for l in leaves if l is not None]

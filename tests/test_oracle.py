@@ -123,3 +123,32 @@ def test_gradients_of_forms_agree():
     b = O.bimamba2_grads(dout, inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], form="chunked", chunk_size=32, **kw)
     for k in a:
         torch.testing.assert_close(a[k], b[k], rtol=1e-10, atol=1e-10, msg=lambda m: f"{k}: {m}")
+
+
+def test_causal_operator_against_the_plain_recurrence():
+    """ssd_causal (what the single-direction comparator is checked against) against the token-by-token recurrence
+    h_t = e^{dt_t A} h_{t-1} + dt_t x_t (x) B_t,  y_t = C_t . h_t + D x_t  written out here, and: the two causal passes
+    (as given, and on the flipped sequence) add up to the bidirectional operator, whose diagonal term is counted twice."""
+    inp = to64(make_case(2, 37, 4, 3, 2, 5, with_z=True, D_has_hdim=True))
+    x, dt, A, B, C, D, z, bias = (inp[k] for k in ("x", "dt", "A", "B", "C", "D", "z", "dt_bias"))
+    out, out_x, final = O.ssd_causal(x, dt, A, B, C, 16, D=D, z=z, dt_bias=bias, dt_softplus=True)
+    dtp = torch.nn.functional.softplus(dt + bias)
+    bsz, L, H, P = x.shape
+    G, N = B.shape[2], B.shape[3]
+    y = torch.zeros_like(x)
+    for b in range(bsz):
+        for h in range(H):
+            g = h // (H // G)
+            st = torch.zeros(P, N, dtype=x.dtype)
+            for t in range(L):
+                st = torch.exp(dtp[b, t, h] * A[h]) * st + dtp[b, t, h] * torch.outer(x[b, t, h], B[b, t, g])
+                y[b, t, h] = st @ C[b, t, g] + D[h] * x[b, t, h]
+            torch.testing.assert_close(final[b, h], st, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(out_x, y, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(out, y * z * torch.sigmoid(z), rtol=1e-10, atol=1e-10)
+    # bidirectional = causal + flip(causal(flip)); the diagonal term dt_t (C_t.B_t) x_t is in both passes
+    kw = dict(dt_bias=bias, dt_softplus=True)
+    yf = O.ssd_causal(x, dt, A, B, C, 16, **kw)[0]
+    yb = O.ssd_causal(x.flip(1), dt.flip(1), A, B.flip(1), C.flip(1), 16, **kw)[0].flip(1)
+    bi = O.bimamba2_sequential(x, dt, A, B, C, **kw)[0]
+    torch.testing.assert_close(yf + yb, bi, rtol=1e-10, atol=1e-10)
