@@ -33,6 +33,20 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// Global loads the compiler does not know of: it neither moves them (a load it knows of may be sunk below later requests
+// and then be waited for with vmcnt(0), which drains every request in flight) nor waits for them.  The caller waits with
+// wait_vmcnt<N>() and then ties each value to that wait with raw_lds_use() before its first use.
+__device__ __forceinline__ float raw_global_load_f32(const float *p) {
+    float v;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ unsigned raw_global_load_u16(const void *p) {      // zero-extended 16 bits
+    unsigned v;
+    asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+
 // ---- row-major tiles as MFMA operands: LDS transpose reads ------------------------------------------------------
 // A tile of 16-bit elements lies in LDS as it lies in global memory, [k][n] with n contiguous (rows of 64 elements,
 // 128 bytes), brought there by direct loads.  Its 16-byte chunks are swizzled, chunk c of row k sits at position

@@ -225,39 +225,86 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     int64_t bs;
     if (DSTATES) { bs = p.C_sl; bp = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * bs + g * p.C_sg; }
     else { bs = p.B_sl; bp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * bs + g * p.B_sg; }
-    const int rows = (limit + 31) & ~31;                   // K steps of 32 positions
-    tile64_request(xt, xp + pt * 64, xs, rows, limit, wave, NTHREADS / 64, lane);
-    tile64_request(bt, bp + nt * 64, bs, rows, limit, wave, NTHREADS / 64, lane);
+    const int rows = (limit + 31) & ~31, nsteps = rows / 32;     // K steps of 32 positions
     const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
-    if constexpr (CUMSUM && !DSTATES) {
-        __shared__ float dts[BIMAMBA2_MAX_CHUNK], csfs[BIMAMBA2_MAX_CHUNK], csbs[BIMAMBA2_MAX_CHUNK];
+    constexpr bool DO_CUMSUM = CUMSUM && !DSTATES;
+    // Order of this wave's vector memory operations: first the few register loads the weight tables need, then, K step by
+    // K step, one request for 8 rows of the x tile and one for 8 rows of the B tile (4 waves x 8 rows = the 32 rows of a
+    // step).  Loads complete in order, so "at most 2 (nsteps - 1 - s) outstanding" means that the register loads and this
+    // wave's part of steps 0..s have landed; a barrier then covers the other waves' parts.  The products of step s run
+    // while the later steps are still under way.  Until the last step every LDS access is a raw one (the compiler would
+    // make an access it knows of wait for all outstanding requests).
+    float r_cf = 0.f, r_cb = 0.f, r_dt = 0.f, e_f = 0.f, e_b = 0.f, A_h = 0.f, bias_h = 0.f;
+    unsigned dt_raw[4] = {0u, 0u, 0u, 0u};                   // DO_CUMSUM, wave 0: bits of dt at this lane's four positions
+    if constexpr (DO_CUMSUM) {
         if (wave == 0) {
-            const float A = p.A[h];
-            const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
             const int64_t dto = b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
-            float v[4], a[4], raw[4];
             int64_t at[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) at[e] = dto + (int64_t)min(lane * 4 + e, limit - 1) * p.dt_sl;
-            // one branch on the type around all four loads, so that they go out together
             if (p.dt_dtype == BIMAMBA2_F32) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) raw[e] = reinterpret_cast<const float *>(p.dt)[at[e]];
-            } else if (p.dt_dtype == BIMAMBA2_BF16) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) raw[e] = to_f(reinterpret_cast<const bf16_t *>(p.dt)[at[e]]);
+                for (int e = 0; e < 4; ++e) dt_raw[e] = __float_as_uint(raw_global_load_f32(reinterpret_cast<const float *>(p.dt) + at[e]));
             } else {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) raw[e] = to_f(reinterpret_cast<const f16_t *>(p.dt)[at[e]]);
+                for (int e = 0; e < 4; ++e) dt_raw[e] = raw_global_load_u16(reinterpret_cast<const uint16_t *>(p.dt) + at[e]);
             }
+            A_h = raw_global_load_f32(p.A + h);
+            bias_h = raw_global_load_f32(p.has_dt_bias ? p.dt_bias + h : p.A + h);
+        }
+    } else {
+        const int q = min((int)threadIdx.x, limit - 1);      // chunk_size <= 256 = NTHREADS: one position per thread
+        r_cf = raw_global_load_f32(p.cs_f + o + q);
+        r_cb = raw_global_load_f32(p.cs_b + o + q);
+        if (!DSTATES) {
+            r_dt = raw_global_load_f32(p.dt_out + o + q);
+            e_f = raw_global_load_f32(p.cs_f + o + Q - 1);
+            e_b = raw_global_load_f32(p.cs_b + o);
+        }
+    }
+    for (int s = 0; s < nsteps; ++s) {
+        const int u = 4 * s + wave, row = u * 8 + (lane >> 3);
+        const int col = ((lane & 7) ^ tile64_swz(row)) << 3;
+        load16_to_lds(xp + pt * 64 + (int64_t)min(row, limit - 1) * xs + col, xt + u * 512);
+        load16_to_lds(bp + nt * 64 + (int64_t)min(row, limit - 1) * bs + col, bt + u * 512);
+    }
+    auto wait_steps = [&](int newer) {       // at most 2 * newer requests outstanding (newer is wave-uniform, 0..7)
+        switch (newer) {
+            case 0: wait_vmcnt<0>(); break;
+            case 1: wait_vmcnt<2>(); break;
+            case 2: wait_vmcnt<4>(); break;
+            case 3: wait_vmcnt<6>(); break;
+            case 4: wait_vmcnt<8>(); break;
+            case 5: wait_vmcnt<10>(); break;
+            case 6: wait_vmcnt<12>(); break;
+            case 7: wait_vmcnt<14>(); break;
+            default: wait_vmcnt<16>(); break;
+        }
+    };
+    const unsigned wf_a = lds_addr(wf), wb_a = lds_addr(wb);
+    float keep_dt[4], keep_f[4], keep_b[4];                  // DO_CUMSUM, wave 0: what the first tile's workgroup writes out at the end
+    if constexpr (DO_CUMSUM) {
+        __shared__ float dts[BIMAMBA2_MAX_CHUNK], csfs[BIMAMBA2_MAX_CHUNK], csbs[BIMAMBA2_MAX_CHUNK];
+        const unsigned dts_a = lds_addr(dts), csf_a = lds_addr(csfs), csb_a = lds_addr(csbs);
+        if (wave == 0) {
+            wait_steps(nsteps);
+            raw_lds_use(A_h); raw_lds_use(bias_h);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) raw_lds_use(dt_raw[e]);
+            const float A = A_h;
+            const float bias = p.has_dt_bias ? bias_h : 0.f;
+            float a[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int q = lane * 4 + e;
-                float d = raw[e] + bias;
+                const float dtv = p.dt_dtype == BIMAMBA2_F32 ? __uint_as_float(dt_raw[e])
+                                  : p.dt_dtype == BIMAMBA2_BF16 ? __uint_as_float(dt_raw[e] << 16)
+                                                                : to_f(__builtin_bit_cast(f16_t, (unsigned short)dt_raw[e]));
+                float d = dtv + bias;
                 if (p.dt_softplus) d = d > 20.f ? d : log1pf(expf(d));
                 d = fminf(fmaxf(d, p.dt_min), p.dt_max);
                 if (q >= limit) d = 0.f;
-                v[e] = d;
+                keep_dt[e] = d;
                 a[e] = d * A;
             }
             float pf[4], sb[4];
@@ -267,44 +314,65 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
             const float before = wave_incl_prefix(tot, lane) - tot, after = wave_incl_suffix(tot, lane) - tot;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int q = lane * 4 + e;
-                dts[q] = v[e];
-                csfs[q] = before + pf[e];
-                csbs[q] = after + sb[e];
-                if (q < Q && nt == 0 && pt == 0) {
-                    p.dt_out[o + q] = v[e];
-                    p.cs_f[o + q] = before + pf[e];
-                    p.cs_b[o + q] = after + sb[e];
-                }
+                keep_f[e] = before + pf[e];
+                keep_b[e] = after + sb[e];
             }
+            raw_lds_write128_at<0>(dts_a + lane * 16, f32x4{keep_dt[0], keep_dt[1], keep_dt[2], keep_dt[3]});
+            raw_lds_write128_at<0>(csf_a + lane * 16, f32x4{keep_f[0], keep_f[1], keep_f[2], keep_f[3]});
+            raw_lds_write128_at<0>(csb_a + lane * 16, f32x4{keep_b[0], keep_b[1], keep_b[2], keep_b[3]});
+            raw_lds_wait();
         }
-        __syncthreads();
-        for (int q = threadIdx.x; q < rows; q += NTHREADS) {
-            wf[q] = q < limit ? __expf(csfs[Q - 1] - csfs[q]) * dts[q] : 0.f;
-            wb[q] = q < limit ? __expf(csbs[0] - csbs[q]) * dts[q] : 0.f;
+        raw_lds_barrier();
+        {
+            const int q = threadIdx.x;
+            float d = raw_lds_read_at<float, 0>(dts_a + q * 4), cf = raw_lds_read_at<float, 0>(csf_a + q * 4);
+            float cb = raw_lds_read_at<float, 0>(csb_a + q * 4);
+            float ef = raw_lds_read_at<float, 0>(csf_a + (Q - 1) * 4), eb = raw_lds_read_at<float, 0>(csb_a);
+            raw_lds_wait();
+            raw_lds_use(d); raw_lds_use(cf); raw_lds_use(cb); raw_lds_use(ef); raw_lds_use(eb);
+            const bool in = q < limit;
+            raw_lds_write_at<0>(wf_a + q * 4, in ? __expf(ef - cf) * d : 0.f);
+            raw_lds_write_at<0>(wb_a + q * 4, in ? __expf(eb - cb) * d : 0.f);
+            raw_lds_wait();
         }
-    } else
-    for (int q = threadIdx.x; q < rows; q += NTHREADS) {
+    } else {
+        wait_steps(nsteps);
+        raw_lds_use(r_cf); raw_lds_use(r_cb); raw_lds_use(r_dt); raw_lds_use(e_f); raw_lds_use(e_b);
+        const int q = threadIdx.x;
         float f = 0.f, r = 0.f;
         if (q < limit) {
-            if (DSTATES) {
-                f = __expf(p.cs_f[o + q]);
-                r = __expf(p.cs_b[o + q]);
-            } else {
-                const float d = p.dt_out[o + q];
-                f = __expf(p.cs_f[o + Q - 1] - p.cs_f[o + q]) * d;
-                r = __expf(p.cs_b[o] - p.cs_b[o + q]) * d;
-            }
+            if (DSTATES) { f = __expf(r_cf); r = __expf(r_cb); }
+            else { f = __expf(e_f - r_cf) * r_dt; r = __expf(e_b - r_cb) * r_dt; }
         }
-        wf[q] = f;
-        wb[q] = r;
+        raw_lds_write_at<0>(wf_a + q * 4, f);
+        raw_lds_write_at<0>(wb_a + q * 4, r);
+        raw_lds_wait();
     }
-    __syncthreads();       // (the compiler drains this wave's requests before its first LDS access; the barrier covers the rest)
+    // lane parts of the fragment addresses (see tile64_tr_frag): rows kk and kk + 4 of a step, 4 columns from nn on
+    const int kk = 8 * lg + (lr >> 2), nn = 4 * (lr & 3);
+    const unsigned xa_lo = lds_addr(xt) + tile64_tr_offset(kk, wave * 16 + nn), xa_hi = lds_addr(xt) + tile64_tr_offset(kk + 4, wave * 16 + nn);
+    unsigned ba_lo[4], ba_hi[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        ba_lo[j] = lds_addr(bt) + tile64_tr_offset(kk, j * 16 + nn);
+        ba_hi[j] = lds_addr(bt) + tile64_tr_offset(kk + 4, j * 16 + nn);
+    }
+    const unsigned wfl = wf_a + 32 * lg, wbl = wb_a + 32 * lg;
     f32x4 accf[4] = {}, accb[4] = {};
-    for (int k0 = 0; k0 < rows; k0 += 32) {
-        const Frag a = tile64_tr_frag<Frag>(xt, k0, wave * 16, lr, lg);
-        const f32x4 f0 = *reinterpret_cast<const f32x4 *>(wf + k0 + 8 * lg), f1 = *reinterpret_cast<const f32x4 *>(wf + k0 + 8 * lg + 4);
-        const f32x4 r0 = *reinterpret_cast<const f32x4 *>(wb + k0 + 8 * lg), r1 = *reinterpret_cast<const f32x4 *>(wb + k0 + 8 * lg + 4);
+    auto kstep = [&](auto S) {
+        constexpr int s = decltype(S)::value;
+        constexpr int TO = s * 32 * 128, WO = s * 32 * 4;      // byte offsets of the step in the tiles / the weight tables
+        wait_steps(nsteps - 1 - s);
+        raw_lds_barrier();
+        i16x4 alo = raw_lds_tr16_read_at<TO>(xa_lo), ahi = raw_lds_tr16_read_at<TO>(xa_hi);
+        f32x4 f0 = raw_lds_read_at<f32x4, WO>(wfl), f1 = raw_lds_read_at<f32x4, WO + 16>(wfl);
+        f32x4 r0 = raw_lds_read_at<f32x4, WO>(wbl), r1 = raw_lds_read_at<f32x4, WO + 16>(wbl);
+        i16x4 blo[4], bhi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { blo[j] = raw_lds_tr16_read_at<TO>(ba_lo[j]); bhi[j] = raw_lds_tr16_read_at<TO>(ba_hi[j]); }
+        raw_lds_wait();
+        raw_lds_use(alo); raw_lds_use(ahi); raw_lds_use(f0); raw_lds_use(f1); raw_lds_use(r0); raw_lds_use(r1);
+        const Frag a = __builtin_bit_cast(Frag, __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7));
         float vf[8], vb[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -315,11 +383,21 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
         const Frag af = M::pack(vf), ab = M::pack(vb);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const Frag bfr = tile64_tr_frag<Frag>(bt, k0, j * 16, lr, lg);
+            raw_lds_use(blo[j]); raw_lds_use(bhi[j]);
+            const Frag bfr = __builtin_bit_cast(Frag, __builtin_shufflevector(blo[j], bhi[j], 0, 1, 2, 3, 4, 5, 6, 7));
             accf[j] = M::mma(af, bfr, accf[j]);
             if (!UNI) accb[j] = M::mma(ab, bfr, accb[j]);
         }
-    }
+    };
+    static_assert(BIMAMBA2_MAX_CHUNK == 256, "eight K steps of 32 positions");
+    kstep(std::integral_constant<int, 0>());
+    if (nsteps > 1) kstep(std::integral_constant<int, 1>());
+    if (nsteps > 2) kstep(std::integral_constant<int, 2>());
+    if (nsteps > 3) kstep(std::integral_constant<int, 3>());
+    if (nsteps > 4) kstep(std::integral_constant<int, 4>());
+    if (nsteps > 5) kstep(std::integral_constant<int, 5>());
+    if (nsteps > 6) kstep(std::integral_constant<int, 6>());
+    if (nsteps > 7) kstep(std::integral_constant<int, 7>());
     float *of = (DSTATES ? p.dstates_f : p.states_f) + (int64_t)blockIdx.z * P * N;
     float *ob = (DSTATES ? p.dstates_b : p.states_b) + (int64_t)blockIdx.z * P * N;
 #pragma unroll
@@ -330,6 +408,19 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
             of[(int64_t)pp * N + n] = accf[j][i];
             if (!UNI) ob[(int64_t)pp * N + n] = accb[j][i];
         }
+    if constexpr (DO_CUMSUM) {
+        if (wave == 0 && nt == 0 && pt == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int q = lane * 4 + e;
+                if (q < Q) {
+                    p.dt_out[o + q] = keep_dt[e];
+                    p.cs_f[o + q] = keep_f[e];
+                    p.cs_b[o + q] = keep_b[e];
+                }
+            }
+        }
+    }
 }
 
 // =========================================================================================================
