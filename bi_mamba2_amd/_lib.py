@@ -44,9 +44,11 @@ ENTRY_POINTS = (
     "bimamba2_chunk_scan_bwd_dcb", "bimamba2_bmm_chunk_bwd", "bimamba2_chunk_cumsum_bwd",
 )
 NORM_ENTRY_POINTS = ("bimamba2_rmsnorm_gated_fwd", "bimamba2_rmsnorm_gated_bwd")
+CONV_ENTRY_POINTS = ("bimamba2_conv1d_silu_fwd", "bimamba2_conv1d_silu_bwd")
 ALL_SYMBOLS = ENTRY_POINTS + ("bimamba2_strerror", "bimamba2_version", "bimamba2_params_size",
                               "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb", "bimamba2_norm_params_size",
-                              "bimamba2_rmsnorm_gated_workspace_bytes") + NORM_ENTRY_POINTS
+                              "bimamba2_rmsnorm_gated_workspace_bytes", "bimamba2_conv_params_size",
+                              "bimamba2_conv1d_silu_workspace_bytes") + NORM_ENTRY_POINTS + CONV_ENTRY_POINTS
 
 _lib = None
 
@@ -58,6 +60,16 @@ class NormParams(ctypes.Structure):
          ("norm_before_gate", _i32), ("eps", _f32), ("reserved0", _i32)]
         + [(n, _i64) for n in ("x_rs", "z_rs", "out_rs", "dout_rs", "dx_rs", "dz_rs")]
         + [(n, _vp) for n in ("x", "z", "weight", "bias", "out", "rstd", "dout", "dx", "dz", "dweight", "dbias", "workspace")]
+        + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
+    )
+
+
+class ConvParams(ctypes.Structure):
+    """Mirror of ``struct bimamba2_conv_params`` (depthwise conv1d + SiLU)."""
+    _fields_ = (
+        [("batch", _i64), ("seqlen", _i64), ("channels", _i32), ("width", _i32), ("dtype", _i32), ("has_bias", _i32)]
+        + [(n, _i64) for n in ("x_sb", "x_sl", "dout_sb", "dout_sl")]
+        + [(n, _vp) for n in ("x", "weight", "bias", "out", "dout", "dx", "dweight", "dbias", "workspace")]
         + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
     )
 
@@ -95,6 +107,15 @@ def load():
         raise RuntimeError("bimamba2_norm_params layout mismatch between the library and its Python mirror")
     lib.bimamba2_rmsnorm_gated_workspace_bytes.argtypes = [ctypes.POINTER(NormParams)]
     lib.bimamba2_rmsnorm_gated_workspace_bytes.restype = ctypes.c_size_t
+    for name in CONV_ENTRY_POINTS:
+        fn = getattr(lib, name)
+        fn.argtypes = [ctypes.POINTER(ConvParams)]
+        fn.restype = ctypes.c_int
+    lib.bimamba2_conv_params_size.restype = ctypes.c_size_t
+    if lib.bimamba2_conv_params_size() != ctypes.sizeof(ConvParams):
+        raise RuntimeError("bimamba2_conv_params layout mismatch between the library and its Python mirror")
+    lib.bimamba2_conv1d_silu_workspace_bytes.argtypes = [ctypes.POINTER(ConvParams)]
+    lib.bimamba2_conv1d_silu_workspace_bytes.restype = ctypes.c_size_t
     _lib = lib
     return lib
 

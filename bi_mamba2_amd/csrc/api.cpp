@@ -347,4 +347,41 @@ int bimamba2_rmsnorm_gated_bwd(const bimamba2_norm_params *p) {
     return launch_rmsnorm_gated(p, true);
 }
 
+size_t bimamba2_conv_params_size(void) { return sizeof(bimamba2_conv_params); }
+
+static int check_conv(const bimamba2_conv_params *p) {
+    if (!p) return BIMAMBA2_EINVAL;
+    if (p->batch < 0 || p->seqlen < 0 || p->channels <= 0) return BIMAMBA2_EINVAL;
+    if (p->dtype != BIMAMBA2_F32 && p->dtype != BIMAMBA2_BF16 && p->dtype != BIMAMBA2_F16) return BIMAMBA2_EUNSUPPORTED;
+    if (p->width < 1 || p->width > 9 || p->width % 2 == 0) return BIMAMBA2_EUNSUPPORTED;
+    if (p->seqlen > (1 << 30)) return BIMAMBA2_EUNSUPPORTED;
+    if (!p->x || !p->weight || (p->has_bias && !p->bias)) return BIMAMBA2_EINVAL;
+    return BIMAMBA2_OK;
+}
+
+size_t bimamba2_conv1d_silu_workspace_bytes(const bimamba2_conv_params *p) {
+    if (check_conv(p)) return 0;
+    return conv_workspace_bytes(p);
+}
+
+int bimamba2_conv1d_silu_fwd(const bimamba2_conv_params *p) {
+    TRY(check_conv(p));
+    REQUIRE(p->out);
+    if (p->batch == 0 || p->seqlen == 0) return BIMAMBA2_OK;
+    return launch_conv1d_silu(p, false);
+}
+
+int bimamba2_conv1d_silu_bwd(const bimamba2_conv_params *p) {
+    TRY(check_conv(p));
+    REQUIRE(p->dout); REQUIRE(p->dx); REQUIRE(p->dweight);
+    if (p->has_bias) REQUIRE(p->dbias);
+    if (!p->workspace || p->workspace_bytes < conv_workspace_bytes(p)) return BIMAMBA2_EWORKSPACE;
+    if (p->batch == 0 || p->seqlen == 0) {
+        TRY(launch_fill(p->dweight, (size_t)p->channels * p->width, 0.f, reinterpret_cast<hipStream_t>(p->stream)));
+        if (p->has_bias) TRY(launch_fill(p->dbias, (size_t)p->channels, 0.f, reinterpret_cast<hipStream_t>(p->stream)));
+        return BIMAMBA2_OK;
+    }
+    return launch_conv1d_silu(p, true);
+}
+
 }  // extern "C"

@@ -288,6 +288,11 @@ __global__ __launch_bounds__(NTHREADS) void colsum_kernel(const float *in0, floa
     }
 }
 
+int launch_colsum(const float *in, float *out, int ni, int nj, hipStream_t stream) {
+    hipLaunchKernelGGL(colsum_kernel, dim3((nj + 15) / 16, 1), dim3(NTHREADS), 0, stream, in, out, nullptr, nullptr, ni, nj);
+    return check_launch();
+}
+
 static bool norm_vec_ok(const bimamba2_norm_params *p, bool bwd, int elem) {
     const int vs = 16 / elem;
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };

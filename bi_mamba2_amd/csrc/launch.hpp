@@ -38,5 +38,11 @@ int launch_reduce(const float *in, float *out, int ni, int nj, int nk, hipStream
 // gated RMSNorm (kernels_norm.hip)
 int launch_rmsnorm_gated(const bimamba2_norm_params *p, bool bwd);
 size_t norm_workspace_bytes(const bimamba2_norm_params *p);
+// out[j] = sum_i in[i * nj + j], fixed order
+int launch_colsum(const float *in, float *out, int ni, int nj, hipStream_t stream);
+
+// depthwise conv1d + SiLU (kernels_conv.hip)
+int launch_conv1d_silu(const bimamba2_conv_params *p, bool bwd);
+size_t conv_workspace_bytes(const bimamba2_conv_params *p);
 
 }  // namespace bm2

@@ -12,6 +12,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from .conv1d import conv1d_silu_fn
 from .layernorm_gated import RMSNorm
 from .ops import bimamba_chunk_scan_combined
 
@@ -75,13 +76,15 @@ class BiMamba2(nn.Module):
         zxbcdt = self.in_proj(u)
         A = -torch.exp(self.A_log.float())
         z, xBC, dt = torch.split(zxbcdt, [self.d_inner, self.d_inner + 2 * bc, self.nheads], dim=-1)
-        dt = F.softplus(dt + self.dt_bias)
-        xBC = self.act(self.conv1d(xBC.transpose(1, 2)).transpose(1, 2))
+        # conv1d + SiLU on the channels-last view, one HIP kernel (the reference transposes, calls nn.Conv1d, transposes
+        # back and applies the activation, modules.py:162-164 there); self.conv1d only holds the parameters
+        xBC = conv1d_silu_fn(xBC, self.conv1d.weight, self.conv1d.bias)
         x, B, C = torch.split(xBC, [self.d_inner, bc, bc], dim=-1)
         kw = {} if tuple(self.dt_limit) == (0.0, float("inf")) else {"dt_limit": tuple(self.dt_limit)}
+        # softplus(dt + dt_bias) (modules.py:158 there) happens inside the operator's first kernel
         y = bimamba_chunk_scan_combined(
             x.unflatten(-1, (self.nheads, self.headdim)), dt, A,
             B.unflatten(-1, (self.ngroups, self.d_state)), C.unflatten(-1, (self.ngroups, self.d_state)),
-            chunk_size=self.chunk_size, D=self.D, z=None, **kw)
+            chunk_size=self.chunk_size, D=self.D, z=None, dt_bias=self.dt_bias, dt_softplus=True, **kw)
         y = self.norm(y.flatten(-2), z)
         return self.out_proj(y)

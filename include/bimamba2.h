@@ -214,6 +214,44 @@ int bimamba2_rmsnorm_gated_fwd(const bimamba2_norm_params *p);
 /* x [z] weight [bias] rstd dout -> dx [dz] dweight [dbias] */
 int bimamba2_rmsnorm_gated_bwd(const bimamba2_norm_params *p);
 
+/* ---------------------------------------------------------------------------------------------------------
+ * Non-causal depthwise conv1d + SiLU on channels-last activations: the step in front of the operator in the
+ * BiMamba2 layer.  Replaces  act(conv1d(xBC.transpose(1, 2)).transpose(1, 2))  of the reference
+ * (src/ssd/modules.py:162-164; the convolution is constructed at :68-75 with groups = channels and
+ * padding = d_conv // 2) without the two transposes:
+ *   out[b, l, c] = silu(bias[c] + sum_k weight[c, k] * x[b, l + k - width / 2, c]),   zero padding.
+ * width is odd, 1..9.  x and dout may be strided views (batch and position strides in elements, channels contiguous);
+ * out and dx are written contiguous as (batch, seqlen, channels).  weight (channels, width), bias, dweight, dbias are
+ * float32.  The backward pass recomputes the pre-activation from x, and needs
+ * bimamba2_conv1d_silu_workspace_bytes() bytes of workspace for its fixed-order partial sums.
+ * --------------------------------------------------------------------------------------------------------- */
+typedef struct bimamba2_conv_params {
+    int64_t batch, seqlen;
+    int32_t channels, width;
+    int32_t dtype;              /* BIMAMBA2_* : x, out, dout, dx */
+    int32_t has_bias;
+    int64_t x_sb, x_sl;         /* element strides of x: batch, position */
+    int64_t dout_sb, dout_sl;   /* of dout (backward) */
+    const void *x;
+    const float *weight;        /* (channels, width) */
+    const float *bias;          /* (channels) or NULL */
+    void *out;                  /* forward: (batch, seqlen, channels) */
+    const void *dout;           /* backward */
+    void *dx;                   /* backward: (batch, seqlen, channels) */
+    float *dweight;             /* backward: (channels, width) */
+    float *dbias;               /* backward: (channels) when has_bias */
+    void *workspace;
+    size_t workspace_bytes;
+    void *stream;               /* hipStream_t */
+} bimamba2_conv_params;
+
+size_t bimamba2_conv_params_size(void);
+size_t bimamba2_conv1d_silu_workspace_bytes(const bimamba2_conv_params *p);
+/* x weight [bias] -> out */
+int bimamba2_conv1d_silu_fwd(const bimamba2_conv_params *p);
+/* x weight [bias] dout -> dx dweight [dbias] */
+int bimamba2_conv1d_silu_bwd(const bimamba2_conv_params *p);
+
 #ifdef __cplusplus
 }
 #endif
