@@ -110,6 +110,51 @@ def rmsnorm_line(w, dtype, dev, reps):
             "fwd_GBs": round(3 * e * rows * cols / t_f / 1e3, 1), "bwd_GBs": round(5 * e * rows * cols / t_b / 1e3, 1)}
 
 
+def conv_line(w, dtype, dev, reps):
+    """The layer's depthwise conv1d + SiLU at the workload's size (channels = nheads * headdim + 2 * ngroups * dstate, read
+    as a view of a wider projection output): durations of the forward and the backward pass through autograd
+    (host wrapper included), their algorithmic HBM rates, and torch's transposes + nn.Conv1d + SiLU on the same view."""
+    import torch
+    import torch.nn.functional as F
+    from bi_mamba2_amd.conv1d import conv1d_silu_fn
+    batch, L = w["batch"], w["seqlen"]
+    C = w["nheads"] * w["headdim"] + 2 * w["ngroups"] * w["dstate"]
+    wide = torch.randn(batch, L, 2 * C + 64, device=dev).to(dtype)
+    x = wide[..., C:2 * C].detach().requires_grad_(True)
+    wt = (torch.randn(C, 1, 7, device=dev) * 0.3).to(dtype).requires_grad_(True)
+    bias = torch.zeros(C, device=dev, dtype=dtype).requires_grad_(True)
+    dy = torch.randn(batch, L, C, device=dev).to(dtype)
+    e = x.element_size()
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(reps):
+            fn()
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) * 1e3 / reps
+
+    def ours_fwd():
+        with torch.no_grad():
+            conv1d_silu_fn(x, wt, bias)
+
+    def ours_step():
+        torch.autograd.grad(conv1d_silu_fn(x, wt, bias), (x, wt, bias), dy)
+
+    def torch_step():
+        y = F.silu(F.conv1d(x.transpose(1, 2), wt, bias, padding=3, groups=C)).transpose(1, 2)
+        torch.autograd.grad(y, (x, wt, bias), dy)
+
+    t_f, t_s, t_t = timed(ours_fwd), timed(ours_step), timed(torch_step)
+    n = batch * L * C
+    return {"rows": batch * L, "channels": C, "width": 7, "fwd_us": round(t_f, 2), "fwd_bwd_us": round(t_s, 2),
+            "fwd_GBs": round(2 * e * n / t_f / 1e3, 1), "fwd_bwd_GBs": round(5 * e * n / t_s / 1e3, 1),
+            "torch_conv1d_fwd_bwd_us": round(t_t, 2)}
+
+
 def whole_op_bytes(w, e, has_z):
     B, L, H, P, G, N = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate"))
     T4, T2, T1 = B * L * H * P, B * L * G * N, B * L * H
@@ -336,6 +381,7 @@ def main():
                                       "kernels with the reverse direction compiled out, same shape and dtypes"},
         "kernels": kernels,
         "gated_rmsnorm": rmsnorm_line(w, dtype, dev, max(10, args.steps)),
+        "conv1d_silu": conv_line(w, dtype, dev, max(10, args.steps)),
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w)

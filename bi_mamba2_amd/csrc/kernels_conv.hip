@@ -232,10 +232,8 @@ static int launch_conv_w(const bimamba2_conv_params *p, bool bwd) {
     return check_launch();
 }
 
-template <typename T>
-static int launch_conv_t(const bimamba2_conv_params *p, bool bwd) {
-    // 4 channels per thread (8- resp. 16-byte accesses) when the rows allow it, else one
-    constexpr int VS = 4;
+template <typename T, int VS>
+static int launch_conv_vs(const bimamba2_conv_params *p, bool bwd) {
     auto al = [](const void *q, size_t a) { return (reinterpret_cast<uintptr_t>(q) % a) == 0; };
     const size_t va = sizeof(T) * VS;
     bool vec = p->channels % VS == 0 && al(p->x, va) && p->x_sb % VS == 0 && p->x_sl % VS == 0;
@@ -252,6 +250,13 @@ static int launch_conv_t(const bimamba2_conv_params *p, bool bwd) {
         default: return BIMAMBA2_EUNSUPPORTED;
     }
 #undef BM2_CONV
+}
+
+// two channels per thread when the rows allow it (else one): measured faster than four or eight - the backward pass has
+// three register windows plus the filter-gradient sums per channel, and more, narrower threads hide the load latency better
+template <typename T>
+static int launch_conv_t(const bimamba2_conv_params *p, bool bwd) {
+    return launch_conv_vs<T, 2>(p, bwd);
 }
 
 int launch_conv1d_silu(const bimamba2_conv_params *p, bool bwd) {
