@@ -30,7 +30,8 @@ class Params(ctypes.Structure):
                               "dt_out", "cs_f", "cs_b", "CB", "dCB", "CBT", "dCBT", "states_f", "states_b",
                               "dstates_f", "dstates_b", "dout_x",
                               "ddt_direct", "u_f", "u_b", "v_f", "v_b", "da_intra",
-                              "ddA_chunk_f", "ddA_chunk_b", "dBs", "dCs", "red", "workspace")]
+                              "ddA_chunk_f", "ddA_chunk_b", "dBs", "dCs", "red",
+                              "initial_f", "initial_b", "dfinal_f", "dfinal_b", "dinitial_f", "dinitial_b", "workspace")]
         + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
     )
 

@@ -142,8 +142,9 @@ int launch_bwd_dz(const bimamba2_params *p) {
 // =========================================================================================================
 // adjoint of the inter-chunk recurrences.  On entry dstates_* hold the gradient w.r.t. the state entering
 // each chunk (dprev); on exit they hold the gradient w.r.t. each chunk's own state S[c]:
-//   forward dir : g = 0; for c = nc-1..0 : dS_f[c] = g; ddA_chunk_f[c] = e^{tot_c} <g, prev_f[c]>; g = dprev_f[c] + e^{tot_c} g
-//   reverse dir : g = 0; for c = 0..nc-1 : dS_b[c] = g; ddA_chunk_b[c] = e^{tot_c} <g, prev_b[c]>; g = dprev_b[c] + e^{tot_c} g
+//   forward dir : g = dfinal_f (or 0); for c = nc-1..0 : dS_f[c] = g; ddA_chunk_f[c] = e^{tot_c} <g, prev_f[c]>; g = dprev_f[c] + e^{tot_c} g
+//   reverse dir : g = dfinal_b (or 0); for c = 0..nc-1 : dS_b[c] = g; ddA_chunk_b[c] = e^{tot_c} <g, prev_b[c]>; g = dprev_b[c] + e^{tot_c} g
+// What g holds at the end is the gradient with respect to the initial state (written to dinitial_* when given).
 // A workgroup owns SP_EPT*256 of the P*N elements of one (b, h); its partial inner products go to
 // ddA_chunk_*[b, h, c, split].
 // =========================================================================================================
@@ -163,9 +164,15 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_kernel(const bimam
         const float *prev = (dir == 0 ? p.states_f : p.states_b) + base;
         float *ds = (dir == 0 ? p.dstates_f : p.dstates_b) + base;
         float *dda = (dir == 0 ? p.ddA_chunk_f : p.ddA_chunk_b) + ((int64_t)b * p.nheads + h) * nc * nsplit + split;
+        const float *dfin = dir == 0 ? p.dfinal_f : p.dfinal_b;
+        float *dini = dir == 0 ? p.dinitial_f : p.dinitial_b;
+        const int64_t bh = ((int64_t)b * p.nheads + h) * PN;
         float g[SP_EPT];
 #pragma unroll
-        for (int i = 0; i < SP_EPT; ++i) g[i] = 0.f;
+        for (int i = 0; i < SP_EPT; ++i) {
+            const int e = e0 + i * NTHREADS;
+            g[i] = (dfin && e < PN) ? dfin[bh + e] : 0.f;
+        }
         for (int step = 0; step < nc; ++step) {
             const int c = dir == 0 ? nc - 1 - step : step;
             const float dec = __expf(dir == 0 ? csf[(int64_t)c * Q + Q - 1] : csb[(int64_t)c * Q]);
@@ -185,6 +192,13 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_kernel(const bimam
             if (lane == 0) red[step & 1][wave] = dot;
             __syncthreads();
             if (threadIdx.x == 0) dda[(int64_t)c * nsplit] = dec * (red[step & 1][0] + red[step & 1][1] + red[step & 1][2] + red[step & 1][3]);
+        }
+        if (dini) {
+#pragma unroll
+            for (int i = 0; i < SP_EPT; ++i) {
+                const int e = e0 + i * NTHREADS;
+                if (e < PN) dini[bh + e] = g[i];
+            }
         }
         __syncthreads();
     }
@@ -209,7 +223,11 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const b
     const float *prev = (dir == 0 ? p.states_f : p.states_b) + base + e;
     float *ds = (dir == 0 ? p.dstates_f : p.dstates_b) + base + e;
     float *dda = (dir == 0 ? p.ddA_chunk_f : p.ddA_chunk_b) + ((int64_t)b * p.nheads + h) * nc * nsplit + split;
+    const float *dfin = dir == 0 ? p.dfinal_f : p.dfinal_b;
+    float *dini = dir == 0 ? p.dinitial_f : p.dinitial_b;
+    const int64_t bh = ((int64_t)b * p.nheads + h) * PN + e;
     f32x4 g = {0.f, 0.f, 0.f, 0.f};
+    if (dfin) g = *reinterpret_cast<const f32x4 *>(dfin + bh);
     for (int s0 = 0; s0 < nc; s0 += SP_CH) {
         const int nb = min(SP_CH, nc - s0);
         f32x4 dp[SP_CH], pv[SP_CH];
@@ -244,6 +262,7 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const b
         }
         __syncthreads();
     }
+    if (dini && live) *reinterpret_cast<f32x4 *>(dini + bh) = g;
 }
 
 int launch_state_passing_bwd(const bimamba2_params *p) {
@@ -251,7 +270,8 @@ int launch_state_passing_bwd(const bimamba2_params *p) {
     const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS);
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     const int ndir = p->causal ? 1 : 2;
-    if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->dstates_f) && al(p->dstates_b)) {
+    if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->dstates_f) && al(p->dstates_b) && al(p->dfinal_f) && al(p->dfinal_b) &&
+        al(p->dinitial_f) && al(p->dinitial_b)) {
         dim3 grid(nsplit, p->nheads, p->batch * ndir);
         hipLaunchKernelGGL(state_passing_bwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit, ndir);
         return check_launch();

@@ -440,7 +440,7 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_kernel(const bimam
     const int64_t cstride = (int64_t)p.nheads * PN;
     float *sf = p.states_f + ((int64_t)b * nc * p.nheads + h) * PN + e;
     float *sb = p.states_b + ((int64_t)b * nc * p.nheads + h) * PN + e;
-    float s = 0.f;
+    float s = p.initial_f ? p.initial_f[((int64_t)b * p.nheads + h) * PN + e] : 0.f;
     for (int c0 = 0; c0 < nc; c0 += 8) {
         float v[8], d[8];
 #pragma unroll
@@ -457,7 +457,7 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_kernel(const bimam
             }
     }
     if (p.final_f) p.final_f[((int64_t)b * p.nheads + h) * PN + e] = s;
-    s = 0.f;
+    s = p.initial_b ? p.initial_b[((int64_t)b * p.nheads + h) * PN + e] : 0.f;
     for (int c0 = nc - 1; c0 >= 0; c0 -= 8) {
         float v[8], d[8];
 #pragma unroll
@@ -586,7 +586,9 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const b
     const float *cs = (dir == 0 ? p.cs_f : p.cs_b) + ((int64_t)b * p.nheads + h) * nc * Q + (dir == 0 ? Q - 1 : 0);
     const int64_t cstride = (int64_t)p.nheads * PN;
     float *st = (dir == 0 ? p.states_f : p.states_b) + ((int64_t)b * nc * p.nheads + h) * PN + e;
+    const float *ini = dir == 0 ? p.initial_f : p.initial_b;
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    if (ini) s = *reinterpret_cast<const f32x4 *>(ini + ((int64_t)b * p.nheads + h) * PN + e);
     for (int s0 = 0; s0 < nc; s0 += 8) {
         f32x4 v[8];
         float d[8];
@@ -612,7 +614,7 @@ int launch_state_passing_fwd(const bimamba2_params *p) {
     const int nc = nchunks(p), PN = p->headdim * p->dstate;
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     const int ndir = p->causal ? 1 : 2;
-    if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->final_f) && al(p->final_b)) {
+    if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->final_f) && al(p->final_b) && al(p->initial_f) && al(p->initial_b)) {
         dim3 grid((PN / 4 + NTHREADS - 1) / NTHREADS, p->nheads, p->batch * ndir);
         hipLaunchKernelGGL(state_passing_fwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, ndir);
         return check_launch();

@@ -438,8 +438,20 @@ def _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit):
     return c
 
 
+def _set_states(c, fields, states, x, B):
+    """Points the two (batch, nheads, headdim, dstate) float32 fields at the given tensors (None entries stay NULL)."""
+    if states is None:
+        return
+    shape = (x.shape[0], x.shape[2], x.shape[3], B.shape[3])
+    for field, t in zip(fields, states):
+        if t is not None:
+            assert tuple(t.shape) == shape, f"{field}: expected {shape}, got {tuple(t.shape)}"
+            c.put(field, _f32c(t), torch.float32)
+
+
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
-                                   dt_limit=(0.0, _INF), return_intermediates=True, keep_for_bwd=False, causal=False):
+                                   dt_limit=(0.0, _INF), return_intermediates=True, keep_for_bwd=False, causal=False,
+                                   initial_states=None):
     """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
     like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
     out, out_x and the final states are materialised as tensors (the rest lives in a workspace).
@@ -447,9 +459,11 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     _mamba_chunk_scan_combined_bwd accepts as `saved` to skip its recomputation (snapshot: the input half of the
     parameter block, reused when the backward pass gets the same tensors).
     causal=True runs the single-direction operator (see causal_chunk_scan_combined): no reverse states, final_states_b
-    is None."""
+    is None.  initial_states = (initial_f, initial_b), each (batch, nheads, headdim, dstate) or None: the state of the
+    forward recurrence in front of the first position and of the reverse recurrence behind the last one."""
     c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
     c.p.causal = 1 if causal else 0
+    _set_states(c, ("initial_f", "initial_b"), initial_states, x, B)
     batch, seqlen, nheads, headdim = x.shape
     ngroups, dstate = B.shape[2], B.shape[3]
     snap = c.snapshot() if keep_for_bwd else None
@@ -474,11 +488,12 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
 def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
                                    dfinal_states=None, dt_softplus=False, dt_limit=(0.0, _INF),
                                    dx=None, ddt=None, dB=None, dC=None, dz=None, recompute_output=False, saved=None,
-                                   causal=False):
+                                   causal=False, initial_states=None):
     """Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias).  `out` must be the pre-gate output out_x when z is
     given (it is what the autograd function saves); it is not read otherwise.  `saved` is the tuple the forward
-    returns with keep_for_bwd=True; without it the forward intermediates are recomputed, as in the reference."""
-    assert dfinal_states is None, "final states are not supported in the backward pass"
+    returns with keep_for_bwd=True; without it the forward intermediates are recomputed, as in the reference.
+    dfinal_states = (dfinal_f, dfinal_b): gradients with respect to the final states (None entries count as zero).
+    With initial_states = (initial_f, initial_b) given, the result has a ninth element (dinitial_f, dinitial_b)."""
     assert not recompute_output, "recompute_output is not supported"
     assert dout.shape == x.shape
     snap = saved[5] if saved is not None and len(saved) > 5 else None
@@ -494,6 +509,14 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
         c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
     c.p.causal = 1 if causal else 0
     batch, seqlen, nheads, headdim = x.shape
+    c.p.initial_f = c.p.initial_b = None          # (a snapshot of the forward call may carry them)
+    _set_states(c, ("initial_f", "initial_b"), initial_states, x, B)
+    _set_states(c, ("dfinal_f", "dfinal_b"), dfinal_states, x, B)
+    dinit = None
+    if initial_states is not None:
+        sshape = (batch, nheads, headdim, B.shape[3])
+        dinit = tuple(c.new(f, sshape) if t is not None else None
+                      for f, t in zip(("dinitial_f", "dinitial_b"), initial_states))
     c.set_dout(dout)
     if saved is not None:
         for name, t in zip(("dt_out", "cs_f", "cs_b", "states_f", "states_b"), saved[:5]):
@@ -512,9 +535,10 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     ddt_bias = c.new("ddt_bias", (nheads,)) if dt_bias is not None else None
     c.workspace(True)
     c.run("bimamba2_bwd")
-    return (dx, ddt, dA.to(A.dtype), dB.to(B.dtype), dC.to(C.dtype),
-            dD.to(D.dtype) if dD is not None else None, dz,
-            ddt_bias.to(dt_bias.dtype) if ddt_bias is not None else None)
+    res = (dx, ddt, dA.to(A.dtype), dB.to(B.dtype), dC.to(C.dtype),
+           dD.to(D.dtype) if dD is not None else None, dz,
+           ddt_bias.to(dt_bias.dtype) if ddt_bias is not None else None)
+    return res + (dinit,) if dinit is not None else res
 
 
 # True: the autograd function keeps the forward's small and state intermediates for the backward pass (about
@@ -528,40 +552,55 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
-                dt_limit=(0.0, _INF), return_final_states=False):
+                dt_limit=(0.0, _INF), return_final_states=False, *initial_states):
+        # initial_states: nothing (as in the reference), or (initial_states_f, initial_states_b) - an extension
+        assert len(initial_states) in (0, 2)
         ctx.dt_dtype = dt.dtype
+        init = tuple(initial_states) if any(t is not None for t in initial_states) else None
         keep = KEEP_FORWARD_INTERMEDIATES and any(
-            t is not None and t.requires_grad for t in (x, dt, A, B, C, D, z, dt_bias))
+            t is not None and t.requires_grad for t in (x, dt, A, B, C, D, z, dt_bias) + tuple(initial_states))
         res = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit,
-            return_intermediates=False, keep_for_bwd=keep)
+            return_intermediates=False, keep_for_bwd=keep, initial_states=init)
         out, out_x, ff, fb = res[0], res[1], res[7], res[8]
         saved = res[9] if keep else ()
         ctx.n_saved = len(saved)
         ctx.snap = saved[5] if keep else None
-        ctx.save_for_backward(out_x if z is not None else None, x, dt, A, B, C, D, z, dt_bias, *saved[:5])
+        ctx.n_init = len(initial_states)
+        ctx.save_for_backward(out_x if z is not None else None, x, dt, A, B, C, D, z, dt_bias,
+                              *(initial_states if ctx.n_init else (None, None)), *saved[:5])
         ctx.dt_softplus = dt_softplus
         ctx.chunk_size = chunk_size
         ctx.dt_limit = dt_limit
         ctx.return_final_states = return_final_states
         if not return_final_states:
             return out
-        ctx.mark_non_differentiable(ff, fb)
+        # unlike the reference (which refuses a backward pass when final states were returned), gradients flow through
+        # the final states; an unused one arrives as None
+        ctx.set_materialize_grads(False)
         return out, ff, fb
 
     @staticmethod
-    def backward(ctx, dout, *args):
-        out_x, x, dt, A, B, C, D, z, dt_bias = ctx.saved_tensors[:9]
-        saved = tuple(ctx.saved_tensors[9:]) + (ctx.snap,) if ctx.n_saved else None
-        assert not ctx.return_final_states, "final states are not currently supported in the bwd pass"
-        dx, ddt, dA, dB, dC, dD, dz, ddt_bias = _mamba_chunk_scan_combined_bwd(
+    def backward(ctx, dout, *dfinal):
+        out_x, x, dt, A, B, C, D, z, dt_bias, init_f, init_b = ctx.saved_tensors[:11]
+        saved = tuple(ctx.saved_tensors[11:]) + (ctx.snap,) if ctx.n_saved else None
+        if dout is None:
+            dout = torch.zeros_like(x)
+        init = (init_f, init_b) if (init_f is not None or init_b is not None) else None
+        dfin = tuple(dfinal) if any(t is not None for t in dfinal) else None
+        res = _mamba_chunk_scan_combined_bwd(
             dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
-            dt_limit=ctx.dt_limit, saved=saved)
-        return dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, None, None, None
+            dt_limit=ctx.dt_limit, saved=saved, dfinal_states=dfin, initial_states=init)
+        dx, ddt, dA, dB, dC, dD, dz, ddt_bias = res[:8]
+        grads = (dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, None, None, None)
+        if ctx.n_init:
+            grads += tuple(res[8]) if init is not None else (None, None)
+        return grads
 
 
 def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
-                                dt_limit=(0.0, _INF), return_final_states=False):
+                                dt_limit=(0.0, _INF), return_final_states=False, initial_states_f=None,
+                                initial_states_b=None):
     """Bidirectional SSD:  y = SS(x) + flip(SS(flip(x))) + D*x, gated by silu(z) when z is given.
 
     Argument:
@@ -577,11 +616,19 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
         dt_softplus: whether to apply softplus to dt (+ dt_bias)
         dt_limit: clamp range for the transformed dt
     Return:
+        initial_states_f, initial_states_b: (batch, nheads, headdim, dstate), optional - not in the reference, whose
+            bidirectional path starts both recurrences from zero: the state of the forward recurrence in front of the
+            first position and of the reverse recurrence behind the last one (e.g. the final states of the
+            neighbouring pieces of a longer sequence).  Gradients flow into them and through the final states.
+    Return:
         out: (batch, seqlen, nheads, headdim), or (out, final_states_f, final_states_b) with
         return_final_states=True (final states are (batch, nheads, headdim, dstate) float32)
     """
+    if initial_states_f is None and initial_states_b is None:
+        return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
+                                              return_final_states)
     return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
-                                          return_final_states)
+                                          return_final_states, initial_states_f, initial_states_b)
 
 
 class CausalChunkScanCombinedFn(torch.autograd.Function):

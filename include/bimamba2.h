@@ -94,6 +94,17 @@ typedef struct bimamba2_params {
     float *dBs, *dCs;                   /* (S, B, L, G, N) float32 partial gradients, S = ceil(H/G/4) head slices */
     float *red;                         /* scratch for two-stage reductions: max(B*nc*H*P, 2*B*nc*H) floats for the single
                                            stages, B*nc*H*P + 2*B*nc*H for bimamba2_bwd */
+    /* States at the ends of the sequence, all (B, H, P, N) float32, all optional (NULL = absent).  The reference's
+       bidirectional path has neither initial states nor a backward pass through its final states
+       (README.md:66, src/ssd/bi/ssd_combined.py:571 there); they are what chunked / streaming use and a split of the
+       sequence over devices need.
+       initial_f: state of the forward recurrence in front of position 0 (instead of 0);
+       initial_b: state of the reverse recurrence behind position L-1.
+       dfinal_f, dfinal_b (backward): gradients with respect to final_f, final_b.
+       dinitial_f, dinitial_b (backward, outputs): gradients with respect to initial_f, initial_b. */
+    const float *initial_f, *initial_b;
+    const float *dfinal_f, *dfinal_b;
+    float *dinitial_f, *dinitial_b;
     void *workspace;
     size_t workspace_bytes;
     void *stream;                   /* hipStream_t */
@@ -143,7 +154,7 @@ int bimamba2_bmm_chunk_fwd(const bimamba2_params *p);
  * (src/ssd/bi/ssd_chunk_state.py:764-798). */
 int bimamba2_chunk_state_fwd(const bimamba2_params *p);
 /* states_f/b (chunk states) -> states_f/b (state entering each chunk), in place, both directions in one
- * launch; optional final_f/final_b.  Replaces the two _state_passing_fwd calls
+ * launch; optional final_f/final_b and initial_f/initial_b.  Replaces the two _state_passing_fwd calls
  * (src/ssd/bi/ssd_state_passing.py:190-207; src/ssd/bi/ssd_combined.py:324-327). */
 int bimamba2_state_passing_fwd(const bimamba2_params *p);
 /* CB, x, z, dt_out, cs_f, cs_b, Cm, Bm, states_f/b, D -> out, out_x.  Replaces _chunk_scan_fwd
@@ -157,8 +168,8 @@ int bimamba2_chunk_scan_bwd_dz(const bimamba2_params *p);
 /* dout (dout_x when has_z), Cm, cs_f, cs_b -> dstates_f/b.  Replaces _chunk_scan_bwd_dstates
  * (src/ssd/bi/ssd_chunk_scan.py:1801-1826). */
 int bimamba2_chunk_scan_bwd_dstates(const bimamba2_params *p);
-/* states_f/b, dstates_f/b (in place), cs -> dstates_f/b (gradient of each chunk state), ddA_chunk_f/b.
- * Replaces the two _state_passing_bwd calls (src/ssd/bi/ssd_state_passing.py:210-248). */
+/* states_f/b, dstates_f/b (in place), cs [dfinal_f/b] -> dstates_f/b (gradient of each chunk state), ddA_chunk_f/b
+ * [dinitial_f/b].  Replaces the two _state_passing_bwd calls (src/ssd/bi/ssd_state_passing.py:210-248). */
 int bimamba2_state_passing_bwd(const bimamba2_params *p);
 /* -> dx, ddt_direct, dD partials (reduced into dD).  Replaces _chunk_scan_chunk_state_bwd_dx
  * (src/ssd/bi/ssd_combined.py:235-294).  With CBT = NULL, allowed when bimamba2_chunk_scan_reads_cb(p, 1) is 0,

@@ -63,8 +63,10 @@ def _finish(y, x, D, z):
 # 1. literal recurrence
 # --------------------------------------------------------------------------------------------------------
 def bimamba2_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=False,
-                        dt_limit=(0.0, float("inf"))):
-    """Returns (out, out_x, final_f, final_b).  Shapes: x (B,L,H,P), dt (B,L,H), A (H,), B/C (B,L,G,N)."""
+                        dt_limit=(0.0, float("inf")), initial_states_f=None, initial_states_b=None):
+    """Returns (out, out_x, final_f, final_b).  Shapes: x (B,L,H,P), dt (B,L,H), A (H,), B/C (B,L,G,N).
+    initial_states_f / _b (B,H,P,N): where the forward recurrence starts in front of position 0 resp. the reverse one
+    behind position L-1 (zero when absent, as in the reference)."""
     bsz, L, H, P = x.shape
     dtp = dt_transform(dt, dt_bias, dt_softplus, dt_limit)
     Bh, Ch = _expand_groups(B, H), _expand_groups(C, H)
@@ -72,12 +74,12 @@ def bimamba2_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplu
     decay = torch.exp(dtp * A.to(dtp.dtype))                       # (B, L, H)
     inj = (dtp[..., None, None] * x[..., :, None]) * Bh[..., None, :]  # (B, L, H, P, N)
     yf, yb = [None] * L, [None] * L
-    h = x.new_zeros(bsz, H, P, N)
+    h = x.new_zeros(bsz, H, P, N) if initial_states_f is None else initial_states_f
     for t in range(L):
         h = decay[:, t, :, None, None] * h + inj[:, t]
         yf[t] = (h * Ch[:, t, :, None, :]).sum(-1)
     final_f = h
-    g = x.new_zeros(bsz, H, P, N)
+    g = x.new_zeros(bsz, H, P, N) if initial_states_b is None else initial_states_b
     for t in range(L - 1, -1, -1):
         g = decay[:, t, :, None, None] * g + inj[:, t]
         yb[t] = (g * Ch[:, t, :, None, :]).sum(-1)

@@ -152,3 +152,22 @@ def test_causal_operator_against_the_plain_recurrence():
     yb = O.ssd_causal(x.flip(1), dt.flip(1), A, B.flip(1), C.flip(1), 16, **kw)[0].flip(1)
     bi = O.bimamba2_sequential(x, dt, A, B, C, **kw)[0]
     torch.testing.assert_close(yf + yb, bi, rtol=1e-10, atol=1e-10)
+
+
+def test_initial_states_make_a_split_sequence_equal_the_whole():
+    """The oracle's initial states: a sequence cut in two pieces, the second started from the first's final forward
+    state and the first from the second's final reverse state, reproduces the uncut result (outputs and final states)."""
+    inp = to64(make_case(2, 41, 4, 3, 2, 5, with_z=True))
+    x, dt, A, B, C, D, z, bias = (inp[k] for k in ("x", "dt", "A", "B", "C", "D", "z", "dt_bias"))
+    kw = dict(dt_bias=bias, dt_softplus=True)
+    full = O.bimamba2_sequential(x, dt, A, B, C, D=D, z=z, **kw)
+    cut = 17
+    a = lambda t: t[:, :cut]
+    b = lambda t: t[:, cut:]
+    fin_f1 = O.bimamba2_sequential(a(x), a(dt), A, a(B), a(C), D=D, z=a(z), **kw)[2]
+    fin_b2 = O.bimamba2_sequential(b(x), b(dt), A, b(B), b(C), D=D, z=b(z), **kw)[3]
+    r1 = O.bimamba2_sequential(a(x), a(dt), A, a(B), a(C), D=D, z=a(z), initial_states_b=fin_b2, **kw)
+    r2 = O.bimamba2_sequential(b(x), b(dt), A, b(B), b(C), D=D, z=b(z), initial_states_f=fin_f1, **kw)
+    torch.testing.assert_close(torch.cat([r1[0], r2[0]], 1), full[0], rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(r2[2], full[2], rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(r1[3], full[3], rtol=1e-10, atol=1e-10)
