@@ -31,7 +31,8 @@ class Params(ctypes.Structure):
                               "dstates_f", "dstates_b", "dout_x",
                               "ddt_direct", "u_f", "u_b", "v_f", "v_b", "da_intra",
                               "ddA_chunk_f", "ddA_chunk_b", "dBs", "dCs", "red",
-                              "initial_f", "initial_b", "dfinal_f", "dfinal_b", "dinitial_f", "dinitial_b", "workspace")]
+                              "initial_f", "initial_b", "dfinal_f", "dfinal_b", "dinitial_f", "dinitial_b", "seq_idx",
+                              "workspace")]
         + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
     )
 

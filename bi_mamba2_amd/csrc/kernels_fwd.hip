@@ -23,7 +23,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_fwd_kernel(const bimamb
     const DT *dt = reinterpret_cast<const DT *>(p.dt) + b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
     const float A = p.A[h];
     const float bias = p.has_dt_bias ? p.dt_bias[h] : 0.f;
-    float v[4], a[4];
+    float v[4], a[4], ar[4];                          // ar: exponents of the reverse direction (differ with seq_idx only)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int q = lane * 4 + e;
@@ -34,17 +34,26 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_fwd_kernel(const bimamb
             d = fminf(fmaxf(d, p.dt_min), p.dt_max);
         }
         v[e] = d;
-        a[e] = d * A;
+        a[e] = ar[e] = d * A;
+        if (p.seq_idx && q < limit) {
+            // packed sequences: cut the forward recurrence in front of a sequence's first position, the reverse one
+            // behind its last
+            const int l = c * Q + q;
+            const int32_t *si = p.seq_idx + (int64_t)b * p.seqlen + l;
+            const int32_t cur = si[0];
+            if (l > 0 && si[-1] != cur) a[e] += BIMAMBA2_SEQ_CUT;
+            if (l + 1 < p.seqlen && si[1] != cur) ar[e] += BIMAMBA2_SEQ_CUT;
+        }
     }
-    // forward inclusive scan
+    // forward inclusive scan, reverse inclusive scan
     float pf[4], sb[4];
     pf[0] = a[0]; pf[1] = pf[0] + a[1]; pf[2] = pf[1] + a[2]; pf[3] = pf[2] + a[3];
-    sb[3] = a[3]; sb[2] = sb[3] + a[2]; sb[1] = sb[2] + a[1]; sb[0] = sb[1] + a[0];
-    const float tot = pf[3];
+    sb[3] = ar[3]; sb[2] = sb[3] + ar[2]; sb[1] = sb[2] + ar[1]; sb[0] = sb[1] + ar[0];
+    const float tot = pf[3], tot_r = sb[0];
     const float incl = wave_incl_prefix(tot, lane);
     const float before = incl - tot;
-    const float incl_s = wave_incl_suffix(tot, lane);
-    const float after = incl_s - tot;
+    const float incl_s = wave_incl_suffix(tot_r, lane);
+    const float after = incl_s - tot_r;
     const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -569,6 +578,7 @@ int launch_chunk_state(const bimamba2_params *p, bool dstates, bool cumsum) {
 bool chunk_state_does_cumsum(const bimamba2_params *p) {
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
+    if (p->seq_idx) return false;                 // packed sequences: the stand-alone cumsum kernel applies the cuts
     return p->dtype != BIMAMBA2_F32 && p->headdim % 64 == 0 && p->dstate % 64 == 0 && p->chunk_size % 32 == 0 && al(p->Bm) &&
            mult(p->B_sb, p->B_sl, p->B_sg) && al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
 }

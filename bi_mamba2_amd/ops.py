@@ -438,6 +438,14 @@ def _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit):
     return c
 
 
+def _set_seq_idx(c, seq_idx, x):
+    """seq_idx: (batch, seqlen) integer tensor, constant over each packed sequence; None = one sequence per row."""
+    c.p.seq_idx = None
+    if seq_idx is not None:
+        assert tuple(seq_idx.shape) == tuple(x.shape[:2]), "seq_idx: expected (batch, seqlen)"
+        c.put("seq_idx", seq_idx.detach().to(torch.int32).contiguous(), torch.int32)
+
+
 def _set_states(c, fields, states, x, B):
     """Points the two (batch, nheads, headdim, dstate) float32 fields at the given tensors (None entries stay NULL)."""
     if states is None:
@@ -451,7 +459,7 @@ def _set_states(c, fields, states, x, B):
 
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
                                    dt_limit=(0.0, _INF), return_intermediates=True, keep_for_bwd=False, causal=False,
-                                   initial_states=None):
+                                   initial_states=None, seq_idx=None):
     """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
     like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
     out, out_x and the final states are materialised as tensors (the rest lives in a workspace).
@@ -464,6 +472,7 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     c = _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit)
     c.p.causal = 1 if causal else 0
     _set_states(c, ("initial_f", "initial_b"), initial_states, x, B)
+    _set_seq_idx(c, seq_idx, x)
     batch, seqlen, nheads, headdim = x.shape
     ngroups, dstate = B.shape[2], B.shape[3]
     snap = c.snapshot() if keep_for_bwd else None
@@ -488,7 +497,7 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
 def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None, z=None, dt_bias=None,
                                    dfinal_states=None, dt_softplus=False, dt_limit=(0.0, _INF),
                                    dx=None, ddt=None, dB=None, dC=None, dz=None, recompute_output=False, saved=None,
-                                   causal=False, initial_states=None):
+                                   causal=False, initial_states=None, seq_idx=None):
     """Returns (dx, ddt, dA, dB, dC, dD, dz, ddt_bias).  `out` must be the pre-gate output out_x when z is
     given (it is what the autograd function saves); it is not read otherwise.  `saved` is the tuple the forward
     returns with keep_for_bwd=True; without it the forward intermediates are recomputed, as in the reference.
@@ -512,6 +521,7 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     c.p.initial_f = c.p.initial_b = None          # (a snapshot of the forward call may carry them)
     _set_states(c, ("initial_f", "initial_b"), initial_states, x, B)
     _set_states(c, ("dfinal_f", "dfinal_b"), dfinal_states, x, B)
+    _set_seq_idx(c, seq_idx, x)
     dinit = None
     if initial_states is not None:
         sshape = (batch, nheads, headdim, B.shape[3])
@@ -552,16 +562,19 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
-                dt_limit=(0.0, _INF), return_final_states=False, *initial_states):
-        # initial_states: nothing (as in the reference), or (initial_states_f, initial_states_b) - an extension
-        assert len(initial_states) in (0, 2)
+                dt_limit=(0.0, _INF), return_final_states=False, *extra):
+        # extra: nothing (as in the reference), or (initial_states_f, initial_states_b[, seq_idx]) - extensions
+        assert len(extra) in (0, 2, 3)
+        initial_states, seq_idx = tuple(extra[:2]), (extra[2] if len(extra) == 3 else None)
+        ctx.seq_idx = seq_idx
+        ctx.n_extra = len(extra)
         ctx.dt_dtype = dt.dtype
         init = tuple(initial_states) if any(t is not None for t in initial_states) else None
         keep = KEEP_FORWARD_INTERMEDIATES and any(
             t is not None and t.requires_grad for t in (x, dt, A, B, C, D, z, dt_bias) + tuple(initial_states))
         res = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit,
-            return_intermediates=False, keep_for_bwd=keep, initial_states=init)
+            return_intermediates=False, keep_for_bwd=keep, initial_states=init, seq_idx=seq_idx)
         out, out_x, ff, fb = res[0], res[1], res[7], res[8]
         saved = res[9] if keep else ()
         ctx.n_saved = len(saved)
@@ -590,17 +603,19 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
         dfin = tuple(dfinal) if any(t is not None for t in dfinal) else None
         res = _mamba_chunk_scan_combined_bwd(
             dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
-            dt_limit=ctx.dt_limit, saved=saved, dfinal_states=dfin, initial_states=init)
+            dt_limit=ctx.dt_limit, saved=saved, dfinal_states=dfin, initial_states=init, seq_idx=ctx.seq_idx)
         dx, ddt, dA, dB, dC, dD, dz, ddt_bias = res[:8]
         grads = (dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, None, None, None)
         if ctx.n_init:
             grads += tuple(res[8]) if init is not None else (None, None)
+        if ctx.n_extra == 3:
+            grads += (None,)
         return grads
 
 
 def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
                                 dt_limit=(0.0, _INF), return_final_states=False, initial_states_f=None,
-                                initial_states_b=None):
+                                initial_states_b=None, seq_idx=None):
     """Bidirectional SSD:  y = SS(x) + flip(SS(flip(x))) + D*x, gated by silu(z) when z is given.
 
     Argument:
@@ -620,15 +635,21 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
             bidirectional path starts both recurrences from zero: the state of the forward recurrence in front of the
             first position and of the reverse recurrence behind the last one (e.g. the final states of the
             neighbouring pieces of a longer sequence).  Gradients flow into them and through the final states.
+        seq_idx: (batch, seqlen) integers, optional - not in the bidirectional reference (its causal sibling has it):
+            constant over each of several sequences packed one behind the other; positions with different seq_idx do
+            not interact in either direction.
     Return:
         out: (batch, seqlen, nheads, headdim), or (out, final_states_f, final_states_b) with
         return_final_states=True (final states are (batch, nheads, headdim, dstate) float32)
     """
-    if initial_states_f is None and initial_states_b is None:
+    if initial_states_f is None and initial_states_b is None and seq_idx is None:
         return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
                                               return_final_states)
+    if seq_idx is None:
+        return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
+                                              return_final_states, initial_states_f, initial_states_b)
     return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
-                                          return_final_states, initial_states_f, initial_states_b)
+                                          return_final_states, initial_states_f, initial_states_b, seq_idx)
 
 
 class CausalChunkScanCombinedFn(torch.autograd.Function):

@@ -48,6 +48,8 @@ enum {
 #define BIMAMBA2_MAX_HEADDIM 128
 #define BIMAMBA2_MAX_DSTATE 256
 
+#define BIMAMBA2_SEQ_CUT (-64.0f)   /* added to the decay exponent across a change of seq_idx: e^-64 = 1.6e-28 */
+
 typedef struct bimamba2_params {
     /* problem */
     int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
@@ -105,6 +107,13 @@ typedef struct bimamba2_params {
     const float *initial_f, *initial_b;
     const float *dfinal_f, *dfinal_b;
     float *dinitial_f, *dinitial_b;
+    /* Packed sequences (optional): seq_idx (B, L) int32, constant over each of the sequences packed one behind the other
+       along L.  Positions with different seq_idx do not interact: neither recurrence carries state across a change.
+       The bidirectional reference has no such argument (its causal sibling has, src/ssd/uni/ssd_combined.py there).
+       It is applied where the decay exponents are formed (bimamba2_chunk_cumsum_fwd, or bimamba2_fwd / bimamba2_bwd):
+       the forward cumulative sum gets BIMAMBA2_SEQ_CUT added at the first position of a sequence, the reverse one at
+       the last, so that every decay factor across a change underflows to zero and no other kernel needs to know. */
+    const int32_t *seq_idx;
     void *workspace;
     size_t workspace_bytes;
     void *stream;                   /* hipStream_t */

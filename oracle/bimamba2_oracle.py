@@ -63,10 +63,12 @@ def _finish(y, x, D, z):
 # 1. literal recurrence
 # --------------------------------------------------------------------------------------------------------
 def bimamba2_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplus=False,
-                        dt_limit=(0.0, float("inf")), initial_states_f=None, initial_states_b=None):
+                        dt_limit=(0.0, float("inf")), initial_states_f=None, initial_states_b=None, seq_idx=None):
     """Returns (out, out_x, final_f, final_b).  Shapes: x (B,L,H,P), dt (B,L,H), A (H,), B/C (B,L,G,N).
     initial_states_f / _b (B,H,P,N): where the forward recurrence starts in front of position 0 resp. the reverse one
-    behind position L-1 (zero when absent, as in the reference)."""
+    behind position L-1 (zero when absent, as in the reference).  seq_idx (B,L) integers: sequences packed one behind
+    the other; a recurrence restarts from zero wherever seq_idx changes (the causal reference's seq_idx semantics,
+    src/ssd/uni/ssd_chunk_state.py:592-665 there, applied to both directions)."""
     bsz, L, H, P = x.shape
     dtp = dt_transform(dt, dt_bias, dt_softplus, dt_limit)
     Bh, Ch = _expand_groups(B, H), _expand_groups(C, H)
@@ -76,11 +78,15 @@ def bimamba2_sequential(x, dt, A, B, C, D=None, z=None, dt_bias=None, dt_softplu
     yf, yb = [None] * L, [None] * L
     h = x.new_zeros(bsz, H, P, N) if initial_states_f is None else initial_states_f
     for t in range(L):
+        if seq_idx is not None and t > 0:
+            h = h * (seq_idx[:, t] == seq_idx[:, t - 1]).to(h.dtype)[:, None, None, None]
         h = decay[:, t, :, None, None] * h + inj[:, t]
         yf[t] = (h * Ch[:, t, :, None, :]).sum(-1)
     final_f = h
     g = x.new_zeros(bsz, H, P, N) if initial_states_b is None else initial_states_b
     for t in range(L - 1, -1, -1):
+        if seq_idx is not None and t < L - 1:
+            g = g * (seq_idx[:, t] == seq_idx[:, t + 1]).to(g.dtype)[:, None, None, None]
         g = decay[:, t, :, None, None] * g + inj[:, t]
         yb[t] = (g * Ch[:, t, :, None, :]).sum(-1)
     final_b = g

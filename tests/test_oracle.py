@@ -171,3 +171,19 @@ def test_initial_states_make_a_split_sequence_equal_the_whole():
     torch.testing.assert_close(torch.cat([r1[0], r2[0]], 1), full[0], rtol=1e-10, atol=1e-10)
     torch.testing.assert_close(r2[2], full[2], rtol=1e-10, atol=1e-10)
     torch.testing.assert_close(r1[3], full[3], rtol=1e-10, atol=1e-10)
+
+
+def test_packed_sequences_equal_separate_runs():
+    """The oracle's seq_idx: three sequences packed into one row give, piece by piece, what each gives on its own."""
+    inp = to64(make_case(1, 40, 4, 3, 2, 5, with_z=True))
+    x, dt, A, B, C, D, z, bias = (inp[k] for k in ("x", "dt", "A", "B", "C", "D", "z", "dt_bias"))
+    kw = dict(dt_bias=bias, dt_softplus=True)
+    bounds = [0, 13, 14, 40]
+    seq_idx = torch.zeros(1, 40, dtype=torch.int64)
+    for i in range(3):
+        seq_idx[:, bounds[i]:bounds[i + 1]] = i
+    packed = O.bimamba2_sequential(x, dt, A, B, C, D=D, z=z, seq_idx=seq_idx, **kw)[0]
+    for i in range(3):
+        s = slice(bounds[i], bounds[i + 1])
+        alone = O.bimamba2_sequential(x[:, s], dt[:, s], A, B[:, s], C[:, s], D=D, z=z[:, s], **kw)[0]
+        torch.testing.assert_close(packed[:, s], alone, rtol=1e-10, atol=1e-10)
