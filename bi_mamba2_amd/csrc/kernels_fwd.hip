@@ -210,8 +210,9 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
     static_assert(sizeof(T) == 2, "16-bit operands");
-    __shared__ __attribute__((aligned(16))) T xt[BIMAMBA2_MAX_CHUNK * 64];
-    __shared__ __attribute__((aligned(16))) T bt[BIMAMBA2_MAX_CHUNK * 64];
+    constexpr int KR = 4;                                  // ring of K steps (32 positions each): requests run KR - 1 steps ahead
+    __shared__ __attribute__((aligned(16))) T xt[KR * 32 * 64];
+    __shared__ __attribute__((aligned(16))) T bt[KR * 32 * 64];
     __shared__ __attribute__((aligned(16))) float wf[BIMAMBA2_MAX_CHUNK], wb[BIMAMBA2_MAX_CHUNK];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lr = lane & 15, lg = lane >> 4;
@@ -271,12 +272,16 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
             e_b = raw_global_load_f32(p.cs_b + o);
         }
     }
-    for (int s = 0; s < nsteps; ++s) {
-        const int u = 4 * s + wave, row = u * 8 + (lane >> 3);
+    // step s: this wave's 8 rows of the x tile and of the B tile, into slot s % KR (the swizzle of a row does not depend on s)
+    auto issue = [&](int s) {
+        const int row = 32 * s + 8 * wave + (lane >> 3);
         const int col = ((lane & 7) ^ tile64_swz(row)) << 3;
-        load16_to_lds(xp + pt * 64 + (int64_t)min(row, limit - 1) * xs + col, xt + u * 512);
-        load16_to_lds(bp + nt * 64 + (int64_t)min(row, limit - 1) * bs + col, bt + u * 512);
-    }
+        const int at = ((s % KR) * 4 + wave) * 512;
+        load16_to_lds(xp + pt * 64 + (int64_t)min(row, limit - 1) * xs + col, xt + at);
+        load16_to_lds(bp + nt * 64 + (int64_t)min(row, limit - 1) * bs + col, bt + at);
+    };
+    const int nahead = min(KR - 1, nsteps);
+    for (int s = 0; s < nahead; ++s) issue(s);
     auto wait_steps = [&](int newer) {       // at most 2 * newer requests outstanding (newer is wave-uniform, 0..7)
         switch (newer) {
             case 0: wait_vmcnt<0>(); break;
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
         __shared__ float dts[BIMAMBA2_MAX_CHUNK], csfs[BIMAMBA2_MAX_CHUNK], csbs[BIMAMBA2_MAX_CHUNK];
         const unsigned dts_a = lds_addr(dts), csf_a = lds_addr(csfs), csb_a = lds_addr(csbs);
         if (wave == 0) {
-            wait_steps(nsteps);
+            wait_steps(nahead);
             raw_lds_use(A_h); raw_lds_use(bias_h);
 #pragma unroll
             for (int e = 0; e < 4; ++e) raw_lds_use(dt_raw[e]);
@@ -345,7 +350,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
             raw_lds_wait();
         }
     } else {
-        wait_steps(nsteps);
+        wait_steps(nahead);
         raw_lds_use(r_cf); raw_lds_use(r_cb); raw_lds_use(r_dt); raw_lds_use(e_f); raw_lds_use(e_b);
         const int q = threadIdx.x;
         float f = 0.f, r = 0.f;
@@ -370,9 +375,10 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     f32x4 accf[4] = {}, accb[4] = {};
     auto kstep = [&](auto S) {
         constexpr int s = decltype(S)::value;
-        constexpr int TO = s * 32 * 128, WO = s * 32 * 4;      // byte offsets of the step in the tiles / the weight tables
-        wait_steps(nsteps - 1 - s);
-        raw_lds_barrier();
+        constexpr int TO = (s % KR) * 32 * 128, WO = s * 32 * 4;   // byte offsets of the step's slot / in the weight tables
+        wait_steps(min(KR - 2, nsteps - 1 - s));           // this wave's part of step s has landed ...
+        raw_lds_barrier();                                  // ... and everybody's; the slot of step s - 1 is free again
+        if (s + KR - 1 < nsteps) issue(s + KR - 1);
         i16x4 alo = raw_lds_tr16_read_at<TO>(xa_lo), ahi = raw_lds_tr16_read_at<TO>(xa_hi);
         f32x4 f0 = raw_lds_read_at<f32x4, WO>(wfl), f1 = raw_lds_read_at<f32x4, WO + 16>(wfl);
         f32x4 r0 = raw_lds_read_at<f32x4, WO>(wbl), r1 = raw_lds_read_at<f32x4, WO + 16>(wbl);
