@@ -28,11 +28,11 @@ WORKLOAD = dict(batch=4, seqlen=2048, nheads=32, headdim=64, ngroups=1, dstate=6
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
 # size); None until measured for the kernel in question.  Source: the summaries under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "bimamba2_chunk_scan_bwd_dcb": 104.1e6, "bimamba2_chunk_scan_bwd_dc": 90.0e6, "bimamba2_chunk_state_bwd_db": 90.0e6,
-    "bimamba2_chunk_scan_fwd": 213.6e6, "bimamba2_chunk_scan_bwd_dx": 174.7e6, "bimamba2_chunk_scan_bwd_dz": 167.9e6,
-    "bimamba2_state_passing_bwd": 101.9e6, "bimamba2_bmm_chunk_bwd": 61.0e6, "bimamba2_chunk_state_fwd": 78.1e6,
-    "bimamba2_chunk_scan_bwd_dstates": 78.1e6, "bimamba2_state_passing_fwd": 69.5e6, "bimamba2_chunk_cumsum_bwd": 24.3e6,
-    "bimamba2_bmm_chunk_fwd": 23.1e6,
+    "bimamba2_chunk_scan_bwd_dcb": 103.9e6, "bimamba2_chunk_scan_bwd_dc": 89.9e6, "bimamba2_chunk_state_bwd_db": 89.9e6,
+    "bimamba2_chunk_scan_fwd": 203.6e6, "bimamba2_chunk_scan_bwd_dx": 171.8e6, "bimamba2_chunk_scan_bwd_dz": 167.9e6,
+    "bimamba2_state_passing_bwd": 101.9e6, "bimamba2_bmm_chunk_bwd": 61.0e6, "bimamba2_chunk_state_fwd": 78.2e6,
+    "bimamba2_chunk_scan_bwd_dstates": 78.2e6, "bimamba2_state_passing_fwd": 69.5e6, "bimamba2_chunk_cumsum_bwd": 24.3e6,
+    "bimamba2_bmm_chunk_fwd": 23.2e6,
 }
 
 
@@ -202,6 +202,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-z", action="store_true", help="benchmark without the z gate")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the causal comparator and the layer's norm / conv legs (keeps a profile of the run to the operator)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build measures the operator on ONE GPU; --gpus must be 1 "
@@ -256,9 +258,11 @@ def main():
     t_step = timed(step, args.steps)
     t_fwd = timed(fwd_only, args.steps)
     # the single-direction comparator: the same kernels with the reverse direction left out, same shape, same run
-    for _ in range(args.warmup):
-        causal_step()
-    t_causal = timed(causal_step, args.steps)
+    t_causal = None
+    if not args.no_extras:
+        for _ in range(args.warmup):
+            causal_step()
+        t_causal = timed(causal_step, args.steps)
     tokens = w["batch"] * w["seqlen"]
     fwd_b, bwd_b = whole_op_bytes(w, e, has_z)
 
@@ -375,14 +379,16 @@ def main():
                      "fwd_hbm_frac": fwd_b / t_fwd / (HBM_PEAK_GBS * 1e9),
                      "sum_kernel_us": round(sum(k["us"] for k in kernels.values()), 1),
                      "measured_copy_GBs": round(copy_gbs, 1)},
-        "causal_comparator": {"ms_per_step": t_causal * 1e3, "Mtokens_s": tokens / t_causal / 1e6,
-                              "bidirectional_over_causal": t_step / t_causal,
-                              "what": "single-direction SSD (y = SS(x) + D x, z gate) forward + backward from the same "
-                                      "kernels with the reverse direction compiled out, same shape and dtypes"},
         "kernels": kernels,
-        "gated_rmsnorm": rmsnorm_line(w, dtype, dev, max(10, args.steps)),
-        "conv1d_silu": conv_line(w, dtype, dev, max(10, args.steps)),
     }
+    if not args.no_extras:
+        result["causal_comparator"] = {
+            "ms_per_step": t_causal * 1e3, "Mtokens_s": tokens / t_causal / 1e6,
+            "bidirectional_over_causal": t_step / t_causal,
+            "what": "single-direction SSD (y = SS(x) + D x, z gate) forward + backward from the same kernels with the "
+                    "reverse direction compiled out, same shape and dtypes"}
+        result["gated_rmsnorm"] = rmsnorm_line(w, dtype, dev, max(10, args.steps))
+        result["conv1d_silu"] = conv_line(w, dtype, dev, max(10, args.steps))
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(result))
