@@ -303,13 +303,18 @@ int bimamba2_bwd(const bimamba2_params *p) {
     TRY(bimamba2_chunk_state_bwd_db(&q));
     TRY(bimamba2_chunk_scan_bwd_dc(&q));
     TRY(bimamba2_chunk_scan_bwd_dcb(&q));
-    TRY(bimamba2_bmm_chunk_bwd(&q));
     {
-        // as bimamba2_chunk_cumsum_bwd, its partial sums behind those of dD
+        // as bimamba2_bmm_chunk_bwd and bimamba2_chunk_cumsum_bwd (its partial sums behind those of dD): one launch for
+        // both where the kernel for it exists
         bimamba2_params qc = q;
         qc.red = q.red + (size_t)q.batch * nchunks(&q) * q.nheads * q.headdim;
-        REQUIRE(q.ddt); REQUIRE(q.dA);
-        TRY(launch_chunk_cumsum_bwd(&qc, &jobs));
+        REQUIRE(q.ddt); REQUIRE(q.dA); REQUIRE(q.dB); REQUIRE(q.dC);
+        if (bwd_tail_merged(&q)) {
+            TRY(launch_bwd_tail(&qc, &jobs));
+        } else {
+            TRY(bimamba2_bmm_chunk_bwd(&q));
+            TRY(launch_chunk_cumsum_bwd(&qc, &jobs));
+        }
     }
     TRY(launch_reduce_jobs(jobs, stream_of(&q)));
     return BIMAMBA2_OK;

@@ -1295,16 +1295,18 @@ int launch_bwd_dcb(const bimamba2_params *p) {
 // =========================================================================================================
 // FAST (16-bit types, chunk_size == QP, dstate a multiple of 64, aligned operands, at most 8 slices): every global load
 // of a thread (its dCB row pieces, the slices it adds, the K operand) is requested before the first one is used.
+struct BlockId { int x, y, z; };
+
 template <typename T, int QP, bool FAST>
-__global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_params p, int nc, int nslices) {
+__device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int nc, int nslices, BlockId bid) {
     typedef Mma<T> M;
     constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
     constexpr int LDX = QP + 16 / (int)sizeof(T);
     __shared__ __attribute__((aligned(16))) T kT[64 * LDX];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lr = lane & 15, lg = lane >> 4;
-    const int nt = blockIdx.x, rt = blockIdx.y;
-    const int which = blockIdx.z & 1, bcg = blockIdx.z >> 1;
+    const int nt = bid.x, rt = bid.y;
+    const int which = bid.z & 1, bcg = bid.z >> 1;
     const int g = bcg % p.ngroups, bc = bcg / p.ngroups, c = bc % nc, b = bc / nc;
     const int Q = p.chunk_size, N = p.dstate;
     const int limit = min(Q, p.seqlen - c * Q);
@@ -1327,7 +1329,10 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
             raw[s][0] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL);
             raw[s][1] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL + 4);
         }
-        float4 sv[NIT][MAXSL][2];
+        // slices: the first half is requested here, the second half after the products, into the registers of the row pieces
+        // (keeps the kernel at two workgroups per CU)
+        constexpr int HSL = MAXSL / 2;
+        float4 sv[NIT][HSL][2];
         int64_t oa[NIT];
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
@@ -1336,7 +1341,7 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
             const int r = min(r0 + rl, limit - 1);
             oa[it] = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + nt * 64 + cc;
 #pragma unroll
-            for (int sl = 0; sl < MAXSL; ++sl) {
+            for (int sl = 0; sl < HSL; ++sl) {
                 const float *q = res + oa[it] + (int64_t)min(sl, nslices - 1) * slice;
                 sv[it][sl][0] = *reinterpret_cast<const float4 *>(q);
                 sv[it][sl][1] = *reinterpret_cast<const float4 *>(q + 4);
@@ -1354,6 +1359,15 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
                 for (int j = 0; j < 4; ++j) acc[j] = M::mma(af, M::load(kT + xt_index<T, LDX>(j * 16 + lr, s * KSTEP + lg * KPL)), acc[j]);
             }
         }
+        float4 sw[NIT][HSL][2];
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+            for (int sl = 0; sl < HSL; ++sl) {
+                const float *q = res + oa[it] + (int64_t)min(HSL + sl, nslices - 1) * slice;
+                sw[it][sl][0] = *reinterpret_cast<const float4 *>(q);
+                sw[it][sl][1] = *reinterpret_cast<const float4 *>(q + 4);
+            }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -1369,8 +1383,9 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
 #pragma unroll
             for (int sl = 0; sl < MAXSL; ++sl) {
                 if (sl < nslices) {
-                    v[0] += sv[it][sl][0].x; v[1] += sv[it][sl][0].y; v[2] += sv[it][sl][0].z; v[3] += sv[it][sl][0].w;
-                    v[4] += sv[it][sl][1].x; v[5] += sv[it][sl][1].y; v[6] += sv[it][sl][1].z; v[7] += sv[it][sl][1].w;
+                    const float4 a0 = sl < HSL ? sv[it][sl % HSL][0] : sw[it][sl % HSL][0], a1 = sl < HSL ? sv[it][sl % HSL][1] : sw[it][sl % HSL][1];
+                    v[0] += a0.x; v[1] += a0.y; v[2] += a0.z; v[3] += a0.w;
+                    v[4] += a1.x; v[5] += a1.y; v[6] += a1.z; v[7] += a1.w;
                 }
             }
             if (r0 + rl < limit) {
@@ -1446,6 +1461,11 @@ __global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_
     }
 }
 
+template <typename T, int QP, bool FAST>
+__global__ __launch_bounds__(NTHREADS) void bmm_chunk_bwd_kernel(const bimamba2_params p, int nc, int nslices) {
+    bmm_chunk_bwd_body<T, QP, FAST>(p, nc, nslices, BlockId{(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z});
+}
+
 template <typename T>
 static int launch_bmm_bwd_t(const bimamba2_params *p) {
     const int nc = nchunks(p), Q = p->chunk_size, nsl = dbdc_slices(p);
@@ -1486,9 +1506,9 @@ int launch_bmm_chunk_bwd(const bimamba2_params *p) {
 // Partials per (b, c) go to red[(b*nc + c)*H + h] (dA) and red[B*nc*H + ...] (ddt_bias).
 // =========================================================================================================
 template <typename DT>
-__global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamba2_params p, int nc, int nqt, int nsplit) {
+__device__ __forceinline__ void chunk_cumsum_bwd_body(const bimamba2_params &p, int nc, int nqt, int nsplit, BlockId bid) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int h = blockIdx.x * 4 + wave, c = blockIdx.y, b = blockIdx.z;
+    const int h = bid.x * 4 + wave, c = bid.y, b = bid.z;
     if (h >= p.nheads) return;
     const int Q = p.chunk_size, H = p.nheads;
     const int limit = min(Q, p.seqlen - c * Q);
@@ -1624,6 +1644,68 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
         p.red[(int64_t)(b * nc + c) * H + h] = sA;
         p.red[(int64_t)p.batch * nc * H + (int64_t)(b * nc + c) * H + h] = sb;
     }
+}
+
+template <typename DT>
+__global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamba2_params p, int nc, int nqt, int nsplit) {
+    chunk_cumsum_bwd_body<DT>(p, nc, nqt, nsplit, BlockId{(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z});
+}
+
+// The last two kernels of the backward pass in one launch: the first `nbmm` workgroups do the work of
+// bmm_chunk_bwd_kernel (16-bit path, chunk_size 256), the others that of chunk_cumsum_bwd_kernel.  Neither depends on the
+// other, both are short and latency-bound, and together they fit the machine in one wave of workgroups.
+template <typename T, typename DT>
+__global__ __launch_bounds__(NTHREADS) void bwd_tail_kernel(const bimamba2_params p, int nc, int nslices, int nqt, int nsplit, int nbmm,
+                                                            int bmm_gy, int cs_gx) {
+    const int id = blockIdx.x;
+    if (id < nbmm) {
+        // bmm grid (1, bmm_gy, z)
+        bmm_chunk_bwd_body<T, 256, true>(p, nc, nslices, BlockId{0, id % bmm_gy, id / bmm_gy});
+    } else {
+        const int k = id - nbmm;                  // cumsum grid (cs_gx, nc, batch)
+        chunk_cumsum_bwd_body<DT>(p, nc, nqt, nsplit, BlockId{k % cs_gx, (k / cs_gx) % nc, k / (cs_gx * nc)});
+    }
+}
+
+static bool bmm_bwd_fast(const bimamba2_params *p) {
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
+    const int Q = p->chunk_size;
+    return p->dtype != BIMAMBA2_F32 && (Q == 64 || Q == 128 || Q == 256) && p->dstate % 64 == 0 && dbdc_slices(p) <= 8 && al(p->Bm) &&
+           al(p->Cm) && mult(p->B_sb, p->B_sl, p->B_sg) && mult(p->C_sb, p->C_sl, p->C_sg) && al(p->dCB) && al(p->dCBT) && al(p->dBs) &&
+           al(p->dCs) && al(p->dB) && al(p->dC);
+}
+
+// whether launch_bwd_tail() exists for this problem
+bool bwd_tail_merged(const bimamba2_params *p) { return bmm_bwd_fast(p) && p->chunk_size == 256 && p->dstate == 64; }
+
+template <typename T>
+static int launch_bwd_tail_t(const bimamba2_params *p, int nc, int nqt, int nsplit) {
+    const int bmm_gy = (p->chunk_size + 63) / 64, nbmm = bmm_gy * p->batch * nc * p->ngroups * 2;
+    const int cs_gx = (p->nheads + 3) / 4, ncs = cs_gx * nc * p->batch;
+    dim3 grid(nbmm + ncs);
+    const int nsl = dbdc_slices(p);
+    switch (p->dt_dtype) {
+        case BIMAMBA2_F32: hipLaunchKernelGGL((bwd_tail_kernel<T, float>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL((bwd_tail_kernel<T, bf16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL((bwd_tail_kernel<T, f16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx); break;
+        default: return BIMAMBA2_EUNSUPPORTED;
+    }
+    return check_launch();
+}
+
+// bmm_chunk_bwd + chunk_cumsum_bwd in one launch (the caller checked bwd_tail_merged()); reductions as in
+// launch_chunk_cumsum_bwd
+int launch_bwd_tail(const bimamba2_params *p, ReduceJobs *defer) {
+    const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
+    const int PN = p->headdim * p->dstate;
+    const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS);
+    int rc = p->dtype == BIMAMBA2_BF16 ? launch_bwd_tail_t<bf16_t>(p, nc, nqt, nsplit) : launch_bwd_tail_t<f16_t>(p, nc, nqt, nsplit);
+    if (rc) return rc;
+    const int ni = p->batch * nc;
+    defer->job[defer->n++] = ReduceJob{p->red, p->dA, ni, p->nheads, 1};
+    if (p->has_dt_bias && p->ddt_bias) defer->job[defer->n++] = ReduceJob{p->red + (int64_t)ni * p->nheads, p->ddt_bias, ni, p->nheads, 1};
+    return BIMAMBA2_OK;
 }
 
 int launch_chunk_cumsum_bwd(const bimamba2_params *p, ReduceJobs *defer) {
