@@ -41,6 +41,12 @@ __device__ __forceinline__ float raw_global_load_f32(const float *p) {
     asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
     return v;
 }
+template <typename V> __device__ __forceinline__ V raw_global_load_b128(const void *p) {
+    static_assert(sizeof(V) == 16, "16-byte value");
+    V v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
 __device__ __forceinline__ unsigned raw_global_load_u16(const void *p) {      // zero-extended 16 bits
     unsigned v;
     asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p) : "memory");

@@ -512,6 +512,273 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_p
                 }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// The same for 16-bit types with dstate 64 and headdim % 64 == 0, with every load of the head loop taken out of the
+// compiler's hands.  The workgroup is alone on its CU (register-bound), so nothing hides a load it waits for; here the
+// float32 state tiles of a step travel straight into a 3-slot LDS ring (no registers), two steps ahead of their use, and
+// the x / dout fragments into registers, likewise two steps ahead, from inline assembly.  A step then reads its tiles
+// from the ring, transposes them in registers into the 16-bit operand image as before, and multiplies.  All LDS traffic
+// of the loop goes through the raw accessors (an access the compiler knows of would wait for every request in flight).
+// Order of a wave's vector memory operations per step: NDIR * 2 ring requests, then QT * 2 fragment loads; "at most one
+// step's worth outstanding" therefore means that the step in hand has landed.
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, int QT, bool IS_DB, bool UNI>
+__global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamba2_params p, int nc) {
+    typedef Mma<T> M;
+    typedef typename M::Frag Frag;
+    static_assert(sizeof(T) == 2, "16-bit operands");
+    constexpr int KSTEP = 32, KC = 64, NKS = 2, VK = 8, LDX = KC + VK;
+    constexpr int ROWS = DBDC_WAVES * 16 * QT;
+    constexpr int NBLK = (KC / VK) * 16;                       // 8 x 4 blocks of a 64 x 64 tile
+    constexpr int RING = 3, NDIR = UNI ? 1 : 2;
+    constexpr int TILE_B = 64 * 64 * 4;                        // bytes of a float32 state tile
+    constexpr int IMG_B = 64 * LDX * 2;                        // bytes of a 16-bit operand image
+    constexpr int PER_STEP = NDIR * 2 + QT * NKS;              // vector memory operations of a wave per step
+    static_assert(NDIR * NBLK <= DBDC_THREADS, "one block per thread");
+    __shared__ __attribute__((aligned(16))) unsigned char ring[RING * NDIR * TILE_B];
+    __shared__ __attribute__((aligned(16))) unsigned char img[2 * NDIR * IMG_B];
+    __shared__ __attribute__((aligned(16))) float sfs[DBDC_HEADS][ROWS], sbs[DBDC_HEADS][ROWS];
+    // the per-head decay gradients wait here for the end of the kernel: a global store inside the loop would sit in the
+    // same counter as the requests and be waited for with them
+    __shared__ __attribute__((aligned(16))) float uvs[DBDC_HEADS][NDIR][ROWS];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lr = lane & 15, lg = lane >> 4;
+    const int rt = blockIdx.y;
+    const int g = blockIdx.x % p.ngroups, bc = blockIdx.x / p.ngroups, c = bc % nc, b = bc / nc;
+    const int Q = p.chunk_size, N = p.dstate, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int r0 = rt * ROWS;
+    const int hh0 = blockIdx.z * DBDC_HEADS, hh_end = min(hpg, hh0 + DBDC_HEADS);
+    const int nkc = P / KC, nsteps = (hh_end - hh0) * nkc;
+    int arow[QT];
+#pragma unroll
+    for (int q = 0; q < QT; ++q) arow[q] = min(r0 + (wave * QT + q) * 16 + lr, limit - 1);
+
+    // requests of a step: this wave's two 4-row units of each state tile, then its fragments
+    auto issue_states = [&](int step) {
+        const int hh = hh0 + step / nkc, kc = step % nkc, h = g * hpg + hh;
+        const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * N + (int64_t)kc * KC * N;
+#pragma unroll
+        for (int d = 0; d < NDIR; ++d) {
+            const float *st = (IS_DB ? (d ? p.dstates_b : p.dstates_f) : (d ? p.states_b : p.states_f)) + so;
+#pragma unroll
+            for (int uu = 0; uu < 2; ++uu) {
+                const int u = wave * 2 + uu;
+                load16_to_lds(st + (4 * u + (lane >> 4)) * 64 + (lane & 15) * 4, ring + ((step % RING) * NDIR + d) * TILE_B + u * 1024);
+            }
+        }
+    };
+    auto issue_frags = [&](int step, Frag (&af)[QT][NKS]) {
+        const int hh = hh0 + step / nkc, kc = step % nkc, h = g * hpg + hh;
+        const T *ap;
+        int64_t as;
+        if (IS_DB) { as = p.x_sl; ap = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * as + h * p.x_sh; }
+        else if (p.has_z) { as = (int64_t)H * P; ap = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * as + (int64_t)h * P; }
+        else { as = p.dout_sl; ap = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * as + h * p.dout_sh; }
+#pragma unroll
+        for (int q = 0; q < QT; ++q)
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) af[q][ks] = raw_global_load_b128<Frag>(ap + (int64_t)arow[q] * as + kc * KC + ks * KSTEP + lg * 8);
+    };
+    Frag afA[QT][NKS], afB[QT][NKS];                           // fragments of the even / odd steps
+    issue_states(0);
+    issue_frags(0, afA);
+    if (nsteps > 1) { issue_states(1); issue_frags(1, afB); }
+
+    // ---- everything below up to the loop is ordinary code; its waits drain the requests above, which costs nothing here ----
+    int tl[QT][4];
+#pragma unroll
+    for (int q = 0; q < QT; ++q)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tl[q][i] = (wave * QT + q) * 16 + lg * 4 + i;
+    // one round trip for everything the loop needs besides its requests: the decay vectors of the slice's heads and the
+    // B / C values of this lane's output elements, all loaded unconditionally from clamped addresses before the first use
+    constexpr int NTAB = DBDC_HEADS * ROWS / DBDC_THREADS;
+    static_assert(NTAB * DBDC_THREADS == DBDC_HEADS * ROWS, "table entries per thread");
+    float t_dt[NTAB], t_cf[NTAB], t_cb[NTAB], t_ef[NTAB], t_eb[NTAB];
+#pragma unroll
+    for (int it = 0; it < NTAB; ++it) {
+        const int idx = threadIdx.x + it * DBDC_THREADS;
+        const int hh = min(idx / ROWS, hh_end - hh0 - 1), r = min(r0 + idx % ROWS, limit - 1);
+        const int64_t o = (((int64_t)b * H + g * hpg + hh0 + hh) * nc + c) * Q;
+        t_cf[it] = p.cs_f[o + r];
+        t_cb[it] = UNI ? 0.f : p.cs_b[o + r];
+        t_dt[it] = IS_DB ? p.dt_out[o + r] : 0.f;
+        t_ef[it] = IS_DB ? p.cs_f[o + Q - 1] : 0.f;
+        t_eb[it] = (IS_DB && !UNI) ? p.cs_b[o] : 0.f;
+    }
+    const T *cbp;
+    int64_t cbs;
+    if (IS_DB) { cbs = p.B_sl; cbp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + ((int64_t)c * Q + r0) * cbs + g * p.B_sg; }
+    else { cbs = p.C_sl; cbp = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + ((int64_t)c * Q + r0) * cbs + g * p.C_sg; }
+    float creg[QT][4][4];
+#pragma unroll
+    for (int q = 0; q < QT; ++q)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) creg[q][j][i] = to_f(cbp[(int64_t)min(tl[q][i], limit - 1 - r0) * cbs + j * 16 + lr]);
+#pragma unroll
+    for (int q = 0; q < QT; ++q)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (r0 + tl[q][i] >= limit) creg[q][j][i] = 0.f;
+#pragma unroll
+    for (int it = 0; it < NTAB; ++it) {
+        const int idx = threadIdx.x + it * DBDC_THREADS;
+        const int hh = idx / ROWS, rl = idx % ROWS;
+        if (hh < hh_end - hh0) {
+            float f = 0.f, rv = 0.f;
+            if (r0 + rl < limit) {
+                if (IS_DB) {
+                    f = t_dt[it] * __expf(t_ef[it] - t_cf[it]);
+                    rv = UNI ? 0.f : t_dt[it] * __expf(t_eb[it] - t_cb[it]);
+                } else {
+                    f = __expf(t_cf[it]);
+                    rv = UNI ? 0.f : __expf(t_cb[it]);
+                }
+            }
+            sfs[hh][rl] = f;
+            sbs[hh][rl] = rv;
+        }
+    }
+    f32x4 tot[QT][4] = {};
+    __syncthreads();
+
+    // ---- the head loop: raw LDS accesses and counted waits only ----
+    const int sblk = threadIdx.x % NBLK, stile = threadIdx.x / NBLK;       // staging: tile stile, block (s_kb, s_rb)
+    const int s_rb = sblk % 16, s_kb = sblk / 16;
+    const unsigned ring_a = lds_addr(ring) + stile * TILE_B + (s_kb * VK) * 256 + s_rb * 16;
+    const unsigned img_w = lds_addr(img) + stile * IMG_B;
+    unsigned img_wo[4];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) img_wo[rr] = img_w + xt_index<T, LDX>(s_rb * 4 + rr, s_kb * VK) * 2;
+    unsigned img_r[NKS][4];                                    // operand fragments of this lane (the swizzle depends on the row block)
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) img_r[ks][j] = lds_addr(img) + xt_index<T, LDX>(j * 16 + lr, ks * KSTEP + lg * 8) * 2;
+    const unsigned sfs_a = lds_addr(sfs) + ((wave * QT) * 16 + lg * 4) * 4, sbs_a = lds_addr(sbs) + ((wave * QT) * 16 + lg * 4) * 4;
+    const unsigned uvs_a = lds_addr(uvs) + ((wave * QT) * 16 + lg * 4) * 4;
+    f32x4 tf[QT][4], tb[QT][4];
+    auto step_body = [&](int step, Frag (&af)[QT][NKS]) {
+        const int hh = hh0 + step / nkc, kc = step % nkc;
+        // this wave's requests of the step have landed (those of the next step may be outstanding) ...
+        if (step + 1 < nsteps) wait_vmcnt<PER_STEP>();
+        else wait_vmcnt<0>();
+        raw_lds_barrier();                                     // ... and everybody's; ring slot and image of step - 1 are free
+        if (step + 2 < nsteps) issue_states(step + 2);
+        const int buf = step & 1;
+        if (stile < NDIR) {
+            // 8 rows (k = p) x 4 columns (n) of the tile from the ring, transposed into the image
+            const unsigned ra = ring_a + ((step % RING) * NDIR) * TILE_B;
+            f32x4 v[VK];
+            v[0] = raw_lds_read_at<f32x4, 0>(ra); v[1] = raw_lds_read_at<f32x4, 256>(ra);
+            v[2] = raw_lds_read_at<f32x4, 512>(ra); v[3] = raw_lds_read_at<f32x4, 768>(ra);
+            v[4] = raw_lds_read_at<f32x4, 1024>(ra); v[5] = raw_lds_read_at<f32x4, 1280>(ra);
+            v[6] = raw_lds_read_at<f32x4, 1536>(ra); v[7] = raw_lds_read_at<f32x4, 1792>(ra);
+            raw_lds_wait();
+#pragma unroll
+            for (int kk = 0; kk < VK; ++kk) raw_lds_use(v[kk]);
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                Vec16<T> o;
+#pragma unroll
+                for (int kk = 0; kk < VK; ++kk) o.v[kk] = from_f<T>(v[kk][rr]);
+                raw_lds_write128_at<0>(img_wo[rr] + buf * NDIR * IMG_B, __builtin_bit_cast(f32x4, o));
+            }
+        }
+        raw_lds_wait();
+        raw_lds_barrier();
+        if (kc == 0) {
+#pragma unroll
+            for (int q = 0; q < QT; ++q)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { tf[q][j] = f32x4{0.f, 0.f, 0.f, 0.f}; tb[q][j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        }
+#pragma unroll
+        for (int q = 0; q < QT; ++q)
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) raw_lds_use(af[q][ks]);
+        const unsigned ib = buf * NDIR * IMG_B;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            Frag bff[4], bfb[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                bff[j] = raw_lds_read_at<Frag, 0>(img_r[ks][j] + ib);
+                if (!UNI) bfb[j] = raw_lds_read_at<Frag, IMG_B>(img_r[ks][j] + ib);
+            }
+            raw_lds_wait();
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                raw_lds_use(bff[j]);
+                if (!UNI) raw_lds_use(bfb[j]);
+#pragma unroll
+                for (int q = 0; q < QT; ++q) {
+                    tf[q][j] = M::mma(af[q][ks], bff[j], tf[q][j]);
+                    if (!UNI) tb[q][j] = M::mma(af[q][ks], bfb[j], tb[q][j]);
+                }
+            }
+        }
+        // the fragments of step + 2 take the place of the ones just used
+        if (step + 2 < nsteps) issue_frags(step + 2, af);
+        if (kc == nkc - 1) {
+            // ---- end of a head: its share of dB / dC and of the decay gradients
+#pragma unroll
+            for (int q = 0; q < QT; ++q) {
+                f32x4 sf4 = raw_lds_read_at<f32x4, 0>(sfs_a + ((hh - hh0) * ROWS + q * 16) * 4);
+                f32x4 sb4 = raw_lds_read_at<f32x4, 0>(sbs_a + ((hh - hh0) * ROWS + q * 16) * 4);
+                raw_lds_wait();
+                raw_lds_use(sf4); raw_lds_use(sb4);
+                f32x4 av, bv;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float uf = 0.f, ub = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        uf += tf[q][j][i] * creg[q][j][i];
+                        if (!UNI) ub += tb[q][j][i] * creg[q][j][i];
+                        tot[q][j][i] += UNI ? sf4[i] * tf[q][j][i] : sf4[i] * tf[q][j][i] + sb4[i] * tb[q][j][i];
+                    }
+                    av[i] = row16_sum(uf) * sf4[i];
+                    bv[i] = UNI ? 0.f : row16_sum(ub) * sb4[i];
+                }
+                if (lr == 0) {
+                    const unsigned ua = uvs_a + (((hh - hh0) * NDIR) * ROWS + q * 16) * 4;
+                    raw_lds_write128_at<0>(ua, av);
+                    if (!UNI) raw_lds_write128_at<ROWS * 4>(ua, bv);
+                }
+            }
+        }
+    };
+    for (int step = 0; step < nsteps; step += 2) {
+        step_body(step, afA);
+        if (step + 1 < nsteps) step_body(step + 1, afB);
+    }
+    raw_lds_wait();
+    __syncthreads();                                           // nothing is in flight any more: ordinary code again
+    for (int idx = threadIdx.x; idx < (hh_end - hh0) * NDIR * ROWS; idx += DBDC_THREADS) {
+        const int hh = idx / (NDIR * ROWS), d = (idx / ROWS) % NDIR, rl = idx % ROWS;
+        if (r0 + rl < Q) {
+            float *dst = IS_DB ? (d ? p.v_b : p.v_f) : (d ? p.u_b : p.u_f);
+            dst[(((int64_t)b * H + g * hpg + hh0 + hh) * nc + c) * Q + r0 + rl] = uvs[hh][d][rl];
+        }
+    }
+    float *out = (IS_DB ? p.dBs : p.dCs) + (int64_t)blockIdx.z * p.batch * p.seqlen * p.ngroups * N;
+#pragma unroll
+    for (int q = 0; q < QT; ++q)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = j * 16 + lr, r = r0 + tl[q][i];
+                if (r < limit) out[(((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n] = tot[q][j][i];
+            }
+}
+
 template <typename T, bool IS_DB>
 static int launch_dbdc_t(const bimamba2_params *p) {
     const int nc = nchunks(p);
@@ -529,6 +796,20 @@ static int launch_dbdc_t(const bimamba2_params *p) {
         if (fast) hipLaunchKernelGGL((bwd_dbdc_kernel<T, NTV, QTV, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc); \
         else hipLaunchKernelGGL((bwd_dbdc_kernel<T, NTV, QTV, IS_DB, false>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);     \
     } while (0)
+    if constexpr (sizeof(T) == 2) {
+        // dstate 64: the variant with the ring of state tiles (16-byte aligned state tensors)
+        const bool st_al = IS_DB ? al(p->dstates_f) && al(p->dstates_b) : al(p->states_f) && al(p->states_b);
+        if (fast && p->dstate == 64 && st_al && getenv("BM2_DBDC_OLD") == nullptr) {
+            if (p->causal) {
+                if (qt == 2) hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 2, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
+                else hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 1, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
+            } else {
+                if (qt == 2) hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 2, IS_DB, false>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
+                else hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 1, IS_DB, false>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
+            }
+            return check_launch();
+        }
+    }
     if (p->causal) {
         if constexpr (sizeof(T) == 2) {
             if (fast && nt == 1) {
