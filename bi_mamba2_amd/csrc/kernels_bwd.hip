@@ -799,7 +799,7 @@ static int launch_dbdc_t(const bimamba2_params *p) {
     if constexpr (sizeof(T) == 2) {
         // dstate 64: the variant with the ring of state tiles (16-byte aligned state tensors)
         const bool st_al = IS_DB ? al(p->dstates_f) && al(p->dstates_b) : al(p->states_f) && al(p->states_b);
-        if (fast && p->dstate == 64 && st_al && getenv("BM2_DBDC_OLD") == nullptr) {
+        if (fast && p->dstate == 64 && st_al) {
             if (p->causal) {
                 if (qt == 2) hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 2, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
                 else hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 1, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
