@@ -1298,23 +1298,54 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
 #endif
         int slot = 0, slot2 = 2 % DCB_RING, kc = 0, par = 0;
         float *tv = tv0 + (wave & 1) * 64 + lane;
-        for (int it = 0; it < nit; ++it) {
-            if (it + 2 < nit) issue(slot2);
-            TSR(0);
-            // the requests of step `it` went out before those of the (up to two) steps after it; waves 0 and 1 make
-            // five requests per step, the others four
-            const int newer = min(2, nit - 1 - it);
+        // the sums of a head are written out one iteration later, after the barrier that the next step needs anyway
+        // (waves 0 and 1; off-diagonal: [0] = column sums, [1] = row sums.  diagonal: [0] = cw_f - rw_f, [1] = cw_b - rw_b,
+        // which the consumer turns into the tile's own contribution with a prefix resp. suffix sum)
+        bool pending = false;
+        auto write_out = [&](int pbuf) __attribute__((always_inline)) {
             if (wave < 2) {
-                if (newer == 2) wait_vmcnt<10>();
-                else if (newer == 1) wait_vmcnt<5>();
-                else wait_vmcnt<0>();
+                const unsigned pq = sbase + DCB_PART_OFF + pbuf * DCB_PART_B + lane * 4;
+                float v;
+                if (st != tt && wave == 1) {
+                    v = raw_lds_read_at<float, 2048>(pq);
+                    raw_lds_wait();
+                    raw_lds_use(v);
+                } else {
+                    float a0, a1, a2, a3, r8 = 0.f;
+                    if (wave == 0) {
+                        a0 = raw_lds_read_at<float, 0>(pq); a1 = raw_lds_read_at<float, 256>(pq);
+                        a2 = raw_lds_read_at<float, 512>(pq); a3 = raw_lds_read_at<float, 768>(pq);
+                        if (st == tt) r8 = raw_lds_read_at<float, 2048>(pq);
+                    } else {
+                        a0 = raw_lds_read_at<float, 1024>(pq); a1 = raw_lds_read_at<float, 1024 + 256>(pq);
+                        a2 = raw_lds_read_at<float, 1024 + 512>(pq); a3 = raw_lds_read_at<float, 1024 + 768>(pq);
+                        r8 = raw_lds_read_at<float, 2048 + 256>(pq);
+                    }
+                    raw_lds_wait();
+                    raw_lds_use(a0); raw_lds_use(a1); raw_lds_use(a2); raw_lds_use(a3); raw_lds_use(r8);
+                    v = a0 + a1 + a2 + a3 - r8;
+                }
+                *tv = v;
+            }
+            tv += tv_head;
+        };
+        for (int it = 0; it < nit; ++it) {
+            TSR(0);
+            // the requests of step `it` went out before those of the step after it (the one after that is requested below);
+            // waves 0 and 1 make five requests per step, the others four
+            if (it + 1 < nit) {
+                if (wave < 2) wait_vmcnt<5>();
+                else wait_vmcnt<4>();
             } else {
-                if (newer == 2) wait_vmcnt<8>();
-                else if (newer == 1) wait_vmcnt<4>();
-                else wait_vmcnt<0>();
+                wait_vmcnt<0>();
             }
             TSR(1);
-            raw_lds_barrier();
+            raw_lds_barrier();     // step `it` has landed for everybody; every wave is done with the slot and the sums of step it - 1
+            if (it + 2 < nit) issue(slot2);
+            if (pending) {
+                write_out(par ^ 1);
+                pending = false;
+            }
             TSR(2);
             const unsigned sb = sbase + slot * DCB_SLOT_B;
             Frag af[NKS], bf[4][NKS];
@@ -1341,9 +1372,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
             asm volatile("" ::"v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3]));
 #endif
             TSR(4);
-            if (++kc < nkc) {
-                raw_lds_barrier();         // the slot is overwritten by the requests of the next iteration
-            } else {
+            if (++kc == nkc) {
                 kc = 0;
                 // ---- decay vectors of this head
                 f32x4 cft_ = raw_lds_read_at<f32x4, 0>(sb + ct_off), cbt_ = raw_lds_read_at<f32x4, 256>(sb + ct_off);
@@ -1461,35 +1490,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
                 }
                 raw_lds_wait();
                 TSR(7);
-                raw_lds_barrier();
-                TSR(8);
-                // off-diagonal: [0] = column sums, [1] = row sums.  diagonal: [0] = cw_f - rw_f, [1] = cw_b - rw_b
-                // (the consumer turns them into the tile's own contribution with a prefix resp. suffix sum)
-                if (wave < 2) {
-                    const unsigned pq = pb + lane * 4;
-                    float v;
-                    if (st != tt && wave == 1) {
-                        v = raw_lds_read_at<float, 2048>(pq);
-                        raw_lds_wait();
-                        raw_lds_use(v);
-                    } else {
-                        float a0, a1, a2, a3, r8 = 0.f;
-                        if (wave == 0) {
-                            a0 = raw_lds_read_at<float, 0>(pq); a1 = raw_lds_read_at<float, 256>(pq);
-                            a2 = raw_lds_read_at<float, 512>(pq); a3 = raw_lds_read_at<float, 768>(pq);
-                            if (st == tt) r8 = raw_lds_read_at<float, 2048>(pq);
-                        } else {
-                            a0 = raw_lds_read_at<float, 1024>(pq); a1 = raw_lds_read_at<float, 1024 + 256>(pq);
-                            a2 = raw_lds_read_at<float, 1024 + 512>(pq); a3 = raw_lds_read_at<float, 1024 + 768>(pq);
-                            r8 = raw_lds_read_at<float, 2048 + 256>(pq);
-                        }
-                        raw_lds_wait();
-                        raw_lds_use(a0); raw_lds_use(a1); raw_lds_use(a2); raw_lds_use(a3); raw_lds_use(r8);
-                        v = a0 + a1 + a2 + a3 - r8;
-                    }
-                    *tv = v;
-                }
-                tv += tv_head;
+                pending = true;            // written out after the next barrier (or after the loop)
                 par ^= 1;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -1497,6 +1498,10 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
             }
             slot = slot + 1 == DCB_RING ? 0 : slot + 1;
             slot2 = slot2 + 1 == DCB_RING ? 0 : slot2 + 1;
+        }
+        if (pending) {
+            raw_lds_barrier();
+            write_out(par ^ 1);
         }
 #ifdef BM2_DBG_TIME
         if (threadIdx.x == 0) {
