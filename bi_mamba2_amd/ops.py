@@ -459,7 +459,7 @@ def _set_states(c, fields, states, x, B):
 
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
                                    dt_limit=(0.0, _INF), return_intermediates=True, keep_for_bwd=False, causal=False,
-                                   initial_states=None, seq_idx=None):
+                                   initial_states=None, seq_idx=None, want_out_x=True):
     """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
     like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
     out, out_x and the final states are materialised as tensors (the rest lives in a workspace).
@@ -477,7 +477,8 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     ngroups, dstate = B.shape[2], B.shape[3]
     snap = c.snapshot() if keep_for_bwd else None
     out = c.new("out", x.shape, x.dtype)
-    out_x = c.new("out_x", x.shape, x.dtype) if z is not None else None
+    # the pre-gate output is what a backward pass needs; without one (want_out_x=False) the scan kernel skips that store
+    out_x = c.new("out_x", x.shape, x.dtype) if (z is not None and want_out_x) else None
     ff = c.new("final_f", (batch, nheads, headdim, dstate))
     fb = None if causal else c.new("final_b", (batch, nheads, headdim, dstate))
     dt_out = cs_f = cs_b = sf = sb = None
@@ -570,11 +571,11 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
         ctx.n_extra = len(extra)
         ctx.dt_dtype = dt.dtype
         init = tuple(initial_states) if any(t is not None for t in initial_states) else None
-        keep = KEEP_FORWARD_INTERMEDIATES and any(
-            t is not None and t.requires_grad for t in (x, dt, A, B, C, D, z, dt_bias) + tuple(initial_states))
+        need_bwd = any(ctx.needs_input_grad)       # False under torch.no_grad() and for inputs without requires_grad
+        keep = KEEP_FORWARD_INTERMEDIATES and need_bwd
         res = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit,
-            return_intermediates=False, keep_for_bwd=keep, initial_states=init, seq_idx=seq_idx)
+            return_intermediates=False, keep_for_bwd=keep, initial_states=init, seq_idx=seq_idx, want_out_x=need_bwd)
         out, out_x, ff, fb = res[0], res[1], res[7], res[8]
         saved = res[9] if keep else ()
         ctx.n_saved = len(saved)
