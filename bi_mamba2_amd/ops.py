@@ -38,6 +38,9 @@ def _f32c(t):
     return t.detach().to(torch.float32).contiguous()
 
 
+_WS_CACHE = {}
+
+
 class _Call:
     """Collects tensors into a ``bimamba2_params`` and keeps them alive until the launch has been enqueued."""
 
@@ -126,8 +129,23 @@ class _Call:
         self.p.has_dt_bias = 1
         return self.put("dt_bias", _f32c(dt_bias))
 
+    def _workspace_bytes(self, is_bwd):
+        return int(_lib.load().bimamba2_workspace_bytes(self.p, int(is_bwd)))
+
     def workspace(self, is_bwd):
-        n = _lib.load().bimamba2_workspace_bytes(self.p, int(is_bwd))
+        p = self.p
+        # the size depends on the problem and on which intermediates the caller brought; ask the library once per such key
+        # (which kernels run, and with them what is carved, also depends on strides and on 16-byte alignment)
+        al = lambda v: (v or 0) & 15
+        key = (is_bwd, p.batch, p.seqlen, p.nheads, p.headdim, p.ngroups, p.dstate, p.chunk_size, p.dtype, p.has_z, p.causal,
+               bool(p.dt_out), bool(p.cs_f), bool(p.states_f), bool(p.states_b), bool(p.CB), bool(p.CBT), bool(p.dCB), bool(p.dCBT),
+               bool(p.dstates_f), bool(p.dout_x), bool(p.red), bool(p.dBs), bool(p.da_intra),
+               p.x_sb, p.x_sl, p.x_sh, p.z_sb, p.z_sl, p.z_sh, p.dout_sb, p.dout_sl, p.dout_sh, p.B_sb, p.B_sl, p.B_sg,
+               p.C_sb, p.C_sl, p.C_sg, al(p.x), al(p.z), al(p.dout), al(p.Bm), al(p.Cm), al(p.out), al(p.out_x), al(p.dx),
+               al(p.states_f), al(p.states_b), al(p.dstates_f), al(p.dstates_b))
+        n = _WS_CACHE.get(key)
+        if n is None:
+            n = _WS_CACHE[key] = self._workspace_bytes(is_bwd)
         ws = torch.empty(max(int(n), 1), device=self.device, dtype=torch.uint8)
         self.keep.append(ws)
         self.p.workspace = ws.data_ptr()
@@ -438,6 +456,17 @@ def _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit):
     return c
 
 
+_BLOB_FIELDS = ("dt_out", "cs_f", "cs_b", "states_f", "states_b")
+
+
+def _point_into(c, blob, offs):
+    """Points the five forward intermediates at their places (float offsets) inside one float32 allocation."""
+    base = blob.data_ptr()
+    for field, o in zip(_BLOB_FIELDS, offs):
+        setattr(c.p, field, base + 4 * o)
+    c.keep.append(blob)
+
+
 def _set_seq_idx(c, seq_idx, x):
     """seq_idx: (batch, seqlen) integer tensor, constant over each packed sequence; None = one sequence per row."""
     c.p.seq_idx = None
@@ -459,7 +488,7 @@ def _set_states(c, fields, states, x, B):
 
 def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
                                    dt_limit=(0.0, _INF), return_intermediates=True, keep_for_bwd=False, causal=False,
-                                   initial_states=None, seq_idx=None, want_out_x=True):
+                                   initial_states=None, seq_idx=None, want_out_x=True, want_final=True):
     """Returns (out, out_x, dt_out, dA_cumsum_f, dA_cumsum_b, states_f, states_b, final_states_f, final_states_b)
     like the reference; states_* are the states entering each chunk.  With return_intermediates=False only
     out, out_x and the final states are materialised as tensors (the rest lives in a workspace).
@@ -475,20 +504,31 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
     _set_seq_idx(c, seq_idx, x)
     batch, seqlen, nheads, headdim = x.shape
     ngroups, dstate = B.shape[2], B.shape[3]
-    snap = c.snapshot() if keep_for_bwd else None
+    dt_out = cs_f = cs_b = sf = sb = None
+    saved = snap = None
+    if keep_for_bwd and not return_intermediates:
+        # what the backward pass reuses, in one allocation (five tensors cost five times the allocator's and Python's
+        # overhead); the snapshot below carries the pointers
+        n1 = (batch * nheads * c.nchunks * chunk_size + 63) // 64 * 64
+        n2 = (batch * c.nchunks * nheads * headdim * dstate + 63) // 64 * 64
+        blob = torch.empty(3 * n1 + 2 * n2, device=x.device, dtype=torch.float32)
+        offs = (0, n1, 2 * n1, 3 * n1, 3 * n1 + n2)
+        _point_into(c, blob, offs)
+        snap = c.snapshot() + (offs,)
+        saved = ("blob", blob, snap)
+    else:
+        snap = c.snapshot() if keep_for_bwd else None
+        if return_intermediates or keep_for_bwd:
+            dt_out = c.new("dt_out", _bhcq(c)); cs_f = c.new("cs_f", _bhcq(c)); cs_b = c.new("cs_b", _bhcq(c))
+            sshape = (batch, c.nchunks, nheads, headdim, dstate)
+            sf = c.new("states_f", sshape); sb = c.new("states_b", sshape)
+        if keep_for_bwd:
+            saved = (dt_out, cs_f, cs_b, sf, sb, snap)
     out = c.new("out", x.shape, x.dtype)
     # the pre-gate output is what a backward pass needs; without one (want_out_x=False) the scan kernel skips that store
     out_x = c.new("out_x", x.shape, x.dtype) if (z is not None and want_out_x) else None
-    ff = c.new("final_f", (batch, nheads, headdim, dstate))
-    fb = None if causal else c.new("final_b", (batch, nheads, headdim, dstate))
-    dt_out = cs_f = cs_b = sf = sb = None
-    saved = None
-    if return_intermediates or keep_for_bwd:
-        dt_out = c.new("dt_out", _bhcq(c)); cs_f = c.new("cs_f", _bhcq(c)); cs_b = c.new("cs_b", _bhcq(c))
-        sshape = (batch, c.nchunks, nheads, headdim, dstate)
-        sf = c.new("states_f", sshape); sb = c.new("states_b", sshape)
-    if keep_for_bwd:
-        saved = (dt_out, cs_f, cs_b, sf, sb, snap)
+    ff = c.new("final_f", (batch, nheads, headdim, dstate)) if want_final else None
+    fb = c.new("final_b", (batch, nheads, headdim, dstate)) if (want_final and not causal) else None
     c.workspace(False)
     c.run("bimamba2_fwd")
     res = (out, out_x, dt_out, cs_f, cs_b, sf, sb, ff, fb)
@@ -506,7 +546,11 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
     With initial_states = (initial_f, initial_b) given, the result has a ninth element (dinitial_f, dinitial_b)."""
     assert not recompute_output, "recompute_output is not supported"
     assert dout.shape == x.shape
-    snap = saved[5] if saved is not None and len(saved) > 5 else None
+    blob = None
+    if saved is not None and isinstance(saved[0], str):      # ("blob", allocation, snapshot): see the forward
+        blob, snap = saved[1], saved[2]
+    else:
+        snap = saved[5] if saved is not None and len(saved) > 5 else None
     c = None
     if snap is not None:
         # the forward's parameter block, if the tensors handed back by autograd are still the ones it describes
@@ -529,8 +573,11 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
         dinit = tuple(c.new(f, sshape) if t is not None else None
                       for f, t in zip(("dinitial_f", "dinitial_b"), initial_states))
     c.set_dout(dout)
-    if saved is not None:
-        for name, t in zip(("dt_out", "cs_f", "cs_b", "states_f", "states_b"), saved[:5]):
+    if blob is not None:
+        _point_into(c, blob, snap[2])
+        c.p.fwd_saved = 1
+    elif saved is not None:
+        for name, t in zip(_BLOB_FIELDS, saved[:5]):
             c.put(name, t, torch.float32)
         c.p.fwd_saved = 1
     if z is not None:
@@ -575,14 +622,14 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
         keep = KEEP_FORWARD_INTERMEDIATES and need_bwd
         res = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit,
-            return_intermediates=False, keep_for_bwd=keep, initial_states=init, seq_idx=seq_idx, want_out_x=need_bwd)
+            return_intermediates=False, keep_for_bwd=keep, initial_states=init, seq_idx=seq_idx, want_out_x=need_bwd,
+            want_final=return_final_states)
         out, out_x, ff, fb = res[0], res[1], res[7], res[8]
-        saved = res[9] if keep else ()
-        ctx.n_saved = len(saved)
-        ctx.snap = saved[5] if keep else None
+        # kept for the backward pass: ("blob", one allocation with dt_out, cs_f, cs_b and the states, snapshot)
+        blob, ctx.snap = (res[9][1], res[9][2]) if keep else (None, None)
         ctx.n_init = len(initial_states)
         ctx.save_for_backward(out_x if z is not None else None, x, dt, A, B, C, D, z, dt_bias,
-                              *(initial_states if ctx.n_init else (None, None)), *saved[:5])
+                              *(initial_states if ctx.n_init else (None, None)), blob)
         ctx.dt_softplus = dt_softplus
         ctx.chunk_size = chunk_size
         ctx.dt_limit = dt_limit
@@ -596,8 +643,8 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *dfinal):
-        out_x, x, dt, A, B, C, D, z, dt_bias, init_f, init_b = ctx.saved_tensors[:11]
-        saved = tuple(ctx.saved_tensors[11:]) + (ctx.snap,) if ctx.n_saved else None
+        out_x, x, dt, A, B, C, D, z, dt_bias, init_f, init_b, blob = ctx.saved_tensors
+        saved = ("blob", blob, ctx.snap) if blob is not None else None
         if dout is None:
             dout = torch.zeros_like(x)
         init = (init_f, init_b) if (init_f is not None or init_b is not None) else None
@@ -665,18 +712,16 @@ class CausalChunkScanCombinedFn(torch.autograd.Function):
         keep = any(t is not None and t.requires_grad for t in (x, dt, A, B, C, D, z, dt_bias))
         res = _mamba_chunk_scan_combined_fwd(
             x, dt, A, B, C, chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=dt_softplus, dt_limit=dt_limit,
-            return_intermediates=False, keep_for_bwd=keep, causal=True)
-        saved = res[9] if keep else ()
-        ctx.n_saved = len(saved)
-        ctx.snap = saved[5] if keep else None
-        ctx.save_for_backward(res[1] if z is not None else None, x, dt, A, B, C, D, z, dt_bias, *saved[:5])
+            return_intermediates=False, keep_for_bwd=keep, causal=True, want_final=False)
+        blob, ctx.snap = (res[9][1], res[9][2]) if keep else (None, None)
+        ctx.save_for_backward(res[1] if z is not None else None, x, dt, A, B, C, D, z, dt_bias, blob)
         ctx.dt_softplus, ctx.chunk_size, ctx.dt_limit = dt_softplus, chunk_size, dt_limit
         return res[0]
 
     @staticmethod
     def backward(ctx, dout):
-        out_x, x, dt, A, B, C, D, z, dt_bias = ctx.saved_tensors[:9]
-        saved = tuple(ctx.saved_tensors[9:]) + (ctx.snap,) if ctx.n_saved else None
+        out_x, x, dt, A, B, C, D, z, dt_bias, blob = ctx.saved_tensors
+        saved = ("blob", blob, ctx.snap) if blob is not None else None
         dx, ddt, dA, dB, dC, dD, dz, ddt_bias = _mamba_chunk_scan_combined_bwd(
             dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
             dt_limit=ctx.dt_limit, saved=saved, causal=True)
