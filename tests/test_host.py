@@ -120,3 +120,34 @@ def test_import_aliases():
     from ssd.modules import BiMamba2 as Alias
     assert bimamba_chunk_scan_combined is ops.bimamba_chunk_scan_combined
     assert MambaChunkScanCombinedFn is ops.MambaChunkScanCombinedFn and Alias is BiMamba2
+
+
+def test_norm_and_conv_argument_checks():
+    """The layer's two extra entry-point families check their arguments before anything is launched."""
+    lib = _lib.load()
+    assert lib.bimamba2_rmsnorm_gated_fwd(None) == -1 and lib.bimamba2_conv1d_silu_fwd(None) == -1
+    n = _lib.NormParams()
+    n.rows, n.cols, n.group_size, n.dtype = 4, 64, 48, _lib.F32
+    assert lib.bimamba2_rmsnorm_gated_fwd(ctypes.byref(n)) == -1                # groups do not divide the row
+    n.group_size = 64
+    assert lib.bimamba2_rmsnorm_gated_fwd(ctypes.byref(n)) == -1                # null pointers
+    assert lib.bimamba2_rmsnorm_gated_workspace_bytes(ctypes.byref(n)) == 0     # (0 for a problem that fails the checks)
+    c = _lib.ConvParams()
+    c.batch, c.seqlen, c.channels, c.width, c.dtype = 2, 16, 8, 4, _lib.BF16
+    c.x = c.weight = c.out = 256                                               # never dereferenced: the width check comes first
+    assert lib.bimamba2_conv1d_silu_fwd(ctypes.byref(c)) == -2                  # even filter width
+    c.width = 11
+    assert lib.bimamba2_conv1d_silu_fwd(ctypes.byref(c)) == -2                  # wider than the kernels are built for
+    c.width, c.x = 7, None
+    assert lib.bimamba2_conv1d_silu_fwd(ctypes.byref(c)) == -1                  # null input
+    c.x = 256
+    c.dout = c.dx = c.dweight = 256
+    assert lib.bimamba2_conv1d_silu_bwd(ctypes.byref(c)) == -3                  # backward without workspace
+    assert lib.bimamba2_conv1d_silu_workspace_bytes(ctypes.byref(c)) >= 2 * 16 // 56 * 8 * 8 * 4
+
+
+def test_causal_flag_and_second_direction_buffers():
+    """The single-direction comparator refuses a reverse final state."""
+    lib = _lib.load()
+    p = _params(causal=1, final_b=256, workspace=256, workspace_bytes=1 << 40)
+    assert lib.bimamba2_fwd(ctypes.byref(p)) == -1
