@@ -207,7 +207,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build measures the operator on ONE GPU; --gpus must be 1 "
-                         "(the path has no multi-GPU part; DESIGN.md says how it would shard).\n")
+                         "(the path has no multi-GPU part: it would shard over batch or head groups without communication).\n")
         sys.exit(2)
 
     import torch
