@@ -163,6 +163,25 @@ def whole_op_bytes(w, e, has_z):
     return fwd, bwd
 
 
+def make_inputs(batch, seqlen, nheads, headdim, ngroups, dstate, dtype, with_z, seed=0):
+    """Synthetic inputs of the benchmark (on the CPU, seeded): x, B, C, z ~ N(0, 1) rounded to `dtype`; dt ~ N(0, 0.5);
+    A = -exp(U(log 1, log 16)); dt_bias = inverse softplus of log-uniform [1e-3, 1e-1] (the layer's own initialisation,
+    src/ssd/modules.py:94 of the reference); D ~ N(0, 1) per head; dt, A, D, dt_bias float32."""
+    import math
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(batch, seqlen, nheads, headdim, generator=g).to(dtype)
+    dt = 0.5 * torch.randn(batch, seqlen, nheads, generator=g)
+    A = -torch.exp(torch.rand(nheads, generator=g) * math.log(16.0))
+    B = torch.randn(batch, seqlen, ngroups, dstate, generator=g).to(dtype)
+    C = torch.randn(batch, seqlen, ngroups, dstate, generator=g).to(dtype)
+    dt0 = torch.exp(torch.rand(nheads, generator=g) * (math.log(1e-1) - math.log(1e-3)) + math.log(1e-3))
+    dt_bias = dt0 + torch.log(-torch.expm1(-dt0))
+    D = torch.randn(nheads, generator=g)
+    z = torch.randn(batch, seqlen, nheads, headdim, generator=g).to(dtype) if with_z else None
+    return dict(x=x, dt=dt, A=A, B=B, C=C, D=D, z=z, dt_bias=dt_bias)
+
+
 def cpu_baseline(w, budget_s=15.0):
     """The oracle's naive flip-and-sum path (chunked causal SSD twice) in float32 PyTorch on the host cores,
     forward + backward, on one batch row of the same workload, repeated for about 15 s."""
@@ -172,7 +191,7 @@ def cpu_baseline(w, budget_s=15.0):
     cores = min(16, os.cpu_count() or 1)
     torch.set_num_threads(cores)
     heads = w["nheads"]
-    inp = O.make_inputs(1, w["seqlen"], heads, w["headdim"], 1, w["dstate"], seed=0, dtype=torch.float32, with_z=True)
+    inp = make_inputs(1, w["seqlen"], heads, w["headdim"], 1, w["dstate"], torch.float32, True)
 
     def step():
         leaves = {k: v.clone().requires_grad_(True) for k, v in inp.items()}
@@ -212,7 +231,6 @@ def main():
 
     import torch
     from bi_mamba2_amd import _lib, ops
-    from oracle import bimamba2_oracle as O
 
     _lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -220,8 +238,7 @@ def main():
     w = WORKLOAD
     dtype, e = torch.bfloat16, 2
     has_z = not args.no_z
-    inp = O.make_inputs(w["batch"], w["seqlen"], w["nheads"], w["headdim"], w["ngroups"], w["dstate"], seed=0,
-                        dtype=dtype, with_z=has_z)
+    inp = make_inputs(w["batch"], w["seqlen"], w["nheads"], w["headdim"], w["ngroups"], w["dstate"], dtype, has_z)
     leaves = {k: (v.to(dev).requires_grad_(True) if v is not None else None) for k, v in inp.items()}
     dout = torch.randn(inp["x"].shape, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
 
