@@ -22,7 +22,11 @@ reference's stage wrappers return them) so that every device kernel can be check
 Pinning: the sequential form is checked against the C restatement in oracle/bimamba2_seq.c (different language,
 scalar loops), the three forms against each other, against special cases with textbook answers (A = 0 turns
 the operator into a plain masked matmul; a single constant channel turns it into a geometric series) and
-against torch.autograd.gradcheck; see tests/test_oracle.py.
+against torch.autograd.gradcheck; see tests/test_oracle.py.  The extensions are pinned there as well:
+``ssd_causal`` (the single-direction operator of the comparator) against the token-by-token recurrence written out in
+the test and by "causal + flipped causal = bidirectional"; the initial states of ``bimamba2_sequential`` by the
+cut-sequence identity (two pieces chained through their final states equal the uncut run); its ``seq_idx`` by "packed
+sequences equal the same sequences run one by one".
 """
 import math
 
