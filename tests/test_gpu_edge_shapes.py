@@ -37,3 +37,46 @@ def test_tiny_and_ragged_shapes(case):
     for k in ("x", "B", "C", "z", "dt", "A", "D", "dt_bias"):
         if ref["d" + k] is not None:
             assert_close(leaves[k].grad, ref["d" + k], dtype, "d" + k)
+
+
+BIG = [
+    # batch, seqlen, H, P, G, N, z: x, z, dout and their gradients pass 2^31 elements inside the last batch row ...
+    (9, 65536, 64, 64, 1, 64, True),
+    # ... and here the per-chunk states (batch * nchunks * H * P * N) do too, on the kernels for other shapes
+    (9, 65536, 64, 128, 2, 128, False),
+]
+
+
+@pytest.mark.parametrize("case", BIG)
+def test_offsets_beyond_32_bits(case):
+    """The last batch row of a problem whose tensors hold more than 2^31 elements must come out exactly as the same row
+    computed alone (no workgroup works on more than one batch row, so every sum has the same order): an element offset
+    that wraps at 32 bits anywhere in the forward or backward kernels breaks this."""
+    from bi_mamba2_amd import ops
+    b, L, H, P, G, N, with_z = case
+    dtype, Q = torch.bfloat16, 256
+    g = torch.Generator(device="cuda").manual_seed(11)
+    rn = lambda *s: torch.randn(*s, device="cuda", dtype=dtype, generator=g)
+    x, Bm, Cm, dout = rn(b, L, H, P), rn(b, L, G, N), rn(b, L, G, N), rn(b, L, H, P)
+    z = rn(b, L, H, P) if with_z else None
+    dt = rn(b, L, H)
+    A = -torch.rand(H, device="cuda", generator=g) - 0.5
+    D = torch.randn(H, device="cuda", generator=g)
+    dt_bias = torch.randn(H, device="cuda", generator=g) * 0.1 - 3.0
+    assert x.numel() > 2 ** 31
+
+    def run(sl):
+        leaves = [t[sl].detach().requires_grad_(True) if t is not None else None for t in (x, dt, Bm, Cm, z)]
+        out = ops.bimamba_chunk_scan_combined(leaves[0], leaves[1], A, leaves[2], leaves[3], Q, D=D, z=leaves[4],
+                                              dt_bias=dt_bias, dt_softplus=True)
+        grads = torch.autograd.grad(out, [t for t in leaves if t is not None], dout[sl])
+        return [out.detach()] + list(grads)
+
+    last = slice(b - 1, b)
+    alone = run(last)
+    full = run(slice(0, b))
+    names = ["out", "dx", "ddt", "dB", "dC"] + (["dz"] if with_z else [])
+    for name, f, a in zip(names, full, alone):
+        assert torch.isfinite(a.float()).all(), name
+        assert a.float().abs().max() > 0, name
+        assert torch.equal(f[last], a), f"{name}: the last batch row differs from the same row computed alone"
