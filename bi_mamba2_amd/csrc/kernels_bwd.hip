@@ -857,6 +857,7 @@ int launch_bwd_dbdc(const bimamba2_params *p, bool is_db) {
 // put into LDS beforehand.
 // =========================================================================================================
 constexpr int DCB_HEADS = 32;
+constexpr int DCB_SLICE_HEADS = 32;     // heads per slice
 constexpr int DCB_SLICES_MAX = 4;
 constexpr int DCB_VEC = 2 * 64;      // floats per tile and head in da_intra
 
@@ -1136,7 +1137,7 @@ __global__ __launch_bounds__(NTHREADS) void sum_slices_kernel(float *dst, size_t
 // head slices of the dCB kernel: one per 32 heads of a group (more slices only cost traffic: measured)
 int dcb_slices(const bimamba2_params *p) {
     const int hpg = p->nheads / p->ngroups;
-    return std::max(1, std::min(DCB_SLICES_MAX, hpg / 32));
+    return std::max(1, std::min(DCB_SLICES_MAX, hpg / DCB_SLICE_HEADS));
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -1145,7 +1146,7 @@ int dcb_slices(const bimamba2_params *p) {
 // The kernel is bound by its instruction count, not by memory, so everything per head is pared down:
 //  * the dout tile, the x tile and the decay vectors of each (head, 64-wide headdim chunk) step travel from global memory
 //    straight into a ring of LDS slots (global_load_lds, 16 bytes per lane, no registers, no address arithmetic beyond
-//    one 64-bit add per request), two steps ahead of the one being multiplied; 16-byte units are XOR-swizzled by the row
+//    one 64-bit add per request), one step ahead of the one being multiplied; 16-byte units are XOR-swizzled by the row
 //    so that the fragment reads spread over the banks;
 //  * a wave owns 16 rows t; against a block of 16 columns s that lies wholly below (s < t) or above (s > t) the diagonal
 //    the decay factor separates, exp(cs[t] - cs[s]) = exp(cs[t] - m) * exp(m - cs[s]) with m taken at the edge of the
@@ -1161,7 +1162,9 @@ __device__ __forceinline__ float lanegroup_sum_mfma(float v) {
     return d[0];
 }
 
-constexpr int DCB_RING = 3;
+// Slots of the ring.  Two (the step being multiplied and the one after it, requested right after the barrier that frees
+// its slot) measured 60 us against 62 us for three slots requested two steps ahead.
+constexpr int DCB_RING = 2;
 constexpr int DCB_TILE_B = 64 * 64 * 2;                    // one 64 x 64 tile of 16-bit elements
 constexpr int DCB_CS_OFF = 2 * DCB_TILE_B;                 // cs_f[t], cs_b[t], cs_f[s], cs_b[s], dt[s]: 5 x 64 floats
 constexpr int DCB_SLOT_B = DCB_CS_OFF + 5 * 64 * 4;
@@ -1263,7 +1266,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
 
         f32x4 acc[4] = {};
         issue(0);
-        if (nit > 1) issue(1);
+        if (DCB_RING > 2 && nit > 1) issue(1);
         if (p.CB) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -1296,7 +1299,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
         long long ph[12] = {}, tlast = wall_clock64();
         const long long tstart = tlast;
 #endif
-        int slot = 0, slot2 = 2 % DCB_RING, kc = 0, par = 0;
+        int slot = 0, slot2 = (DCB_RING - 1) % DCB_RING, kc = 0, par = 0;
         float *tv = tv0 + (wave & 1) * 64 + lane;
         // the sums of a head are written out one iteration later, after the barrier that the next step needs anyway
         // (waves 0 and 1; off-diagonal: [0] = column sums, [1] = row sums.  diagonal: [0] = cw_f - rw_f, [1] = cw_b - rw_b,
@@ -1331,9 +1334,9 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
         };
         for (int it = 0; it < nit; ++it) {
             TSR(0);
-            // the requests of step `it` went out before those of the step after it (the one after that is requested below);
-            // waves 0 and 1 make five requests per step, the others four
-            if (it + 1 < nit) {
+            // with two slots nothing but step `it` is outstanding here; with more, the requests of step `it` went out before
+            // those of the step after it (waves 0 and 1 make five requests per step, the others four)
+            if (DCB_RING > 2 && it + 1 < nit) {
                 if (wave < 2) wait_vmcnt<5>();
                 else wait_vmcnt<4>();
             } else {
@@ -1341,7 +1344,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
             }
             TSR(1);
             raw_lds_barrier();     // step `it` has landed for everybody; every wave is done with the slot and the sums of step it - 1
-            if (it + 2 < nit) issue(slot2);
+            if (it + DCB_RING - 1 < nit) issue(slot2);
             if (pending) {
                 write_out(par ^ 1);
                 pending = false;
