@@ -55,9 +55,17 @@ __global__ __launch_bounds__(NTHREADS) void reduce_jobs_kernel(ReduceJobs jobs) 
     const ReduceJob jb = jobs.job[k];
     float s = 0.f;
     const int total = jb.ni * jb.nk;
-    for (int t = threadIdx.x; t < total; t += NTHREADS) {
-        const int i = t / jb.nk, kk = t - i * jb.nk;
-        s += jb.in[((int64_t)i * jb.nj + j) * jb.nk + kk];
+    // eight loads go out before the first is added: a load that is waited for costs microseconds here
+    for (int t0 = threadIdx.x; t0 < total; t0 += 8 * NTHREADS) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int t = min(t0 + u * NTHREADS, total - 1), i = t / jb.nk, kk = t - i * jb.nk;
+            v[u] = jb.in[((int64_t)i * jb.nj + j) * jb.nk + kk];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (t0 + u * NTHREADS < total) s += v[u];
     }
     s = wave_sum(s);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
