@@ -282,8 +282,13 @@ int bimamba2_bwd(const bimamba2_params *p) {
     if (need_cb) TRY(bimamba2_bmm_chunk_fwd(&q));  // CB for the dCB kernel, CB^T for the dx kernel, unless they rebuild it
     else q.CB = nullptr;
     if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
+    // the dCB kernel is bound by instruction issue and moves little data: right behind dz it runs while the memory system
+    // still writes back dz's output, which the memory-bound kernels after it would otherwise wait behind
+    TRY(bimamba2_chunk_scan_bwd_dcb(&q));
     TRY(bimamba2_chunk_scan_bwd_dstates(&q));
+    TRY(bimamba2_chunk_scan_bwd_dc(&q));           // (between the two memory-bound state kernels: measured best)
     TRY(bimamba2_state_passing_bwd(&q));
+    TRY(bimamba2_chunk_state_bwd_db(&q));
     ReduceJobs jobs;
     {
         // as bimamba2_chunk_scan_bwd_dx, with the reduction of the dD partial sums left for the end
@@ -300,9 +305,6 @@ int bimamba2_bwd(const bimamba2_params *p) {
             else jobs.job[jobs.n++] = ReduceJob{q.red, q.dD, q.batch * nc, q.nheads, q.headdim};
         }
     }
-    TRY(bimamba2_chunk_state_bwd_db(&q));
-    TRY(bimamba2_chunk_scan_bwd_dc(&q));
-    TRY(bimamba2_chunk_scan_bwd_dcb(&q));
     {
         // as bimamba2_bmm_chunk_bwd and bimamba2_chunk_cumsum_bwd (its partial sums behind those of dD): one launch for
         // both where the kernel for it exists
