@@ -36,15 +36,16 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def stage_table(w, e, fused=(False, False, False)):
+def stage_table(w, e, fused=(False, False, False), copies=False):
     """Algorithmic flops and bytes per launch of every stage kernel (e = bytes per element of x/B/C/z).
     fused[0] / [1] / [2]: the forward scan / the dx kernel / the dCB kernel rebuilds its CB tiles from C and B instead of
-    reading them."""
+    reading them.  copies: the states entering the chunks (and their gradients) are kept in e-byte copies."""
     B, L, H, P, G, N, Q = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate", "chunk_size"))
     nc = (L + Q - 1) // Q
     u, ug = B * nc * H, B * nc * G                 # (b, c, h) and (b, c, g) units
     T4, T2, T1 = B * L * H * P, B * L * G * N, B * H * nc * Q
     st = 4 * B * nc * H * P * N                     # one float32 state tensor
+    se = (e if copies else 4) * B * nc * H * P * N  # one tensor of entering states as the kernels read it
     cb = 4 * ug * Q * Q
     scan_cb = [(u * 2 * Q * Q * N, e * T2) if f else (0, cb) for f in fused]   # (extra flops, bytes) for the CB tiles
     return {
@@ -52,16 +53,16 @@ def stage_table(w, e, fused=(False, False, False)):
         "bimamba2_chunk_cumsum_fwd": (0, 4 * B * L * H + 3 * 4 * T1),
         "bimamba2_bmm_chunk_fwd": (ug * 2 * Q * Q * N, 2 * e * T2 + cb),
         "bimamba2_chunk_state_fwd": (u * 4 * P * N * Q, e * T4 + e * T2 + 3 * 4 * T1 + 2 * st),
-        "bimamba2_state_passing_fwd": (0, 4 * st),
+        "bimamba2_state_passing_fwd": (0, 2 * st + 2 * se),
         "bimamba2_chunk_scan_fwd": (u * (2 * Q * Q * P + 4 * Q * P * N) + scan_cb[0][0],
-                                    4 * e * T4 + e * T2 + 3 * 4 * T1 + 2 * st + scan_cb[0][1]),
+                                    4 * e * T4 + e * T2 + 3 * 4 * T1 + 2 * se + scan_cb[0][1]),
         "bimamba2_chunk_scan_bwd_dz": (0, 5 * e * T4),
         "bimamba2_chunk_scan_bwd_dstates": (u * 4 * P * N * Q, e * T4 + e * T2 + 2 * 4 * T1 + 2 * st),
-        "bimamba2_state_passing_bwd": (0, 6 * st),
+        "bimamba2_state_passing_bwd": (0, 2 * st + 4 * se),
         "bimamba2_chunk_scan_bwd_dx": (u * (2 * Q * Q * P + 4 * Q * P * N) + scan_cb[1][0],
-                                       3 * e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + scan_cb[1][1]),
-        "bimamba2_chunk_state_bwd_db": (u * 4 * Q * P * N, e * T4 + e * T2 + 5 * 4 * T1 + 2 * st + 4 * T2),
-        "bimamba2_chunk_scan_bwd_dc": (u * 4 * Q * P * N, e * T4 + e * T2 + 4 * 4 * T1 + 2 * st + 4 * T2),
+                                       3 * e * T4 + e * T2 + 4 * 4 * T1 + 2 * se + scan_cb[1][1]),
+        "bimamba2_chunk_state_bwd_db": (u * 4 * Q * P * N, e * T4 + e * T2 + 5 * 4 * T1 + 2 * se + 4 * T2),
+        "bimamba2_chunk_scan_bwd_dc": (u * 4 * Q * P * N, e * T4 + e * T2 + 4 * 4 * T1 + 2 * se + 4 * T2),
         "bimamba2_chunk_scan_bwd_dcb": (u * 2 * Q * Q * P + (ug * 2 * Q * Q * N if fused[2] else 0),
                                         2 * e * T4 + 3 * 4 * T1 + (2 * e * T2 if fused[2] else cb) + 2 * cb
                                         + 4 * B * H * nc * ((Q + 63) // 64) ** 2 * 128),
@@ -318,7 +319,13 @@ def main():
     c.run("bimamba2_bwd")
     torch.cuda.synchronize()
     reads_cb = [_lib.load().bimamba2_chunk_scan_reads_cb(ctypes.byref(c.p), d) for d in (0, 1, 2)]
-    table = stage_table(w, e, fused=tuple(r == 0 for r in reads_cb))
+    # the stages are timed the way the composites run them: with the 16-bit copies of the entering states where the
+    # kernels of this problem keep them
+    copies = bool(_lib.load().bimamba2_state_copies(ctypes.byref(c.p)))
+    if copies:
+        for f in ("states16_f", "states16_b", "dstates16_f", "dstates16_b"):
+            c.new(f, sts, dtype)
+    table = stage_table(w, e, fused=tuple(r == 0 for r in reads_cb), copies=copies)
     if not any(reads_cb):
         del table["bimamba2_bmm_chunk_fwd"]     # not launched by the composites for this problem
     if _lib.load().bimamba2_chunk_scan_reads_cb(ctypes.byref(c.p), 3) == 0:

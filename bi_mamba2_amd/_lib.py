@@ -32,7 +32,7 @@ class Params(ctypes.Structure):
                               "ddt_direct", "u_f", "u_b", "v_f", "v_b", "da_intra",
                               "ddA_chunk_f", "ddA_chunk_b", "dBs", "dCs", "red",
                               "initial_f", "initial_b", "dfinal_f", "dfinal_b", "dinitial_f", "dinitial_b", "seq_idx",
-                              "workspace")]
+                              "states16_f", "states16_b", "dstates16_f", "dstates16_b", "workspace")]
         + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
     )
 
@@ -48,7 +48,7 @@ ENTRY_POINTS = (
 NORM_ENTRY_POINTS = ("bimamba2_rmsnorm_gated_fwd", "bimamba2_rmsnorm_gated_bwd")
 CONV_ENTRY_POINTS = ("bimamba2_conv1d_silu_fwd", "bimamba2_conv1d_silu_bwd")
 ALL_SYMBOLS = ENTRY_POINTS + ("bimamba2_strerror", "bimamba2_version", "bimamba2_params_size",
-                              "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb", "bimamba2_norm_params_size",
+                              "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb", "bimamba2_state_copies", "bimamba2_norm_params_size",
                               "bimamba2_rmsnorm_gated_workspace_bytes", "bimamba2_conv_params_size",
                               "bimamba2_conv1d_silu_workspace_bytes") + NORM_ENTRY_POINTS + CONV_ENTRY_POINTS
 
@@ -95,6 +95,8 @@ def load():
     lib.bimamba2_version.restype = ctypes.c_int
     lib.bimamba2_chunk_scan_reads_cb.argtypes = [ctypes.POINTER(Params), ctypes.c_int]
     lib.bimamba2_chunk_scan_reads_cb.restype = ctypes.c_int
+    lib.bimamba2_state_copies.argtypes = [ctypes.POINTER(Params)]
+    lib.bimamba2_state_copies.restype = ctypes.c_int
     lib.bimamba2_params_size.restype = ctypes.c_size_t
     if lib.bimamba2_params_size() != ctypes.sizeof(Params):
         raise RuntimeError("bimamba2_params layout mismatch between the library and its Python mirror")

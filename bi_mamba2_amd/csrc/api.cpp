@@ -1,3 +1,4 @@
+#include <cstdlib>
 // C ABI of libbimamba2_hip.so: argument checks, workspace carving and the forward / backward pipelines.
 #include <stdio.h>
 #include <string.h>
@@ -66,8 +67,23 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     need_f(q->cs_b, bhcq);
     // CB: read by the forward scan and by the dCB kernel unless they rebuild it; CB^T: by the dx kernel, likewise
     if (is_bwd ? !(scan_recomputes_cb(q, true) && dcb_recomputes_cb(q)) : !scan_recomputes_cb(q, false)) need_f(q->CB, cbn);
-    need_f(q->states_f, stn);
-    need_f(q->states_b, stn);
+    // 16-bit copies of the entering states (see states16_f in the header): used where the kernels know them and the
+    // caller does not ask for the float32 entering states; a backward pass that got the copies from the forward pass
+    // needs no float32 states at all
+    const bool copies = bimamba2_state_copies(q) != 0;
+    const bool saved_copies = is_bwd && q->fwd_saved && q->states16_f;
+    if (copies && !q->states_f && !q->states16_f) {
+        q->states16_f = cv.take<char>(stn * 2);
+        q->states16_b = cv.take<char>(stn * 2);
+    }
+    if (!saved_copies) {
+        need_f(q->states_f, stn);
+        need_f(q->states_b, stn);
+    }
+    if (is_bwd && copies && !q->dstates_f && !q->dstates16_f) {
+        q->dstates16_f = cv.take<char>(stn * 2);
+        q->dstates16_b = cv.take<char>(stn * 2);
+    }
     if (is_bwd) {
         const size_t nqt = (Q + 63) / 64;
         need_f(q->dCB, cbn * dcb_slices(q));
@@ -120,6 +136,20 @@ size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd) {
     return carve(&q, is_bwd, nullptr);
 }
 
+int bimamba2_state_copies(const bimamba2_params *p) {
+    if (check_problem(p)) return 0;
+    if (p->dtype != BIMAMBA2_BF16 && p->dtype != BIMAMBA2_F16) return 0;
+    if (p->dstate != 64 || p->headdim % 64 || p->chunk_size % 64) return 0;
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    // the vector kernels of the two state-passing stages, the scan kernels that rebuild CB, the dB / dC kernels with the
+    // ring of state tiles: every one of them must be the one that runs
+    if (!(al(p->states_f) && al(p->states_b) && al(p->dstates_f) && al(p->dstates_b) && al(p->final_f) && al(p->final_b) &&
+          al(p->initial_f) && al(p->initial_b) && al(p->dfinal_f) && al(p->dfinal_b) && al(p->dinitial_f) && al(p->dinitial_b)))
+        return 0;
+    if (!al(p->states16_f) || !al(p->states16_b) || !al(p->dstates16_f) || !al(p->dstates16_b)) return 0;
+    return scan_recomputes_cb(p, false) && scan_recomputes_cb(p, true) && dcb_recomputes_cb(p) ? 1 : 0;
+}
+
 int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which) {
     if (check_problem(p)) return 1;
     if (which == 2) return dcb_recomputes_cb(p) ? 0 : 1;
@@ -157,7 +187,8 @@ int bimamba2_chunk_scan_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->x); REQUIRE(p->Cm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
     if (!p->CB && !(p->Bm && scan_recomputes_cb(p, false))) return BIMAMBA2_EINVAL;   // without CB the kernel rebuilds it from Cm, Bm
-    REQUIRE(p->states_f); REQUIRE(p->states_b); REQUIRE(p->out);
+    if (!p->states16_f) { REQUIRE(p->states_f); REQUIRE(p->states_b); }
+    REQUIRE(p->out);
     if (p->has_D) REQUIRE(p->D);
     if (p->has_z) REQUIRE(p->z);
     return launch_chunk_scan(p, false);
@@ -179,7 +210,8 @@ int bimamba2_chunk_scan_bwd_dstates(const bimamba2_params *p) {
 
 int bimamba2_state_passing_bwd(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
+    REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (!p->states16_f) { REQUIRE(p->states_f); REQUIRE(p->states_b); }
     REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->ddA_chunk_f); REQUIRE(p->ddA_chunk_b);
     return launch_state_passing_bwd(p);
 }
@@ -188,7 +220,8 @@ int bimamba2_chunk_scan_bwd_dx(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
     if (!p->CBT && !(p->Cm && scan_recomputes_cb(p, true))) return BIMAMBA2_EINVAL;   // without CBT the kernel rebuilds it from Cm, Bm
-    REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->dx); REQUIRE(p->ddt_direct);
+    if (!p->dstates16_f) { REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); }
+    REQUIRE(p->dx); REQUIRE(p->ddt_direct);
     if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
     if (p->has_D) { REQUIRE(p->D); REQUIRE(p->dD); REQUIRE(p->red); }
     const int nc = nchunks(p);
@@ -205,13 +238,15 @@ int bimamba2_chunk_scan_bwd_dx(const bimamba2_params *p) {
 int bimamba2_chunk_state_bwd_db(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
-    REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->dBs); REQUIRE(p->v_f); REQUIRE(p->v_b);
+    if (!p->dstates16_f) { REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); }
+    REQUIRE(p->dBs); REQUIRE(p->v_f); REQUIRE(p->v_b);
     return launch_bwd_dbdc(p, true);
 }
 
 int bimamba2_chunk_scan_bwd_dc(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
+    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (!p->states16_f) { REQUIRE(p->states_f); REQUIRE(p->states_b); }
     REQUIRE(p->dCs); REQUIRE(p->u_f); REQUIRE(p->u_b);
     if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
     return launch_bwd_dbdc(p, false);
@@ -272,7 +307,8 @@ int bimamba2_bwd(const bimamba2_params *p) {
     const size_t need = carve(&q, 1, p->workspace);
     if (need > 256 && (!p->workspace || p->workspace_bytes < need)) return BIMAMBA2_EWORKSPACE;
     if (p->fwd_saved) {
-        REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
+        REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+        if (!p->states16_f) { REQUIRE(p->states_f); REQUIRE(p->states_b); }
     } else {
         // recompute the forward intermediates (the reference does the same, src/ssd/bi/ssd_combined.py:373-380)
         TRY(forward_cumsum_and_states(&q));

@@ -215,8 +215,12 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_kernel(const bimam
 // The same with 16-byte accesses, one direction per workgroup (blockIdx.z = 2 b + dir) and the loads of SP_CH chunks in
 // flight before the first of them is used: the recurrence is a chain over the chunks, and a global access that has to be
 // waited for at every link costs microseconds.  Needs P*N % 4 == 0 and 16-byte aligned tensors.
+// PREV16: the entering states are read from their 16-bit copies (states16_*); DS16: the gradients with respect to the
+// entering states go to dstates16_* and the per-chunk gradients in dstates_* stay as they are.
 constexpr int SP_CH = 8;
+template <typename T16, bool PREV16, bool DS16>
 __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const bimamba2_params p, int nc, int nsplit, int ndir) {
+    struct alignas(8) V4 { T16 v[4]; };
     __shared__ float red[SP_CH][4];
     const int PN = p.headdim * p.dstate;
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z / ndir, dir = blockIdx.z % ndir;   // ndir = 1: forward direction only
@@ -229,7 +233,9 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const b
     const bool live = e_own < PN;
     const int e = live ? e_own : PN - SP_EPT;              // loads are unconditional (so that they all go out together)
     const float *prev = (dir == 0 ? p.states_f : p.states_b) + base + e;
+    const T16 *prev16 = reinterpret_cast<const T16 *>(dir == 0 ? p.states16_f : p.states16_b) + base + e;
     float *ds = (dir == 0 ? p.dstates_f : p.dstates_b) + base + e;
+    T16 *ds16 = reinterpret_cast<T16 *>(dir == 0 ? p.dstates16_f : p.dstates16_b) + base + e;
     float *dda = (dir == 0 ? p.ddA_chunk_f : p.ddA_chunk_b) + ((int64_t)b * p.nheads + h) * nc * nsplit + split;
     const float *dfin = dir == 0 ? p.dfinal_f : p.dfinal_b;
     float *dini = dir == 0 ? p.dinitial_f : p.dinitial_b;
@@ -246,7 +252,13 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const b
             const int c = dir == 0 ? nc - 1 - sj : sj;
             dec[j] = cs[(int64_t)c * Q];
             dp[j] = *reinterpret_cast<const f32x4 *>(ds + c * cstride);
-            pv[j] = *reinterpret_cast<const f32x4 *>(prev + c * cstride);
+            if constexpr (PREV16) {
+                const V4 t = *reinterpret_cast<const V4 *>(prev16 + c * cstride);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) pv[j][k] = to_f(t.v[k]);
+            } else {
+                pv[j] = *reinterpret_cast<const f32x4 *>(prev + c * cstride);
+            }
         }
 #pragma unroll
         for (int j = 0; j < SP_CH; ++j) {
@@ -256,7 +268,14 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const b
                 float dot = 0.f;
                 if (live) {
                     dot = g[0] * pv[j][0] + g[1] * pv[j][1] + g[2] * pv[j][2] + g[3] * pv[j][3];
-                    *reinterpret_cast<f32x4 *>(ds + c * cstride) = g;
+                    if constexpr (DS16) {
+                        V4 t;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) t.v[k] = from_f<T16>(g[k]);
+                        *reinterpret_cast<V4 *>(ds16 + c * cstride) = t;
+                    } else {
+                        *reinterpret_cast<f32x4 *>(ds + c * cstride) = g;
+                    }
                     g = dp[j] + d * g;
                 }
                 dot = wave_sum(dot) * d;
@@ -281,9 +300,22 @@ int launch_state_passing_bwd(const bimamba2_params *p) {
     if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->dstates_f) && al(p->dstates_b) && al(p->dfinal_f) && al(p->dfinal_b) &&
         al(p->dinitial_f) && al(p->dinitial_b)) {
         dim3 grid(nsplit, p->nheads, p->batch * ndir);
-        hipLaunchKernelGGL(state_passing_bwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit, ndir);
+        const bool prev16 = p->states16_f != nullptr, ds16 = p->dstates16_f != nullptr;
+        if (prev16 && (!(p->causal || p->states16_b) || !al(p->states16_f) || !al(p->states16_b))) return BIMAMBA2_EINVAL;
+        if (ds16 && (!(p->causal || p->dstates16_b) || !al(p->dstates16_f) || !al(p->dstates16_b))) return BIMAMBA2_EINVAL;
+        if ((prev16 || ds16) && p->dtype != BIMAMBA2_BF16 && p->dtype != BIMAMBA2_F16) return BIMAMBA2_EUNSUPPORTED;
+#define BM2_SPB(TT, A, B) hipLaunchKernelGGL((state_passing_bwd_vec_kernel<TT, A, B>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit, ndir)
+        if (p->dtype == BIMAMBA2_F16) {
+            if (prev16 && ds16) BM2_SPB(f16_t, true, true); else if (prev16) BM2_SPB(f16_t, true, false);
+            else if (ds16) BM2_SPB(f16_t, false, true); else BM2_SPB(f16_t, false, false);
+        } else {
+            if (prev16 && ds16) BM2_SPB(bf16_t, true, true); else if (prev16) BM2_SPB(bf16_t, true, false);
+            else if (ds16) BM2_SPB(bf16_t, false, true); else BM2_SPB(bf16_t, false, false);
+        }
+#undef BM2_SPB
         return check_launch();
     }
+    if (p->states16_f || p->dstates16_f) return BIMAMBA2_EUNSUPPORTED;
     if (p->causal) return BIMAMBA2_EUNSUPPORTED;
     dim3 grid(nsplit, p->nheads, p->batch);
     hipLaunchKernelGGL(state_passing_bwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit);
@@ -530,7 +562,10 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_kernel(const bimamba2_p
 // Order of a wave's vector memory operations per step: NDIR * 2 ring requests, then QT * 2 fragment loads; "at most one
 // step's worth outstanding" therefore means that the step in hand has landed.
 // ---------------------------------------------------------------------------------------------------------
-template <typename T, int QT, bool IS_DB, bool UNI>
+// S16: the state tiles come from their 16-bit copies (states16_* / dstates16_*).  They lie in the ring as they lie in
+// memory ([p][n], 16-byte chunks swizzled as tile64_request does), and the operand fragments are LDS transpose reads
+// straight from the ring slot: no operand image, one barrier per step, a third of the LDS.
+template <typename T, int QT, bool IS_DB, bool UNI, bool S16>
 __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamba2_params p, int nc) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
@@ -539,12 +574,13 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
     constexpr int ROWS = DBDC_WAVES * 16 * QT;
     constexpr int NBLK = (KC / VK) * 16;                       // 8 x 4 blocks of a 64 x 64 tile
     constexpr int RING = 3, NDIR = UNI ? 1 : 2;
-    constexpr int TILE_B = 64 * 64 * 4;                        // bytes of a float32 state tile
+    constexpr int TILE_B = 64 * 64 * (S16 ? 2 : 4);            // bytes of a state tile
     constexpr int IMG_B = 64 * LDX * 2;                        // bytes of a 16-bit operand image
-    constexpr int PER_STEP = NDIR * 2 + QT * NKS;              // vector memory operations of a wave per step
+    constexpr int PER_STEP = NDIR * (S16 ? 1 : 2) + QT * NKS;  // vector memory operations of a wave per step
     static_assert(NDIR * NBLK <= DBDC_THREADS, "one block per thread");
+    static_assert(DBDC_WAVES == 8, "a wave brings 8 (16-bit) resp. 2 x 4 (float32) rows of each tile");
     __shared__ __attribute__((aligned(16))) unsigned char ring[RING * NDIR * TILE_B];
-    __shared__ __attribute__((aligned(16))) unsigned char img[2 * NDIR * IMG_B];
+    __shared__ __attribute__((aligned(16))) unsigned char img[S16 ? 16 : 2 * NDIR * IMG_B];
     __shared__ __attribute__((aligned(16))) float sfs[DBDC_HEADS][ROWS], sbs[DBDC_HEADS][ROWS];
     // the per-head decay gradients wait here for the end of the kernel: a global store inside the loop would sit in the
     // same counter as the requests and be waited for with them
@@ -568,11 +604,18 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
         const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * N + (int64_t)kc * KC * N;
 #pragma unroll
         for (int d = 0; d < NDIR; ++d) {
-            const float *st = (IS_DB ? (d ? p.dstates_b : p.dstates_f) : (d ? p.states_b : p.states_f)) + so;
+            if constexpr (S16) {
+                // rows 8 wave .. 8 wave + 7, 16-byte chunk (lane % 8) ^ swizzle(row) at chunk position lane % 8
+                const T *st = reinterpret_cast<const T *>(IS_DB ? (d ? p.dstates16_b : p.dstates16_f) : (d ? p.states16_b : p.states16_f)) + so;
+                const int row = wave * 8 + (lane >> 3);
+                load16_to_lds(st + row * 64 + (((lane & 7) ^ tile64_swz(row)) << 3), ring + ((step % RING) * NDIR + d) * TILE_B + wave * 1024);
+            } else {
+                const float *st = (IS_DB ? (d ? p.dstates_b : p.dstates_f) : (d ? p.states_b : p.states_f)) + so;
 #pragma unroll
-            for (int uu = 0; uu < 2; ++uu) {
-                const int u = wave * 2 + uu;
-                load16_to_lds(st + (4 * u + (lane >> 4)) * 64 + (lane & 15) * 4, ring + ((step % RING) * NDIR + d) * TILE_B + u * 1024);
+                for (int uu = 0; uu < 2; ++uu) {
+                    const int u = wave * 2 + uu;
+                    load16_to_lds(st + (4 * u + (lane >> 4)) * 64 + (lane & 15) * 4, ring + ((step % RING) * NDIR + d) * TILE_B + u * 1024);
+                }
             }
         }
     };
@@ -670,6 +713,17 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
         for (int j = 0; j < 4; ++j) img_r[ks][j] = lds_addr(img) + xt_index<T, LDX>(j * 16 + lr, ks * KSTEP + lg * 8) * 2;
     const unsigned sfs_a = lds_addr(sfs) + ((wave * QT) * 16 + lg * 4) * 4, sbs_a = lds_addr(sbs) + ((wave * QT) * 16 + lg * 4) * 4;
     const unsigned uvs_a = lds_addr(uvs) + ((wave * QT) * 16 + lg * 4) * 4;
+    // S16: lane parts of the transpose reads (see tile64_tr_frag): rows kk .. kk + 3 and kk + 4 .. kk + 7 of a K step,
+    // 4 columns from 16 j + nn on; the K step adds 32 rows = 4096 bytes (the swizzle repeats every 16 rows)
+    unsigned tr_lo[4], tr_hi[4];
+    {
+        const int kk = 8 * lg + (lr >> 2), nn = 4 * (lr & 3);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            tr_lo[j] = lds_addr(ring) + tile64_tr_offset(kk, j * 16 + nn);
+            tr_hi[j] = lds_addr(ring) + tile64_tr_offset(kk + 4, j * 16 + nn);
+        }
+    }
     f32x4 tf[QT][4], tb[QT][4];
     auto step_body = [&](int step, Frag (&af)[QT][NKS]) {
         const int hh = hh0 + step / nkc, kc = step % nkc;
@@ -679,6 +733,7 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
         raw_lds_barrier();                                     // ... and everybody's; ring slot and image of step - 1 are free
         if (step + 2 < nsteps) issue_states(step + 2);
         const int buf = step & 1;
+        if constexpr (!S16) {
         if (stile < NDIR) {
             // 8 rows (k = p) x 4 columns (n) of the tile from the ring, transposed into the image
             const unsigned ra = ring_a + ((step % RING) * NDIR) * TILE_B;
@@ -700,6 +755,7 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
         }
         raw_lds_wait();
         raw_lds_barrier();
+        }
         if (kc == 0) {
 #pragma unroll
             for (int q = 0; q < QT; ++q)
@@ -711,13 +767,37 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) raw_lds_use(af[q][ks]);
         const unsigned ib = buf * NDIR * IMG_B;
+        const unsigned rb = ((step % RING) * NDIR) * TILE_B;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
             Frag bff[4], bfb[4];
+            if constexpr (S16) {
+                i16x4 flo[4], fhi[4], blo[4], bhi[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (ks == 0) { flo[j] = raw_lds_tr16_read_at<0>(tr_lo[j] + rb); fhi[j] = raw_lds_tr16_read_at<0>(tr_hi[j] + rb); }
+                    else { flo[j] = raw_lds_tr16_read_at<4096>(tr_lo[j] + rb); fhi[j] = raw_lds_tr16_read_at<4096>(tr_hi[j] + rb); }
+                    if (!UNI) {
+                        if (ks == 0) { blo[j] = raw_lds_tr16_read_at<TILE_B>(tr_lo[j] + rb); bhi[j] = raw_lds_tr16_read_at<TILE_B>(tr_hi[j] + rb); }
+                        else { blo[j] = raw_lds_tr16_read_at<TILE_B + 4096>(tr_lo[j] + rb); bhi[j] = raw_lds_tr16_read_at<TILE_B + 4096>(tr_hi[j] + rb); }
+                    }
+                }
+                raw_lds_wait();
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    raw_lds_use(flo[j]); raw_lds_use(fhi[j]);
+                    bff[j] = __builtin_bit_cast(Frag, __builtin_shufflevector(flo[j], fhi[j], 0, 1, 2, 3, 4, 5, 6, 7));
+                    if (!UNI) {
+                        raw_lds_use(blo[j]); raw_lds_use(bhi[j]);
+                        bfb[j] = __builtin_bit_cast(Frag, __builtin_shufflevector(blo[j], bhi[j], 0, 1, 2, 3, 4, 5, 6, 7));
+                    }
+                }
+            } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 bff[j] = raw_lds_read_at<Frag, 0>(img_r[ks][j] + ib);
                 if (!UNI) bfb[j] = raw_lds_read_at<Frag, IMG_B>(img_r[ks][j] + ib);
+            }
             }
             raw_lds_wait();
 #pragma unroll
@@ -806,18 +886,22 @@ static int launch_dbdc_t(const bimamba2_params *p) {
     } while (0)
     if constexpr (sizeof(T) == 2) {
         // dstate 64: the variant with the ring of state tiles (16-byte aligned state tensors)
-        const bool st_al = IS_DB ? al(p->dstates_f) && al(p->dstates_b) : al(p->states_f) && al(p->states_b);
+        const void *c16f = IS_DB ? p->dstates16_f : p->states16_f, *c16b = IS_DB ? p->dstates16_b : p->states16_b;
+        const bool st_al = c16f ? al(c16f) && al(c16b) && (p->causal || c16b)
+                                : (IS_DB ? al(p->dstates_f) && al(p->dstates_b) : al(p->states_f) && al(p->states_b));
         if (fast && p->dstate == 64 && st_al) {
-            if (p->causal) {
-                if (qt == 2) hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 2, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
-                else hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 1, IS_DB, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
-            } else {
-                if (qt == 2) hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 2, IS_DB, false>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
-                else hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, 1, IS_DB, false>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);
-            }
+#define BM2_DMA(QTV, UNIV)                                                                                                                  \
+    do {                                                                                                                                    \
+        if (c16f) hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, QTV, IS_DB, UNIV, true>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);   \
+        else hipLaunchKernelGGL((bwd_dbdc_dma_kernel<T, QTV, IS_DB, UNIV, false>), grid, dim3(DBDC_THREADS), 0, stream_of(p), *p, nc);       \
+    } while (0)
+            if (p->causal) { if (qt == 2) BM2_DMA(2, true); else BM2_DMA(1, true); }
+            else { if (qt == 2) BM2_DMA(2, false); else BM2_DMA(1, false); }
+#undef BM2_DMA
             return check_launch();
         }
     }
+    if (IS_DB ? p->dstates16_f : p->states16_f) return BIMAMBA2_EUNSUPPORTED;   // only the kernel above knows the 16-bit copies
     if (p->causal) {
         if constexpr (sizeof(T) == 2) {
             if (fast && nt == 1) {

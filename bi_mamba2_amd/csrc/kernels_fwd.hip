@@ -593,6 +593,8 @@ bool chunk_state_does_cumsum(const bimamba2_params *p) {
 // together, unconditionally (past the last chunk a valid chunk is read again and not used).  Needs P*N % 4 == 0 and
 // 16-byte aligned tensors.
 // ndir = 1: the forward recurrence only (blockIdx.z = b).
+// T16 != void: the entering states go to the 16-bit copies (states16_*) and the per-chunk states stay as they are.
+template <typename T16>
 __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const bimamba2_params p, int nc, int ndir) {
     const int PN = p.headdim * p.dstate;
     const int e = (blockIdx.x * NTHREADS + threadIdx.x) * 4;
@@ -602,6 +604,10 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const b
     const float *cs = (dir == 0 ? p.cs_f : p.cs_b) + ((int64_t)b * p.nheads + h) * nc * Q + (dir == 0 ? Q - 1 : 0);
     const int64_t cstride = (int64_t)p.nheads * PN;
     float *st = (dir == 0 ? p.states_f : p.states_b) + ((int64_t)b * nc * p.nheads + h) * PN + e;
+    constexpr bool COPY = !std::is_same<T16, void>::value;
+    typedef typename std::conditional<COPY, T16, bf16_t>::type TC;
+    struct alignas(8) Out4 { TC v[4]; };
+    TC *st16 = reinterpret_cast<TC *>(dir == 0 ? p.states16_f : p.states16_b) + ((int64_t)b * nc * p.nheads + h) * PN + e;
     const float *ini = dir == 0 ? p.initial_f : p.initial_b;
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
     if (ini) s = *reinterpret_cast<const f32x4 *>(ini + ((int64_t)b * p.nheads + h) * PN + e);
@@ -618,7 +624,14 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const b
         for (int i = 0; i < 8; ++i)
             if (s0 + i < nc) {
                 const int c = dir == 0 ? s0 + i : nc - 1 - (s0 + i);
-                *reinterpret_cast<f32x4 *>(st + c * cstride) = s;
+                if constexpr (COPY) {
+                    Out4 o;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) o.v[k] = from_f<TC>(s[k]);
+                    *reinterpret_cast<Out4 *>(st16 + c * cstride) = o;
+                } else {
+                    *reinterpret_cast<f32x4 *>(st + c * cstride) = s;
+                }
                 s = __expf(d[i]) * s + v[i];
             }
     }
@@ -632,9 +645,17 @@ int launch_state_passing_fwd(const bimamba2_params *p) {
     const int ndir = p->causal ? 1 : 2;
     if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->final_f) && al(p->final_b) && al(p->initial_f) && al(p->initial_b)) {
         dim3 grid((PN / 4 + NTHREADS - 1) / NTHREADS, p->nheads, p->batch * ndir);
-        hipLaunchKernelGGL(state_passing_fwd_vec_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, ndir);
+        if (p->states16_f) {
+            if (!(p->causal || p->states16_b) || !al(p->states16_f) || !al(p->states16_b)) return BIMAMBA2_EINVAL;
+            if (p->dtype == BIMAMBA2_BF16) hipLaunchKernelGGL(state_passing_fwd_vec_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, ndir);
+            else if (p->dtype == BIMAMBA2_F16) hipLaunchKernelGGL(state_passing_fwd_vec_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, ndir);
+            else return BIMAMBA2_EUNSUPPORTED;
+        } else {
+            hipLaunchKernelGGL(state_passing_fwd_vec_kernel<void>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, ndir);
+        }
         return check_launch();
     }
+    if (p->states16_f) return BIMAMBA2_EUNSUPPORTED;
     if (p->causal) return BIMAMBA2_EUNSUPPORTED;
     dim3 grid((PN + NTHREADS - 1) / NTHREADS, p->nheads, p->batch);
     hipLaunchKernelGGL(state_passing_fwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);

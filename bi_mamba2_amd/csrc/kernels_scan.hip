@@ -199,7 +199,17 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             static_assert(NF == 0 || NF * KSTEP == NW, "one round of state tiles");
             // full 64 x 64 float tiles (the launcher checked it): every 16-byte load of both tiles goes out
             // before the first one is converted
-            {
+            const T *s16f = reinterpret_cast<const T *>(BWD ? p.dstates16_f : p.states16_f);
+            if (s16f) {
+                // the 16-bit copies of the entering states: 64 x 64 elements per direction, 16 bytes per thread
+                static_assert(PW * NW * (int)sizeof(T) == SCAN_THREADS * 16, "one 16-byte unit per thread and direction");
+                const T *s16b = reinterpret_cast<const T *>(BWD ? p.dstates16_b : p.states16_b);
+                const f32x4 rf = *reinterpret_cast<const f32x4 *>(s16f + so + threadIdx.x * VS);
+                const f32x4 rb = UNI ? rf : *reinterpret_cast<const f32x4 *>(s16b + so + threadIdx.x * VS);
+                const int r = threadIdx.x / (NW / VS), k0 = (threadIdx.x % (NW / VS)) * VS;
+                *reinterpret_cast<f32x4 *>(sF + r * LDS_ + k0) = rf;
+                *reinterpret_cast<f32x4 *>(sB + r * LDS_ + k0) = rb;
+            } else {
                 constexpr int PER = PW * NW / 4 / SCAN_THREADS;
                 float4 rawf[PER], rawb[PER];
 #pragma unroll
@@ -672,6 +682,9 @@ static int launch_scan_t(const bimamba2_params *p) {
         else hipLaunchKernelGGL((chunk_scan_kernel<T, QTV, NJV, BWD, false, 0>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);     \
     } while (0)
     const int qt = Q <= 128 ? 1 : 2;             // 16-row tiles per wave (8 waves)
+    // 16-bit copies of the entering states: known to the kernels that rebuild CB only
+    const void *c16f = BWD ? p->dstates16_f : p->states16_f, *c16b = BWD ? p->dstates16_b : p->states16_b;
+    if (c16f && (!al16(c16f) || !al16(c16b) || !(p->causal || c16b))) return BIMAMBA2_EINVAL;
     if constexpr (sizeof(T) == 2 && NJMAX == 4) {
         if (p->causal) {                                // single-direction comparator: the fused kernels only
             if (!scan_recomputes_cb(p, BWD)) return BIMAMBA2_EUNSUPPORTED;
@@ -685,7 +698,7 @@ static int launch_scan_t(const bimamba2_params *p) {
             return check_launch();
         }
     }
-    if (p->causal) return BIMAMBA2_EUNSUPPORTED;
+    if (p->causal || c16f) return BIMAMBA2_EUNSUPPORTED;
     if ((BWD ? p->CBT : p->CB) == nullptr) return BIMAMBA2_EINVAL;
     if (pw == 16) { if (qt == 1) BM2_SCAN(1, 1); else BM2_SCAN(2, 1); }
     else if (pw == 32) { if (qt == 1) BM2_SCAN(1, 2); else BM2_SCAN(2, 2); }

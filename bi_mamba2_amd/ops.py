@@ -142,7 +142,9 @@ class _Call:
                bool(p.dstates_f), bool(p.dout_x), bool(p.red), bool(p.dBs), bool(p.da_intra),
                p.x_sb, p.x_sl, p.x_sh, p.z_sb, p.z_sl, p.z_sh, p.dout_sb, p.dout_sl, p.dout_sh, p.B_sb, p.B_sl, p.B_sg,
                p.C_sb, p.C_sl, p.C_sg, al(p.x), al(p.z), al(p.dout), al(p.Bm), al(p.Cm), al(p.out), al(p.out_x), al(p.dx),
-               al(p.states_f), al(p.states_b), al(p.dstates_f), al(p.dstates_b))
+               al(p.states_f), al(p.states_b), al(p.dstates_f), al(p.dstates_b),
+               bool(p.states16_f), bool(p.dstates16_f), p.fwd_saved, al(p.states16_f), al(p.states16_b), al(p.final_f), al(p.final_b),
+               al(p.initial_f), al(p.initial_b), al(p.dfinal_f), al(p.dfinal_b), al(p.dinitial_f), al(p.dinitial_b))
         n = _WS_CACHE.get(key)
         if n is None:
             n = _WS_CACHE[key] = self._workspace_bytes(is_bwd)
@@ -459,10 +461,14 @@ def _problem(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit):
 _BLOB_FIELDS = ("dt_out", "cs_f", "cs_b", "states_f", "states_b")
 
 
-def _point_into(c, blob, offs):
+# the same with the entering states in the library's 16-bit copies (half the size) instead of float32
+_BLOB_FIELDS_COPIES = ("dt_out", "cs_f", "cs_b", "states16_f", "states16_b")
+
+
+def _point_into(c, blob, offs, fields=_BLOB_FIELDS):
     """Points the five forward intermediates at their places (float offsets) inside one float32 allocation."""
     base = blob.data_ptr()
-    for field, o in zip(_BLOB_FIELDS, offs):
+    for field, o in zip(fields, offs):
         setattr(c.p, field, base + 4 * o)
     c.keep.append(blob)
 
@@ -511,10 +517,14 @@ def _mamba_chunk_scan_combined_fwd(x, dt, A, B, C, chunk_size, D=None, z=None, d
         # overhead); the snapshot below carries the pointers
         n1 = (batch * nheads * c.nchunks * chunk_size + 63) // 64 * 64
         n2 = (batch * c.nchunks * nheads * headdim * dstate + 63) // 64 * 64
-        blob = torch.empty(3 * n1 + 2 * n2, device=x.device, dtype=torch.float32)
-        offs = (0, n1, 2 * n1, 3 * n1, 3 * n1 + n2)
-        _point_into(c, blob, offs)
-        snap = c.snapshot() + (offs,)
+        # where the kernels can, the states entering the chunks are kept in the input's 16-bit type only
+        copies = bool(_lib.load().bimamba2_state_copies(c.p))
+        fields = _BLOB_FIELDS_COPIES if copies else _BLOB_FIELDS
+        ns = n2 // 2 if copies else n2
+        blob = torch.empty(3 * n1 + 2 * ns, device=x.device, dtype=torch.float32)
+        offs = (0, n1, 2 * n1, 3 * n1, 3 * n1 + ns)
+        _point_into(c, blob, offs, fields)
+        snap = c.snapshot() + (offs, fields)
         saved = ("blob", blob, snap)
     else:
         snap = c.snapshot() if keep_for_bwd else None
@@ -574,7 +584,7 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
                       for f, t in zip(("dinitial_f", "dinitial_b"), initial_states))
     c.set_dout(dout)
     if blob is not None:
-        _point_into(c, blob, snap[2])
+        _point_into(c, blob, snap[2], snap[3])
         c.p.fwd_saved = 1
     elif saved is not None:
         for name, t in zip(_BLOB_FIELDS, saved[:5]):

@@ -114,6 +114,21 @@ typedef struct bimamba2_params {
        the forward cumulative sum gets BIMAMBA2_SEQ_CUT added at the first position of a sequence, the reverse one at
        the last, so that every decay factor across a change underflows to zero and no other kernel needs to know. */
     const int32_t *seq_idx;
+    /* Optional 16-bit copies of the states that enter the chunks (element type `dtype`, which must be a 16-bit one;
+       same shape as states_* / dstates_*).  Every kernel that reads entering states rounds them to `dtype` for its MFMA
+       anyway; kept in that type they cost half the memory traffic.  When states16_f / states16_b are given,
+       bimamba2_state_passing_fwd writes the entering states there and leaves the per-chunk states in states_f / states_b
+       as they were, and bimamba2_chunk_scan_fwd, bimamba2_chunk_scan_bwd_dc and bimamba2_state_passing_bwd read them
+       from there.  dstates16_f / dstates16_b likewise: written by bimamba2_state_passing_bwd (dstates_f / dstates_b keep
+       the per-chunk gradients), read by bimamba2_chunk_scan_bwd_dx and bimamba2_chunk_state_bwd_db.  Only the kernels for
+       16-bit dtype, dstate 64, headdim % 64 == 0, chunk_size % 64 == 0 and 16-byte aligned operands know them
+       (bimamba2_state_copies() == 1); the others return BIMAMBA2_EUNSUPPORTED when they are set.
+       bimamba2_fwd / bimamba2_bwd use such copies on their own, from the workspace, where the caller leaves states_f
+       resp. dstates_f NULL (does not ask for the float32 entering states); a caller that keeps the forward's intermediates
+       for the backward pass (fwd_saved) then passes states16_f / states16_b to both instead of states_f / states_b.
+       The reference keeps its entering states in the input dtype as well (out_dtype=C.dtype, src/ssd/bi/ssd_combined.py:324-327). */
+    void *states16_f, *states16_b;
+    void *dstates16_f, *dstates16_b;
     void *workspace;
     size_t workspace_bytes;
     void *stream;                   /* hipStream_t */
@@ -128,6 +143,9 @@ size_t bimamba2_params_size(void);
 
 /* bytes of workspace the composite entry points need (is_bwd = 0: forward, 1: backward) */
 size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd);
+
+/* 1 if the kernels of this problem can keep the entering states in 16-bit copies (see states16_f), else 0 */
+int bimamba2_state_copies(const bimamba2_params *p);
 
 /* Whether a kernel of this problem reads CB (1) or rebuilds the CB tiles it needs from the C and B rows with MFMAs (0):
  *   which = 0: bimamba2_chunk_scan_fwd reads CB      (0 for 16-bit dtype, dstate 64, headdim % 64 == 0, chunk_size % 32 == 0)

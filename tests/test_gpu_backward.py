@@ -88,3 +88,37 @@ def test_backward_with_recomputation(ops, case, monkeypatch):
     inp = make_case(b, L, H, P, G, N, dtype, with_z=z, with_D=(Dk != "none"), D_has_hdim=(Dk == "hp"), with_bias=bias)
     out, grads, ref = _run_bwd(ops, inp, Q, sp, lim)
     _check(out, grads, ref, dtype)
+
+
+def test_sixteen_bit_state_copies_change_nothing_but_the_chunk_decay_gradient(ops):
+    """Where the kernels can, the composites keep the states entering the chunks (and their gradients) in copies of the
+    input's 16-bit type instead of float32.  Every kernel that reads them rounded them to that type for its MFMA before,
+    so out, dx, dz, dB and dC must come out bit for bit as with float32 states; only the gradient of the chunk decays
+    (a float32 dot product with the entering states inside the backward state passing, which feeds ddt and dA) sees
+    the rounding.  The float32 side: forward with the states returned as tensors, which switches the copies off."""
+    import ctypes
+    from bi_mamba2_amd import _lib
+    Q = 256
+    inp = make_case(2, 700, 4, 64, 2, 64, torch.bfloat16, with_z=True)
+    d = to_dev(inp)
+    args = (d["x"], d["dt"], d["A"], d["B"], d["C"], Q)
+    kw = dict(D=d["D"], z=d["z"], dt_bias=d["dt_bias"], dt_softplus=True)
+    dout = torch.randn(d["x"].shape, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).cuda()
+
+    c = ops._problem(*args, d["D"], d["z"], d["dt_bias"], True, (0.0, INF))
+    assert _lib.load().bimamba2_state_copies(ctypes.byref(c.p)) == 1
+    c32 = ops._problem(d["x"].float(), d["dt"], d["A"], d["B"].float(), d["C"].float(), Q, d["D"], d["z"].float(), d["dt_bias"], True, (0.0, INF))
+    assert _lib.load().bimamba2_state_copies(ctypes.byref(c32.p)) == 0
+
+    res_c = ops._mamba_chunk_scan_combined_fwd(*args, **kw, return_intermediates=False, keep_for_bwd=True)
+    assert res_c[9][2][3] == ops._BLOB_FIELDS_COPIES
+    res_f = ops._mamba_chunk_scan_combined_fwd(*args, **kw, return_intermediates=True, keep_for_bwd=True)
+    assert torch.equal(res_c[0], res_f[0]) and torch.equal(res_c[1], res_f[1])
+    g_c = ops._mamba_chunk_scan_combined_bwd(dout, *args[:5], res_c[1], Q, **kw, saved=res_c[9])
+    g_f = ops._mamba_chunk_scan_combined_bwd(dout, *args[:5], res_f[1], Q, **kw, saved=res_f[9])
+    names = ("dx", "ddt", "dA", "dB", "dC", "dD", "dz", "ddt_bias")
+    for name, a, b in zip(names, g_c, g_f):
+        if name in ("ddt", "dA", "ddt_bias"):
+            assert_close(a, b.double(), torch.bfloat16, name)
+        else:
+            assert torch.equal(a, b), name
