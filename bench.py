@@ -312,7 +312,7 @@ def main():
         c.new("dout_x", inp["x"].shape, dtype)
     nsplit = (w["headdim"] * w["dstate"] + 1023) // 1024
     c.new("ddA_chunk_f", (w["batch"], w["nheads"], nc, nsplit)); c.new("ddA_chunk_b", (w["batch"], w["nheads"], nc, nsplit))
-    slices = (w["nheads"] // w["ngroups"] + 3) // 4
+    slices = (w["nheads"] // w["ngroups"] + 7) // 8
     c.new("dBs", (slices,) + tuple(inp["B"].shape)); c.new("dCs", (slices,) + tuple(inp["B"].shape))
     c.new("red", (w["batch"] * nc * w["nheads"] * w["headdim"] + 2 * w["batch"] * nc * w["nheads"],))
     c.run("bimamba2_fwd")

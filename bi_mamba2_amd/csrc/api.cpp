@@ -101,7 +101,7 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
         need_f(q->da_intra, (size_t)q->batch * q->nheads * nc * nqt * nqt * 128);
         need_f(q->ddA_chunk_f, (size_t)q->batch * q->nheads * nc * sp_nsplit(q));
         need_f(q->ddA_chunk_b, (size_t)q->batch * q->nheads * nc * sp_nsplit(q));
-        const size_t slices = (q->nheads / q->ngroups + 3) / 4;   // head slices of the dB / dC partial sums
+        const size_t slices = (q->nheads / q->ngroups + 7) / 8;   // head slices of the dB / dC partial sums
         const size_t bn = slices * q->batch * q->seqlen * q->ngroups * q->dstate;
         need_f(q->dBs, bn);
         need_f(q->dCs, bn);

@@ -182,8 +182,8 @@ def _check_chunk(chunk_size):
 
 
 def _slices(nheads, ngroups):
-    """Number of head slices whose partial dB / dC sums the kernels keep apart (4 heads per slice)."""
-    return (nheads // ngroups + 3) // 4
+    """Number of head slices whose partial dB / dC sums the kernels keep apart (8 heads per slice)."""
+    return (nheads // ngroups + 7) // 8
 
 
 def _bhcq(c):

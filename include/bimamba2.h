@@ -93,7 +93,7 @@ typedef struct bimamba2_params {
     float *ddt_direct, *u_f, *u_b, *v_f, *v_b;
     float *da_intra;                    /* (B, H, nc, T*T, 2, 64), T = ceil(Q/64): per-tile column / row sums */
     float *ddA_chunk_f, *ddA_chunk_b;   /* (B, H, nc, ceil(P*N/1024)) partial sums */
-    float *dBs, *dCs;                   /* (S, B, L, G, N) float32 partial gradients, S = ceil(H/G/4) head slices */
+    float *dBs, *dCs;                   /* (S, B, L, G, N) float32 partial gradients, S = ceil(H/G/8) head slices */
     float *red;                         /* scratch for two-stage reductions: max(B*nc*H*P, 2*B*nc*H) floats for the single
                                            stages, B*nc*H*P + 2*B*nc*H for bimamba2_bwd */
     /* States at the ends of the sequence, all (B, H, P, N) float32, all optional (NULL = absent).  The reference's
