@@ -320,10 +320,20 @@ int bimamba2_bwd(const bimamba2_params *p) {
     if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
     // the dCB kernel is bound by instruction issue and moves little data: right behind dz it runs while the memory system
     // still writes back dz's output, which the memory-bound kernels after it would otherwise wait behind
-    TRY(bimamba2_chunk_scan_bwd_dcb(&q));
-    TRY(bimamba2_chunk_scan_bwd_dstates(&q));
-    TRY(bimamba2_chunk_scan_bwd_dc(&q));           // (between the two memory-bound state kernels: measured best)
-    TRY(bimamba2_state_passing_bwd(&q));
+    if (bwd_dcb_sp_merged(&q)) {
+        // the backward state passing (streams, few instructions) rides along with the dCB kernel in one launch
+        TRY(bimamba2_chunk_scan_bwd_dc(&q));
+        TRY(bimamba2_chunk_scan_bwd_dstates(&q));
+        REQUIRE(q.x); REQUIRE(q.dt_out); REQUIRE(q.cs_f); REQUIRE(q.cs_b); REQUIRE(q.dCB); REQUIRE(q.dCBT); REQUIRE(q.da_intra);
+        REQUIRE(q.dstates_f); REQUIRE(q.ddA_chunk_f); REQUIRE(q.ddA_chunk_b);
+        if (q.has_z) REQUIRE(q.dout_x); else REQUIRE(q.dout);
+        TRY(launch_bwd_dcb_sp(&q));
+    } else {
+        TRY(bimamba2_chunk_scan_bwd_dcb(&q));
+        TRY(bimamba2_chunk_scan_bwd_dstates(&q));
+        TRY(bimamba2_chunk_scan_bwd_dc(&q));           // (between the two memory-bound state kernels: measured best)
+        TRY(bimamba2_state_passing_bwd(&q));
+    }
     TRY(bimamba2_chunk_state_bwd_db(&q));
     ReduceJobs jobs;
     {

@@ -16,6 +16,9 @@ namespace bm2 {
 static inline int nchunks(const bimamba2_params *p) { return (p->seqlen + p->chunk_size - 1) / p->chunk_size; }
 static inline hipStream_t stream_of(const bimamba2_params *p) { return reinterpret_cast<hipStream_t>(p->stream); }
 
+// block index of a kernel body that may run as one of several roles of a launch
+struct BlockId { int x, y, z; };
+
 // =========================================================================================================
 __global__ void fill_kernel(float *ptr, size_t n, float value) {
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) ptr[i] = value;
@@ -219,11 +222,11 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_kernel(const bimam
 // entering states go to dstates16_* and the per-chunk gradients in dstates_* stay as they are.
 constexpr int SP_CH = 8;
 template <typename T16, bool PREV16, bool DS16>
-__global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const bimamba2_params p, int nc, int nsplit, int ndir) {
+__device__ __forceinline__ void state_passing_bwd_vec_body(const bimamba2_params &p, int nc, int nsplit, int ndir, BlockId bid) {
     struct alignas(8) V4 { T16 v[4]; };
     __shared__ float red[SP_CH][4];
     const int PN = p.headdim * p.dstate;
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z / ndir, dir = blockIdx.z % ndir;   // ndir = 1: forward direction only
+    const int split = bid.x, h = bid.y, b = bid.z / ndir, dir = bid.z % ndir;   // ndir = 1: forward direction only
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int Q = p.chunk_size;
     const float *cs = (dir == 0 ? p.cs_f : p.cs_b) + ((int64_t)b * p.nheads + h) * nc * Q + (dir == 0 ? Q - 1 : 0);
@@ -290,6 +293,10 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const b
         __syncthreads();
     }
     if (dini && live) *reinterpret_cast<f32x4 *>(dini + bh) = g;
+}
+template <typename T16, bool PREV16, bool DS16>
+__global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const bimamba2_params p, int nc, int nsplit, int ndir) {
+    state_passing_bwd_vec_body<T16, PREV16, DS16>(p, nc, nsplit, ndir, BlockId{(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z});
 }
 
 int launch_state_passing_bwd(const bimamba2_params *p) {
@@ -1274,8 +1281,9 @@ constexpr int DCB_PART_B = 10 * 64 * 4;
 #endif
 
 // UNI: the single-direction operator - tiles above the diagonal are empty, tiles on it keep the forward half.
-template <typename T, bool UNI = false>
-__global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_params p, int nc, int nqt) {
+// bid / gdx / gdz: block index and grid extents (x: batch * chunks * groups, y: tiles, z: head slices)
+template <typename T, bool UNI>
+__device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int nc, int nqt, BlockId bid, int gdx, int gdz) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
     static_assert(sizeof(T) == 2, "ring variant is for 16-bit operands");
@@ -1285,23 +1293,23 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
     const int lr = lane & 15, lg = lane >> 4;
     // the tiles on the diagonal cost more: they come first in launch order, which spreads them over the compute units
     int tt, st;
-    if ((int)blockIdx.y < nqt) tt = st = blockIdx.y;
+    if (bid.y < nqt) tt = st = bid.y;
     else {
-        const int k = blockIdx.y - nqt;
+        const int k = bid.y - nqt;
         tt = k / (nqt - 1);
         st = k % (nqt - 1);
         st += st >= tt;
     }
     const int tile = tt * nqt + st;
-    const int g = blockIdx.x % p.ngroups, bc = blockIdx.x / p.ngroups, c = bc % nc, b = bc / nc;
+    const int g = bid.x % p.ngroups, bc = bid.x / p.ngroups, c = bc % nc, b = bc / nc;
     const int Q = p.chunk_size, P = p.headdim, H = p.nheads, hpg = H / p.ngroups;
     const int limit = min(Q, p.seqlen - c * Q);
     const int t0 = tt * 64, s0 = st * 64;
     const bool live = t0 < limit && s0 < limit && !(UNI && st > tt);
     const int trow = wave * 16 + lg * 4;                       // first of this lane's four accumulator rows
     f32x4 cbr[4] = {}, dcb[4] = {};
-    const int hps = (hpg + gridDim.z - 1) / gridDim.z;
-    const int h_begin = blockIdx.z * hps, h_end = min(hpg, h_begin + hps);
+    const int hps = (hpg + gdz - 1) / gdz;
+    const int h_begin = bid.z * hps, h_end = min(hpg, h_begin + hps);
     const int nkc = P / KC, nhs = h_end - h_begin, nit = nhs * nkc;
     const int h0 = g * hpg + h_begin;
     const int64_t tv_head = (int64_t)nc * nqt * nqt * DCB_VEC;
@@ -1604,13 +1612,13 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
         }
 #ifdef BM2_DBG_TIME
         if (threadIdx.x == 0) {
-            long long *lg2 = reinterpret_cast<long long *>(p.workspace) + (blockIdx.y * gridDim.x + blockIdx.x) * 16;
+            long long *lg2 = reinterpret_cast<long long *>(p.workspace) + (bid.y * gdx + bid.x) * 16;
             for (int k = 0; k < 10; ++k) lg2[k] = ph[k];
             lg2[10] = tstart; lg2[11] = tlast;
         }
 #endif
     }
-    const int64_t oo = ((int64_t)blockIdx.z * gridDim.x + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    const int64_t oo = ((int64_t)bid.z * gdx + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
     float *out = p.dCB + oo, *outT = p.dCBT + oo;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -1618,6 +1626,27 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
 #pragma unroll
         for (int i = 0; i < 4; ++i) out[(int64_t)(t0 + trow + i) * Q + s] = dcb[j][i];
         *reinterpret_cast<f32x4 *>(outT + (int64_t)s * Q + t0 + trow) = dcb[j];
+    }
+}
+
+template <typename T, bool UNI = false>
+__global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_params p, int nc, int nqt) {
+    bwd_dcb_ring_body<T, UNI>(p, nc, nqt, BlockId{(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z}, gridDim.x, gridDim.z);
+}
+
+// The dCB kernel and the backward state passing as roles of one launch (16-bit copies of the entering states on both sides
+// of the state passing, one head slice): the first is bound by instruction issue and moves little data, the second streams
+// 70 MB and needs few instructions, and the two depend on different kernels before them.  The first ndcb blocks are the
+// dCB tiles in the order of their own grid (so they are placed first, two per CU as when alone), the rest are the state
+// passing's blocks, which take what is left of each CU.
+template <typename T, bool UNI>
+__global__ __launch_bounds__(NTHREADS) void bwd_dcb_sp_kernel(const bimamba2_params p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir) {
+    const int id = blockIdx.x;
+    if (id < ndcb) {
+        bwd_dcb_ring_body<T, UNI>(p, nc, nqt, BlockId{id % gdx, id / gdx, 0}, gdx, 1);
+    } else {
+        const int k = id - ndcb;                  // grid (nsplit, nheads, batch * ndir) of the state passing
+        state_passing_bwd_vec_body<T, true, true>(p, nc, nsplit, ndir, BlockId{k % nsplit, (k / nsplit) % p.nheads, k / (nsplit * p.nheads)});
     }
 }
 
@@ -1664,6 +1693,34 @@ static int launch_dcb_t(const bimamba2_params *p) {
     return check_launch();
 }
 
+// whether bwd_dcb_sp_kernel exists for the problem (the ring variant of the dCB kernel with one head slice, the vector
+// variant of the state passing, 16-bit copies of the entering states and of their gradients)
+bool bwd_dcb_sp_merged(const bimamba2_params *p) {
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    if (p->dtype != BIMAMBA2_BF16 && p->dtype != BIMAMBA2_F16) return false;
+    if (!dcb_recomputes_cb(p) || dcb_slices(p) != 1) return false;       // (implies the conditions of the ring variant)
+    if (!p->states16_f || !p->dstates16_f || !(p->causal || (p->states16_b && p->dstates16_b))) return false;
+    if ((p->headdim * p->dstate) % 4) return false;
+    return al(p->states16_f) && al(p->states16_b) && al(p->dstates16_f) && al(p->dstates16_b) && al(p->dstates_f) && al(p->dstates_b) &&
+           al(p->dfinal_f) && al(p->dfinal_b) && al(p->dinitial_f) && al(p->dinitial_b);
+}
+
+// bimamba2_chunk_scan_bwd_dcb and bimamba2_state_passing_bwd in one launch (the caller checked bwd_dcb_sp_merged())
+int launch_bwd_dcb_sp(const bimamba2_params *p) {
+    const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64, PN = p->headdim * p->dstate;
+    const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS), ndir = p->causal ? 1 : 2;
+    const int gdx = p->batch * nc * p->ngroups, ndcb = gdx * nqt * nqt, nsp = nsplit * p->nheads * p->batch * ndir;
+    dim3 grid(ndcb + nsp);
+#define BM2_DS(TT)                                                                                                                     \
+    do {                                                                                                                               \
+        if (p->causal) hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir);  \
+        else hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir);           \
+    } while (0)
+    if (p->dtype == BIMAMBA2_BF16) BM2_DS(bf16_t); else BM2_DS(f16_t);
+#undef BM2_DS
+    return check_launch();
+}
+
 int launch_bwd_dcb(const bimamba2_params *p) {
     switch (p->dtype) {
         case BIMAMBA2_F32: return launch_dcb_t<float>(p);
@@ -1680,7 +1737,7 @@ int launch_bwd_dcb(const bimamba2_params *p) {
 // =========================================================================================================
 // FAST (16-bit types, chunk_size == QP, dstate a multiple of 64, aligned operands, at most 8 slices): every global load
 // of a thread (its dCB row pieces, the slices it adds, the K operand) is requested before the first one is used.
-struct BlockId { int x, y, z; };
+
 
 template <typename T, int QP, bool FAST>
 __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int nc, int nslices, BlockId bid) {

@@ -32,6 +32,9 @@ int launch_reduce_jobs(const ReduceJobs &jobs, hipStream_t stream);
 // defer != NULL: the final reductions of dA and ddt_bias are appended to *defer instead of being launched
 int launch_chunk_cumsum_bwd(const bimamba2_params *p, ReduceJobs *defer = nullptr);
 // bmm_chunk_bwd and chunk_cumsum_bwd as one launch, where bwd_tail_merged() says it exists
+// the dCB kernel and the backward state passing as one launch, where bwd_dcb_sp_merged() says it exists
+bool bwd_dcb_sp_merged(const bimamba2_params *p);
+int launch_bwd_dcb_sp(const bimamba2_params *p);
 bool bwd_tail_merged(const bimamba2_params *p);
 int launch_bwd_tail(const bimamba2_params *p, ReduceJobs *defer);
 int launch_fill(float *ptr, size_t n, float value, hipStream_t stream);
