@@ -281,6 +281,23 @@ def main():
         for _ in range(args.warmup):
             causal_step()
         t_causal = timed(causal_step, args.steps)
+    # the same step recorded once into a HIP graph and replayed: what the GPU needs when the host does nothing but one
+    # launch per step (the eager figures above include the host's share whenever the host is the slower side)
+    t_graph = None
+    if not args.no_extras:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(args.warmup):
+            graph.replay()
+        t_graph = timed(graph.replay, args.steps)
     tokens = w["batch"] * w["seqlen"]
     fwd_b, bwd_b = whole_op_bytes(w, e, has_z)
 
@@ -411,6 +428,9 @@ def main():
             "bidirectional_over_causal": t_step / t_causal,
             "what": "single-direction SSD (y = SS(x) + D x, z gate) forward + backward from the same kernels with the "
                     "reverse direction compiled out, same shape and dtypes"}
+        result["graph_replay"] = {
+            "ms_per_step": t_graph * 1e3, "Mtokens_s": tokens / t_graph / 1e6,
+            "what": "the same forward + backward step captured once in a torch.cuda.CUDAGraph and replayed"}
         result["gated_rmsnorm"] = rmsnorm_line(w, dtype, dev, max(10, args.steps))
         result["conv1d_silu"] = conv_line(w, dtype, dev, max(10, args.steps))
     if not args.no_cpu:
