@@ -90,7 +90,8 @@ def test_backward_with_recomputation(ops, case, monkeypatch):
     _check(out, grads, ref, dtype)
 
 
-def test_sixteen_bit_state_copies_change_nothing_but_the_chunk_decay_gradient(ops):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_sixteen_bit_state_copies_change_nothing_but_the_chunk_decay_gradient(ops, dtype):
     """Where the kernels can, the composites keep the states entering the chunks (and their gradients) in copies of the
     input's 16-bit type instead of float32.  Every kernel that reads them rounded them to that type for its MFMA before,
     so out, dx, dz, dB and dC must come out bit for bit as with float32 states; only the gradient of the chunk decays
@@ -99,11 +100,11 @@ def test_sixteen_bit_state_copies_change_nothing_but_the_chunk_decay_gradient(op
     import ctypes
     from bi_mamba2_amd import _lib
     Q = 256
-    inp = make_case(2, 700, 4, 64, 2, 64, torch.bfloat16, with_z=True)
+    inp = make_case(2, 700, 4, 64, 2, 64, dtype, with_z=True)
     d = to_dev(inp)
     args = (d["x"], d["dt"], d["A"], d["B"], d["C"], Q)
     kw = dict(D=d["D"], z=d["z"], dt_bias=d["dt_bias"], dt_softplus=True)
-    dout = torch.randn(d["x"].shape, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).cuda()
+    dout = torch.randn(d["x"].shape, generator=torch.Generator().manual_seed(7)).to(dtype).cuda()
 
     c = ops._problem(*args, d["D"], d["z"], d["dt_bias"], True, (0.0, INF))
     assert _lib.load().bimamba2_state_copies(ctypes.byref(c.p)) == 1
@@ -119,6 +120,6 @@ def test_sixteen_bit_state_copies_change_nothing_but_the_chunk_decay_gradient(op
     names = ("dx", "ddt", "dA", "dB", "dC", "dD", "dz", "ddt_bias")
     for name, a, b in zip(names, g_c, g_f):
         if name in ("ddt", "dA", "ddt_bias"):
-            assert_close(a, b.double(), torch.bfloat16, name)
+            assert_close(a, b.double(), dtype, name)
         else:
             assert torch.equal(a, b), name
