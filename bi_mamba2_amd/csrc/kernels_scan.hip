@@ -336,7 +336,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             if (FAST && id >= 16 * CPR) continue;
             const int rc = min(r, limit - 1);
             load_vec(xrow + (int64_t)rc * p.x_sl + col, xvec, ncol, ex[B_][ps]);
-            if (need2) load_vec(row2 + (int64_t)rc * s2 + col, vec2, ncol, e2[B_][ps]);
+            if (need2 && !BWD) load_vec(row2 + (int64_t)rc * s2 + col, vec2, ncol, e2[B_][ps]);
         }
     };
     typedef std::integral_constant<int, 0> B0;
@@ -531,6 +531,24 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
 
     // ---- epilogue.  Each wave passes its 16-row accumulator tiles through a private LDS patch so that out, out_x,
     // dx are written (and x, z, dy were read) as 16-byte vectors along headdim ----
+    // mirror: the dy rows that the D term needs lie in the operand image (transposed, unscaled; zero past the end of the
+    // sequence and of headdim): they are read from there, 16-bit units a row of the image apart, before the image becomes
+    // the staging area - and before the global requests below, which an LDS access known to the compiler would wait for
+    if (BWD && need2) {
+#pragma unroll
+        for (int rt = 0; rt < QT; ++rt) {
+            if ((wave * QT + rt) * 16 < limit) {
+#pragma unroll
+                for (int ps = 0; ps < NPASS; ++ps) {
+                    const int id = lane + ps * 64;
+                    if (FAST && id >= 16 * CPR) continue;
+                    const int r = (wave * QT + rt) * 16 + min(id / CPR, 15), cc = (id % CPR) * VS;
+#pragma unroll
+                    for (int i = 0; i < VS; ++i) e2[rt][ps].v[i] = xT[xt_index<T, LDX>(cc + i, r)];
+                }
+            }
+        }
+    }
     // the epilogue operands of all row tiles are requested before the barrier
 #pragma unroll
     for (int rt = 0; rt < QT; ++rt) {
