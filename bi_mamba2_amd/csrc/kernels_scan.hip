@@ -57,6 +57,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     __shared__ __attribute__((aligned(16))) char shared_u[XT_BYTES + ST_BYTES > STG_BYTES ? XT_BYTES + ST_BYTES : STG_BYTES];
     __shared__ float lo[QP], up[QP];              // decay exponents (times log2 e), see below
     __shared__ float glo[QP], gup[QP];            // their column factors relative to the edge of the 16-block, see below
+    __shared__ float dtl[BWD ? 4 : QP];           // forward: dt of the columns, for the step across the diagonal
     __shared__ float red[SCAN_WAVES][PW];
     T *xT = reinterpret_cast<T *>(shared_u);
     T *sF = reinterpret_cast<T *>(shared_u + XT_BYTES), *sB = sF + PW * LDS_;
@@ -153,8 +154,12 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
         const float l = BWD ? -r : f, u = BWD ? -f : r;
         lo[q] = l;
         up[q] = u;
-        glo[q] = __builtin_amdgcn_exp2f((BWD ? -csb[qe] : csf[qe]) * LOG2E - l);
-        gup[q] = __builtin_amdgcn_exp2f((BWD ? -csf[qs] : csb[qs]) * LOG2E - u);
+        // forward: dt[k] of the source position rides on the column factors (and on the diagonal step through dtl), so
+        // that the operand image holds x as it is and the D term can take x from there
+        const float dtq = BWD ? 1.f : dto[qq];
+        glo[q] = __builtin_amdgcn_exp2f((BWD ? -csb[qe] : csf[qe]) * LOG2E - l) * dtq;
+        gup[q] = __builtin_amdgcn_exp2f((BWD ? -csf[qs] : csb[qs]) * LOG2E - u) * dtq;
+        if (!BWD) dtl[q] = dtq;
     }
     // K operand of part 2, transposed into LDS
     const T *kp;
@@ -162,8 +167,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     if (!BWD) { ks = p.x_sl; kp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * ks + h * p.x_sh; }
     else if (p.has_z) { ks = (int64_t)H * P; kp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * ks + (int64_t)h * P; }
     else { ks = p.dout_sl; kp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * ks + h * p.dout_sh; }
-    if (BWD) stage_transposed<T, QP, PW, LDX, FAST>(xT, kp + p0, ks, limit, P - p0, [&](int k) { return k < limit ? 1.f : 0.f; });
-    else stage_transposed<T, QP, PW, LDX, FAST>(xT, kp + p0, ks, limit, P - p0, [&](int k) { return k < limit ? dto[k] : 0.f; });
+    stage_transposed<T, QP, PW, LDX, FAST>(xT, kp + p0, ks, limit, P - p0, [&](int k) { return k < limit ? 1.f : 0.f; });
 
     typename M::Frag own[QT][NF > 0 ? NF : 1];     // NF > 0: this lane's rows, 32 dstate columns per fragment
     if constexpr (NF > 0) {
@@ -335,7 +339,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             const int ncol = (id < 16 * CPR && r < limit) ? P - col : 0;
             if (FAST && id >= 16 * CPR) continue;
             const int rc = min(r, limit - 1);
-            load_vec(xrow + (int64_t)rc * p.x_sl + col, xvec, ncol, ex[B_][ps]);
+            if (BWD) load_vec(xrow + (int64_t)rc * p.x_sl + col, xvec, ncol, ex[B_][ps]);
             if (need2 && !BWD) load_vec(row2 + (int64_t)rc * s2 + col, vec2, ncol, e2[B_][ps]);
         }
     };
@@ -405,6 +409,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                         const int k = kb + i;
                         const float e = k < r ? lor[rt] - lo[k] : upr[rt] - up[k];
                         v[i] = cbv[B_][rt][i] * ((k == r) ? 2.f : __builtin_amdgcn_exp2f(e));
+                        if (!BWD) v[i] *= dtl[min(k, QP - 1)];
                     }
                 }
                 const typename M::Frag af = M::pack(v);
@@ -477,8 +482,15 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                     const unsigned la = lds_addr(lo) + k0 * 4 + lg32, ua = lds_addr(up) + k0 * 4 + lg32;
                     f32x4 l0 = raw_lds_read_at<f32x4, 0>(la), l1 = raw_lds_read_at<f32x4, 16>(la);
                     f32x4 u0 = raw_lds_read_at<f32x4, 0>(ua), u1 = raw_lds_read_at<f32x4, 16>(ua);
+                    f32x4 d0 = {1.f, 1.f, 1.f, 1.f}, d1 = d0;
+                    if (!BWD) {
+                        const unsigned da = lds_addr(dtl) + k0 * 4 + lg32;
+                        d0 = raw_lds_read_at<f32x4, 0>(da);
+                        d1 = raw_lds_read_at<f32x4, 16>(da);
+                    }
                     raw_lds_wait();
                     raw_lds_use(l0); raw_lds_use(l1); raw_lds_use(u0); raw_lds_use(u1);
+                    if (!BWD) { raw_lds_use(d0); raw_lds_use(d1); }
 #pragma unroll
                     for (int rt = 0; rt < QT; ++rt) {
                         const int r = (wave * QT + rt) * 16 + lr;
@@ -490,6 +502,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                             const float e = k < r ? lor[rt] - lk : upr[rt] - uk;
                             float w = (k == r) ? (UNI ? 1.f : 2.f) : __builtin_amdgcn_exp2f(e);
                             if (UNI && (BWD ? k < r : k > r)) w = 0.f;
+                            if (!BWD) w *= i < 4 ? d0[i & 3] : d1[i & 3];
                             v[i] = (i < 4 ? cb1[rt][i & 3] : cb2[rt][i & 3]) * w;
                         }
                         af[rt] = M::pack(v);
@@ -531,10 +544,11 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
 
     // ---- epilogue.  Each wave passes its 16-row accumulator tiles through a private LDS patch so that out, out_x,
     // dx are written (and x, z, dy were read) as 16-byte vectors along headdim ----
-    // mirror: the dy rows that the D term needs lie in the operand image (transposed, unscaled; zero past the end of the
-    // sequence and of headdim): they are read from there, 16-bit units a row of the image apart, before the image becomes
-    // the staging area - and before the global requests below, which an LDS access known to the compiler would wait for
-    if (BWD && need2) {
+    // the rows that the D term needs (forward: x, mirror: dy) lie in the operand image (transposed, unscaled; zero past the
+    // end of the sequence and of headdim): they are read from there, elements a row of the image apart, before the image
+    // becomes the staging area - and before the global requests below, which an LDS access known to the compiler would
+    // wait for
+    if (BWD ? need2 : (bool)p.has_D) {
 #pragma unroll
         for (int rt = 0; rt < QT; ++rt) {
             if ((wave * QT + rt) * 16 < limit) {
@@ -544,7 +558,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                     if (FAST && id >= 16 * CPR) continue;
                     const int r = (wave * QT + rt) * 16 + min(id / CPR, 15), cc = (id % CPR) * VS;
 #pragma unroll
-                    for (int i = 0; i < VS; ++i) e2[rt][ps].v[i] = xT[xt_index<T, LDX>(cc + i, r)];
+                    for (int i = 0; i < VS; ++i) (BWD ? e2 : ex)[rt][ps].v[i] = xT[xt_index<T, LDX>(cc + i, r)];
                 }
             }
         }
