@@ -1436,6 +1436,12 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
             }
             tv += tv_head;
         };
+        // The head loop is compiled once per kind of tile: off the diagonal (KIND = -1), and on it once per wave (KIND = the
+        // wave's index, which decides for every column block whether it lies below, on or above the wave's rows), so that
+        // none of these decisions is taken, and no register moved to a common place, inside the loop.
+        auto run = [&](auto KC) __attribute__((always_inline)) {
+            constexpr int KIND = decltype(KC)::value;
+            constexpr bool DIAG = KIND >= 0;
         for (int it = 0; it < nit; ++it) {
             TSR(0);
             // with two slots nothing but step `it` is outstanding here; with more, the requests of step `it` went out before
@@ -1520,7 +1526,7 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                     }
                     col = cp * Fd;
                 };
-                if (st != tt) {
+                if constexpr (!DIAG) {
                     const bool lower = st < tt;                // forward direction below the diagonal, reverse above it
                     float E[4], rp[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -1536,8 +1542,8 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                     for (int i = 0; i < 4; ++i) { Ef[i] = __expf(cft_[i] - mf); Eb[i] = __expf(cbt_[i] - mb); }
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        if (j < wave) { sep_block(j, Ef, dts[j] * __expf(mf - cfs[j]), colF[j], rpf); }
-                        else if (j > wave) { colF[j] = 0.f; if (!UNI) sep_block(j, Eb, dts[j] * __expf(mb - cbs[j]), colB[j], rpb); }
+                        if (j < KIND) { sep_block(j, Ef, dts[j] * __expf(mf - cfs[j]), colF[j], rpf); }
+                        else if (j > KIND) { colF[j] = 0.f; if (!UNI) sep_block(j, Eb, dts[j] * __expf(mb - cbs[j]), colB[j], rpb); }
                         else {
                             // the block on the diagonal: both directions, masked element by element
                             float ca = 0.f, cb2 = 0.f;
@@ -1570,14 +1576,14 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                     float cs4[4], cs4b[4];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) cs4[j] = lanegroup_sum_mfma(colF[j]);
-                    if (st == tt) {
+                    if constexpr (DIAG) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j) cs4b[j] = lanegroup_sum_mfma(colB[j]);
                     }
                     f32x4 rs, rsb;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) rs[i] = row16_sum(rowF[i]);
-                    if (st == tt) {
+                    if constexpr (DIAG) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) rsb[i] = row16_sum(rowB[i]);
                     }
@@ -1585,14 +1591,14 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                     if (lane < 16) {
                         raw_lds_write_at<0>(pw, cs4[0]); raw_lds_write_at<64>(pw, cs4[1]);
                         raw_lds_write_at<128>(pw, cs4[2]); raw_lds_write_at<192>(pw, cs4[3]);
-                        if (st == tt) {
+                        if constexpr (DIAG) {
                             raw_lds_write_at<1024>(pw, cs4b[0]); raw_lds_write_at<1024 + 64>(pw, cs4b[1]);
                             raw_lds_write_at<1024 + 128>(pw, cs4b[2]); raw_lds_write_at<1024 + 192>(pw, cs4b[3]);
                         }
                     }
                     if (lr == 0) {
                         raw_lds_write128_at<2048>(pb + trow * 4, rs);
-                        if (st == tt) raw_lds_write128_at<2048 + 256>(pb + trow * 4, rsb);
+                        if constexpr (DIAG) raw_lds_write128_at<2048 + 256>(pb + trow * 4, rsb);
                     }
                 }
                 raw_lds_wait();
@@ -1606,6 +1612,12 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
             slot = slot + 1 == DCB_RING ? 0 : slot + 1;
             slot2 = slot2 + 1 == DCB_RING ? 0 : slot2 + 1;
         }
+        };
+        if (st != tt) run(std::integral_constant<int, -1>());
+        else if (wave == 0) run(std::integral_constant<int, 0>());
+        else if (wave == 1) run(std::integral_constant<int, 1>());
+        else if (wave == 2) run(std::integral_constant<int, 2>());
+        else run(std::integral_constant<int, 3>());
         if (pending) {
             raw_lds_barrier();
             write_out(par ^ 1);
