@@ -28,7 +28,7 @@ WORKLOAD = dict(batch=4, seqlen=2048, nheads=32, headdim=64, ngroups=1, dstate=6
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
 # size); None until measured for the kernel in question.  Source: the summaries under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "bimamba2_chunk_scan_bwd_dcb": 108.3e6, "bimamba2_chunk_scan_bwd_dc": 64.2e6, "bimamba2_chunk_state_bwd_db": 65.2e6,
+    "bimamba2_chunk_scan_bwd_dcb": 97.9e6, "bimamba2_chunk_scan_bwd_dc": 64.2e6, "bimamba2_chunk_state_bwd_db": 65.2e6,
     "bimamba2_chunk_scan_fwd": 159.8e6, "bimamba2_chunk_scan_bwd_dx": 127.7e6, "bimamba2_chunk_scan_bwd_dz": 167.9e6,
     "bimamba2_state_passing_bwd": 70.8e6, "bimamba2_bmm_chunk_bwd": 44.2e6, "bimamba2_chunk_state_fwd": 78.8e6,
     "bimamba2_chunk_scan_bwd_dstates": 77.7e6, "bimamba2_state_passing_fwd": 53.0e6, "bimamba2_chunk_cumsum_bwd": 24.3e6,
