@@ -222,6 +222,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-z", action="store_true", help="benchmark without the z gate")
+    ap.add_argument("--eager", action="store_true", help="time the eagerly launched step instead of its HIP graph replay")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the causal comparator and the layer's norm / conv legs (keeps a profile of the run to the operator)")
     args = ap.parse_args()
@@ -271,33 +272,43 @@ def main():
                                              dt_softplus=True)
         torch.autograd.grad(out, grad_inputs, dout)
 
-    for _ in range(args.warmup):
-        step()
-    t_step = timed(step, args.steps)
-    t_fwd = timed(fwd_only, args.steps)
-    # the single-direction comparator: the same kernels with the reverse direction left out, same shape, same run
-    t_causal = None
-    if not args.no_extras:
-        for _ in range(args.warmup):
-            causal_step()
-        t_causal = timed(causal_step, args.steps)
-    # the same step recorded once into a HIP graph and replayed: what the GPU needs when the host does nothing but one
-    # launch per step (the eager figures above include the host's share whenever the host is the slower side)
-    t_graph = None
-    if not args.no_extras:
+    def graphed(fn):
+        """fn recorded once into a HIP graph (torch.cuda.CUDAGraph); returns the replay callable."""
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for _ in range(3):
-                step()
+                fn()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            step()
+            fn()
+        return graph.replay
+
+    # The step is timed twice: launched eagerly through autograd (what a caller of the Python function gets; the host
+    # needs 0.18-0.35 ms for it depending on the box, which is more than the GPU needs on the slower hosts), and recorded
+    # once into a HIP graph and replayed (the same kernels on the same buffers, one launch per step).  `value` is the
+    # replayed step, i.e. the GPU's throughput, unless --eager asks for the other; both are in the output.
+    for _ in range(args.warmup):
+        step()
+    t_eager = timed(step, args.steps)
+    t_graph = None
+    if not args.eager:
+        replay = graphed(step)
         for _ in range(args.warmup):
-            graph.replay()
-        t_graph = timed(graph.replay, args.steps)
+            replay()
+        t_graph = timed(replay, args.steps)
+    t_step = t_eager if t_graph is None else t_graph
+    t_fwd = timed(fwd_only, args.steps)
+    # the single-direction comparator: the same kernels with the reverse direction left out, same shape, same run, launched
+    # the same way as the step above
+    t_causal = None
+    if not args.no_extras:
+        causal_fn = causal_step if args.eager else graphed(causal_step)
+        for _ in range(args.warmup):
+            causal_fn()
+        t_causal = timed(causal_fn, args.steps)
     tokens = w["batch"] * w["seqlen"]
     fwd_b, bwd_b = whole_op_bytes(w, e, has_z)
 
@@ -404,6 +415,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": t_step * 1e3,
+        "launch": "eager (autograd, one Python call per pass)" if t_graph is None else "HIP graph replay of the captured forward + backward step",
+        "eager": {"ms_per_step": t_eager * 1e3, "Mtokens_s": tokens / t_eager / 1e6},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -428,9 +441,6 @@ def main():
             "bidirectional_over_causal": t_step / t_causal,
             "what": "single-direction SSD (y = SS(x) + D x, z gate) forward + backward from the same kernels with the "
                     "reverse direction compiled out, same shape and dtypes"}
-        result["graph_replay"] = {
-            "ms_per_step": t_graph * 1e3, "Mtokens_s": tokens / t_graph / 1e6,
-            "what": "the same forward + backward step captured once in a torch.cuda.CUDAGraph and replayed"}
         result["gated_rmsnorm"] = rmsnorm_line(w, dtype, dev, max(10, args.steps))
         result["conv1d_silu"] = conv_line(w, dtype, dev, max(10, args.steps))
     if not args.no_cpu:
