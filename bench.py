@@ -300,7 +300,10 @@ def main():
             replay()
         t_graph = timed(replay, args.steps)
     t_step = t_eager if t_graph is None else t_graph
-    t_fwd = timed(fwd_only, args.steps)
+    fwd_fn = fwd_only if args.eager else graphed(fwd_only)
+    for _ in range(args.warmup):
+        fwd_fn()
+    t_fwd = timed(fwd_fn, args.steps)
     # the single-direction comparator: the same kernels with the reverse direction left out, same shape, same run, launched
     # the same way as the step above
     t_causal = None
