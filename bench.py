@@ -295,10 +295,15 @@ def main():
     t_eager = timed(step, args.steps)
     t_graph = None
     if not args.eager:
-        replay = graphed(step)
-        for _ in range(args.warmup):
-            replay()
-        t_graph = timed(replay, args.steps)
+        try:
+            replay = graphed(step)
+        except RuntimeError as exc:       # capture refused: say so and report the eager step
+            sys.stderr.write(f"bench.py: HIP graph capture failed ({exc}); reporting the eager step\n")
+            args.eager = True
+        else:
+            for _ in range(args.warmup):
+                replay()
+            t_graph = timed(replay, args.steps)
     t_step = t_eager if t_graph is None else t_graph
     fwd_fn = fwd_only if args.eager else graphed(fwd_only)
     for _ in range(args.warmup):
