@@ -74,6 +74,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     const int p0 = pt * PW;
     const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
     const float *csf = p.cs_f + o, *csb = p.cs_b + o, *dto = p.dt_out + o;
+    const float d_head = (p.has_D && !p.D_has_hdim) ? p.D[h] : 0.f;   // read here: in the epilogue its latency would be exposed
 
 #ifdef BM2_DBG_TIME
     long long *tlog = reinterpret_cast<long long *>(p.workspace) + ((int64_t)blockIdx.x * SCAN_WAVES + wave) * 8;
@@ -604,7 +605,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                     if (p.has_D) {
 #pragma unroll
                         for (int i = 0; i < VS; ++i)
-                            a[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : p.D[h]) * to_f(ex[B_][ps].v[i]);
+                            a[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : d_head) * to_f(ex[B_][ps].v[i]);
                     }
                     if (p.has_z) {
                         if (p.out_x) store_vec(reinterpret_cast<T *>(p.out_x) + orow, ovec, ncol, a);
@@ -620,7 +621,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                     if (p.has_D) {
 #pragma unroll
                         for (int i = 0; i < VS; ++i) {
-                            dxv[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : p.D[h]) * to_f(e2[B_][ps].v[i]);
+                            dxv[i] += (p.D_has_hdim ? (i < ncol ? p.D[h * P + col + i] : 0.f) : d_head) * to_f(e2[B_][ps].v[i]);
                             dsum[i] += to_f(e2[B_][ps].v[i]) * to_f(ex[B_][ps].v[i]);
                         }
                     }
