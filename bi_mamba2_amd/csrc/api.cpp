@@ -1,4 +1,3 @@
-#include <cstdlib>
 // C ABI of libbimamba2_hip.so: argument checks, workspace carving and the forward / backward pipelines.
 #include <stdio.h>
 #include <string.h>
