@@ -151,3 +151,24 @@ def test_causal_flag_and_second_direction_buffers():
     lib = _lib.load()
     p = _params(causal=1, final_b=256, workspace=256, workspace_bytes=1 << 40)
     assert lib.bimamba2_fwd(ctypes.byref(p)) == -1
+
+
+def test_state_copies_are_for_the_fast_path_only():
+    """bimamba2_state_copies() says where the kernels can keep the entering states in 16-bit copies; the workspace of the
+    composites holds them there, and a stage that does not know them refuses them (before any launch)."""
+    lib = _lib.load()
+    fast = dict(batch=2, seqlen=512, nheads=8, headdim=64, ngroups=1, dstate=64, chunk_size=256,
+                x_sb=512 * 8 * 64, x_sl=8 * 64, x_sh=64, B_sb=512 * 64, B_sl=64, B_sg=64, C_sb=512 * 64, C_sl=64, C_sg=64,
+                x=256, Bm=256, Cm=256)
+    assert lib.bimamba2_state_copies(ctypes.byref(_params(**fast))) == 1
+    assert lib.bimamba2_state_copies(ctypes.byref(_params(**dict(fast, dtype=_lib.F32)))) == 0
+    assert lib.bimamba2_state_copies(ctypes.byref(_params(**dict(fast, dstate=128, B_sl=128, C_sl=128)))) == 0
+    assert lib.bimamba2_state_copies(ctypes.byref(_params())) == 0
+    # the copies are part of the forward workspace where they are used, and a caller who brings them saves that much
+    stn = 2 * 2 * 8 * 64 * 64
+    own = lib.bimamba2_workspace_bytes(ctypes.byref(_params(**fast)), 0)
+    brought = lib.bimamba2_workspace_bytes(ctypes.byref(_params(**dict(fast, states16_f=256, states16_b=512))), 0)
+    assert own - brought == 2 * stn * 2
+    # the generic state passing (float32 problem) does not know the copies
+    p = _params(cs_f=256, cs_b=256, states_f=256, states_b=256, states16_f=256, states16_b=256, dtype=_lib.F32)
+    assert lib.bimamba2_state_passing_fwd(ctypes.byref(p)) == -2
