@@ -119,11 +119,14 @@ __device__ __forceinline__ float dsilu_f(float z) {
 }
 
 // grid (row blocks, groups); wave w of workgroup bx handles rows bx*4 + w, + 4*gridDim.x, ...
-template <typename T, int NCH, bool HAS_BIAS>
-__global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimamba2_norm_params p, bool vec, bool wvec, float *part_w,
+// FULL: the group is exactly NCH * 512 columns wide and every access is a 16-byte one (the host checked it): no lane is
+// ever out of range, and with the conditions gone the loads of all chunks of a row go out before the first is used.
+template <typename T, int NCH, bool HAS_BIAS, bool FULL>
+__global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimamba2_norm_params p, bool vec_, bool wvec_, float *part_w,
                                                                      float *part_b) {
+    const bool vec = FULL || vec_, wvec = FULL || wvec_;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int ngroups = p.cols / p.group_size, gs = p.group_size;
+    const int ngroups = p.cols / p.group_size, gs = FULL ? NCH * 512 : p.group_size;
     const int g = blockIdx.y;
     const float *w = p.weight + g * gs, *bias = HAS_BIAS ? p.bias + g * gs : nullptr;
     const bool gate_first = p.has_z && !p.norm_before_gate, gate_last = p.has_z && p.norm_before_gate;
@@ -149,11 +152,11 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
         float xh[HOLD ? NCH : 1][8], wd[HOLD ? NCH : 1][8], sl[HOLD ? NCH : 1][8], g2[HOLD ? NCH : 1][8];
         auto element = [&](int k, int c, bool first, float (&xhat)[8], float (&wdy)[8], float (&slv)[8], float (&g2v)[8]) {
             float xv[8], dy[8], zv[8], wv[8], bv[8], dzv[8];
-            load8(x + c, vec, gs - c, xv);
-            load8(dout + c, vec, gs - c, dy);
-            load8(w + c, wvec, gs - c, wv);
-            if (HAS_BIAS && first) load8(bias + c, wvec, gs - c, bv);
-            if (p.has_z) load8(z + c, vec, gs - c, zv);
+            load8(x + c, vec, FULL ? 8 : gs - c, xv);
+            load8(dout + c, vec, FULL ? 8 : gs - c, dy);
+            load8(w + c, wvec, FULL ? 8 : gs - c, wv);
+            if (HAS_BIAS && first) load8(bias + c, wvec, FULL ? 8 : gs - c, bv);
+            if (p.has_z) load8(z + c, vec, FULL ? 8 : gs - c, zv);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 float sg = 0.f, si = 1.f, ds = 0.f;
@@ -175,14 +178,14 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
                     if (HAS_BIAS) db[k][i] += dy[i];
                 }
             }
-            if (gate_last && first) store8(dz + c, vec, gs - c, dzv);
+            if (gate_last && first) store8(dz + c, vec, FULL ? 8 : gs - c, dzv);
         };
         // pass 1: c1 = mean(xhat * wdy), weight / bias gradients, and dz when the gate comes last
         float c1 = 0.f;
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
             const int c = (k * 64 + lane) * 8;
-            if (c >= gs) continue;
+            if (!FULL && c >= gs) continue;
             float xhat[8], wdy[8], slv[8], g2v[8];
             element(k, c, true, xhat, wdy, slv, g2v);
 #pragma unroll
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
             const int c = (k * 64 + lane) * 8;
-            if (c >= gs) continue;
+            if (!FULL && c >= gs) continue;
             float xhat[8], wdy[8], slv[8], g2v[8], dxv[8], dzv[8];
             if (HOLD) {
 #pragma unroll
@@ -210,8 +213,8 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
                 dxv[i] = gate_first ? dxg * slv[i] : dxg;
                 dzv[i] = dxg * g2v[i];
             }
-            store8(dx + c, vec, gs - c, dxv);
-            if (gate_first) store8(dz + c, vec, gs - c, dzv);
+            store8(dx + c, vec, FULL ? 8 : gs - c, dxv);
+            if (gate_first) store8(dz + c, vec, FULL ? 8 : gs - c, dzv);
         }
     }
     if constexpr (NCH <= 8) {
@@ -231,11 +234,11 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
 #pragma unroll
                 for (int k = 0; k < NCH; ++k) {
                     const int c = (k * 64 + lane) * 8;
-                    if (c >= gs) continue;
+                    if (!FULL && c >= gs) continue;
                     float v[8];
 #pragma unroll
                     for (int i = 0; i < 8; ++i) v[i] = (pass ? db[HAS_BIAS ? k : 0][i] : dw[k][i]) + red[0][c + i] + red[1][c + i] + red[2][c + i];
-                    store8((pass ? part_b : part_w) + prow + c, false, gs - c, v);
+                    store8((pass ? part_b : part_w) + prow + c, false, FULL ? 8 : gs - c, v);
                 }
             }
         }
@@ -245,9 +248,9 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
             const int c = (k * 64 + lane) * 8;
-            if (c >= gs) continue;
-            store8(part_w + prow + c, false, gs - c, dw[k]);
-            if (HAS_BIAS) store8(part_b + prow + c, false, gs - c, db[k]);
+            if (!FULL && c >= gs) continue;
+            store8(part_w + prow + c, false, FULL ? 8 : gs - c, dw[k]);
+            if (HAS_BIAS) store8(part_b + prow + c, false, FULL ? 8 : gs - c, db[k]);
         }
     }
 }
@@ -316,8 +319,14 @@ static int launch_norm_nch(const bimamba2_norm_params *p, bool bwd) {
     const int npr = norm_partial_rows(p);
     float *part_b = p->has_bias ? part_w + (size_t)npr * p->cols : nullptr;
     const dim3 grid(nb, p->cols / p->group_size);
-    if (p->has_bias) hipLaunchKernelGGL((rmsnorm_gated_bwd_kernel<T, NCH, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
-    else hipLaunchKernelGGL((rmsnorm_gated_bwd_kernel<T, NCH, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+    const bool full = vec && wvec && p->group_size == NCH * 512 && NCH <= 4;
+    if (full) {
+        if (p->has_bias) hipLaunchKernelGGL((rmsnorm_gated_bwd_kernel<T, NCH, true, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+        else hipLaunchKernelGGL((rmsnorm_gated_bwd_kernel<T, NCH, false, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+    } else {
+        if (p->has_bias) hipLaunchKernelGGL((rmsnorm_gated_bwd_kernel<T, NCH, true, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+        else hipLaunchKernelGGL((rmsnorm_gated_bwd_kernel<T, NCH, false, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+    }
     int rc = check_launch();
     if (rc) return rc;
     hipLaunchKernelGGL(colsum_kernel, dim3((p->cols + 15) / 16, p->has_bias ? 2 : 1), dim3(NTHREADS), 0, stream_of(p), part_w, p->dweight,
