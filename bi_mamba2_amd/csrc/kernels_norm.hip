@@ -52,10 +52,13 @@ template <typename T> __device__ __forceinline__ void store8(T *ptr, bool vec, i
     }
 }
 
-template <typename T, int NCH>
-__global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_fwd_kernel(const bimamba2_norm_params p, bool vec, bool wvec) {
+// FULL: the group is exactly NCH * 512 columns wide and every access is a 16-byte one (the host checked it); the weights are
+// then requested together with the row, in front of the reduction.
+template <typename T, int NCH, bool FULL>
+__global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_fwd_kernel(const bimamba2_norm_params p, bool vec_, bool wvec_) {
+    const bool vec = FULL || vec_, wvec = FULL || wvec_;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int ngroups = p.cols / p.group_size, gs = p.group_size;
+    const int ngroups = p.cols / p.group_size, gs = FULL ? NCH * 512 : p.group_size;
     const int64_t item = (int64_t)blockIdx.x * 4 + wave;
     if (item >= (int64_t)p.rows * ngroups) return;
     const int g = (int)(item % ngroups);
@@ -72,16 +75,21 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_fwd_kernel(const bimam
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
         const int c = (k * 64 + lane) * 8;
-        load8(x + c, vec, gs - c, xv[k]);
+        load8(x + c, vec, FULL ? 8 : gs - c, xv[k]);
         if (p.has_z) {
             float zv[8];
-            load8(z + c, vec, gs - c, zv);
+            load8(z + c, vec, FULL ? 8 : gs - c, zv);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 if (gate_first) xv[k][i] *= silu_f(zv[i]);
                 else zk[k][i] = from_f<T>(zv[i]);      // exact: zv came from a T
             }
         }
+    }
+    float wk[FULL ? NCH : 1][8];
+    if (FULL) {
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) load8(w + (k * 64 + lane) * 8, true, 8, wk[FULL ? k : 0]);
     }
 #pragma unroll
     for (int k = 0; k < NCH; ++k)
@@ -93,14 +101,19 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_fwd_kernel(const bimam
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
         const int c = (k * 64 + lane) * 8;
-        if (c >= gs) continue;
+        if (!FULL && c >= gs) continue;
         float wv[8], yv[8];
-        load8(w + c, wvec, gs - c, wv);
+        if (FULL) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) wv[i] = wk[FULL ? k : 0][i];
+        } else {
+            load8(w + c, wvec, gs - c, wv);
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) yv[i] = xv[k][i] * rstd * wv[i];
         if (bias) {
             float bv[8];
-            load8(bias + c, wvec, gs - c, bv);
+            load8(bias + c, wvec, FULL ? 8 : gs - c, bv);
 #pragma unroll
             for (int i = 0; i < 8; ++i) yv[i] += bv[i];
         }
@@ -108,7 +121,7 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_fwd_kernel(const bimam
 #pragma unroll
             for (int i = 0; i < 8; ++i) yv[i] *= silu_f(to_f(zk[k][i]));
         }
-        store8(out + c, vec, gs - c, yv);
+        store8(out + c, vec, FULL ? 8 : gs - c, yv);
     }
 }
 
@@ -311,7 +324,10 @@ static int launch_norm_nch(const bimamba2_norm_params *p, bool bwd) {
     const bool wvec = p->group_size % 4 == 0 && al(p->weight) && (!p->has_bias || al(p->bias));
     if (!bwd) {
         const int64_t items = (int64_t)p->rows * (p->cols / p->group_size);
-        hipLaunchKernelGGL((rmsnorm_gated_fwd_kernel<T, NCH>), dim3((unsigned)((items + 3) / 4)), dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec);
+        if (vec && wvec && p->group_size == NCH * 512 && NCH <= 4)
+            hipLaunchKernelGGL((rmsnorm_gated_fwd_kernel<T, NCH, true>), dim3((unsigned)((items + 3) / 4)), dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec);
+        else
+            hipLaunchKernelGGL((rmsnorm_gated_fwd_kernel<T, NCH, false>), dim3((unsigned)((items + 3) / 4)), dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec);
         return check_launch();
     }
     const int nb = norm_row_blocks(p);
