@@ -109,8 +109,10 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dz_kernel(const bimamba2_params 
         const bool vec = (c0 + VS <= P) && aligned16(zp, 0) && aligned16(dp, 0) && aligned16(ox + o, 0);
         float zv[VS], dv[VS], ov[VS];
         if (vec) {
-            Vec16<T> a = *reinterpret_cast<const Vec16<T> *>(zp), d = *reinterpret_cast<const Vec16<T> *>(dp),
-                     e = *reinterpret_cast<const Vec16<T> *>(ox + o);
+            // all three are read for the last time in this pass
+            const Vec16<T> a = __builtin_bit_cast(Vec16<T>, __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(zp))),
+                           d = __builtin_bit_cast(Vec16<T>, __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(dp))),
+                           e = __builtin_bit_cast(Vec16<T>, __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(ox + o)));
 #pragma unroll
             for (int i = 0; i < VS; ++i) { zv[i] = to_f(a.v[i]); dv[i] = to_f(d.v[i]); ov[i] = to_f(e.v[i]); }
         } else {
@@ -128,7 +130,8 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dz_kernel(const bimamba2_params 
             r2.v[i] = from_f<T>(dv[i] * zv[i] * sg);
         }
         if (vec) {
-            *reinterpret_cast<Vec16<T> *>(dz + o) = r1;
+            // dz is not read again inside the pass, dout_x by four kernels: the first goes past the caches
+            __builtin_nontemporal_store(__builtin_bit_cast(f32x4, r1), reinterpret_cast<f32x4 *>(dz + o));
             *reinterpret_cast<Vec16<T> *>(dox + o) = r2;
         } else {
 #pragma unroll

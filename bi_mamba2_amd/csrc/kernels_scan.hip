@@ -318,12 +318,14 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             for (int i = 0; i < VS; ++i) v.v[i] = i < ncol ? ptr[i] : from_f<T>(0.f);
         }
     };
-    auto store_vec = [&](T *ptr, bool vec, int ncol, const float (&v)[VS]) {
+    // past_caches: a result that no kernel of the pass reads again (out, dx) leaves the caches to what is read again
+    auto store_vec = [&](T *ptr, bool vec, int ncol, const float (&v)[VS], bool past_caches = false) {
         if (FAST || (vec && ncol >= VS)) {
             Vec16<T> ov;
 #pragma unroll
             for (int i = 0; i < VS; ++i) ov.v[i] = from_f<T>(v[i]);
-            *reinterpret_cast<Vec16<T> *>(ptr) = ov;
+            if (past_caches) __builtin_nontemporal_store(__builtin_bit_cast(f32x4, ov), reinterpret_cast<f32x4 *>(ptr));
+            else *reinterpret_cast<Vec16<T> *>(ptr) = ov;
         } else {
 #pragma unroll
             for (int i = 0; i < VS; ++i)
@@ -612,7 +614,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
 #pragma unroll
                         for (int i = 0; i < VS; ++i) a[i] *= silu_f(to_f(e2[B_][ps].v[i]));
                     }
-                    store_vec(reinterpret_cast<T *>(p.out) + orow, ovec, ncol, a);
+                    store_vec(reinterpret_cast<T *>(p.out) + orow, ovec, ncol, a, true);
                 } else {
                     const float dtr = dto[r];
                     float dxv[VS];
@@ -625,7 +627,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                             dsum[i] += to_f(e2[B_][ps].v[i]) * to_f(ex[B_][ps].v[i]);
                         }
                     }
-                    store_vec(reinterpret_cast<T *>(p.dx) + orow, ovec, ncol, dxv);
+                    store_vec(reinterpret_cast<T *>(p.dx) + orow, ovec, ncol, dxv, true);
                 }
             }
             if (BWD) {
