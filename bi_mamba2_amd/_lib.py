@@ -38,7 +38,7 @@ class Params(ctypes.Structure):
 
 
 ENTRY_POINTS = (
-    "bimamba2_fwd", "bimamba2_bwd",
+    "bimamba2_fwd", "bimamba2_bwd", "bimamba2_fwd_static",
     "bimamba2_chunk_cumsum_fwd", "bimamba2_bmm_chunk_fwd", "bimamba2_chunk_state_fwd",
     "bimamba2_state_passing_fwd", "bimamba2_chunk_scan_fwd",
     "bimamba2_chunk_scan_bwd_dz", "bimamba2_chunk_scan_bwd_dstates", "bimamba2_state_passing_bwd",
@@ -130,5 +130,5 @@ def call(name, params):
     rc = getattr(lib, name)(ctypes.byref(params))
     if rc != 0:
         msg = lib.bimamba2_strerror(rc).decode()
-        exc = ValueError if rc in (-1, -2) else RuntimeError
+        exc = ValueError if rc in (-1, -2, -5) else RuntimeError
         raise exc(f"{name}: {msg} (code {rc})")

@@ -3,6 +3,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 
 #include "../../include/bimamba2.h"
 #include "launch.hpp"
@@ -110,6 +111,27 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     return (cv.off + 255) & ~size_t(255);
 }
 
+// Device memory that lives as long as the process: the workspace of bimamba2_fwd_static.  Every GPU the library runs on
+// holds its own copy at its own address; in host code the array's name is not a device address, so the address is asked
+// for once per device (hipGetSymbolAddress, with that device current) and kept.
+static __device__ __align__(256) unsigned char scratch[BIMAMBA2_STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<void *> scratch_of_device[MAX_DEVICES];
+
+int static_scratch(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return BIMAMBA2_ELAUNCH;
+    void *ptr = scratch_of_device[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        // two host threads may both get here: they are given the same address
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return BIMAMBA2_ELAUNCH;
+        scratch_of_device[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return BIMAMBA2_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -122,6 +144,7 @@ const char *bimamba2_strerror(int code) {
             return "unsupported problem (need 32 <= chunk_size <= 256, headdim <= 128, dstate <= 256, dtype f32/bf16/f16)";
         case BIMAMBA2_EWORKSPACE: return "workspace missing or too small";
         case BIMAMBA2_ELAUNCH: return "HIP kernel launch failed";
+        case BIMAMBA2_ESCRATCH: return "the problem needs more intermediate memory than the static scratch buffer holds";
         default: return "unknown error";
     }
 }
@@ -297,6 +320,22 @@ int bimamba2_fwd(const bimamba2_params *p) {
     if (scan_recomputes_cb(&q, false)) q.CB = nullptr;
     TRY(bimamba2_chunk_scan_fwd(&q));
     return BIMAMBA2_OK;
+}
+
+int bimamba2_fwd_static(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    bimamba2_params q = *p;
+    q.workspace = nullptr;
+    q.workspace_bytes = 0;
+    {
+        bimamba2_params sized = q;
+        if (carve(&sized, 0, nullptr) > BIMAMBA2_STATIC_SCRATCH_BYTES) return BIMAMBA2_ESCRATCH;
+    }
+    // nothing in the forward pipeline accumulates into its intermediates: every one is written in full before it is
+    // read, so what the last call left in the buffer does not matter
+    TRY(static_scratch(&q.workspace));
+    q.workspace_bytes = BIMAMBA2_STATIC_SCRATCH_BYTES;
+    return bimamba2_fwd(&q);
 }
 
 int bimamba2_bwd(const bimamba2_params *p) {

@@ -39,7 +39,8 @@ enum {
     BIMAMBA2_EINVAL = -1,      /* null pointer / inconsistent dimensions */
     BIMAMBA2_EUNSUPPORTED = -2,/* shape or dtype outside what the kernels are built for */
     BIMAMBA2_EWORKSPACE = -3,  /* workspace missing or too small */
-    BIMAMBA2_ELAUNCH = -4      /* HIP reported a launch error */
+    BIMAMBA2_ELAUNCH = -4,     /* HIP reported a launch error */
+    BIMAMBA2_ESCRATCH = -5     /* bimamba2_fwd_static: the problem needs more than BIMAMBA2_STATIC_SCRATCH_BYTES */
 };
 
 /* limits of the compiled kernels */
@@ -164,6 +165,17 @@ int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which);
  * caller can keep them for the backward pass (CB and CBT are only computed when given or when the scan kernel
  * reads them). */
 int bimamba2_fwd(const bimamba2_params *p);
+
+/* bimamba2_fwd for callers that cannot allocate device memory or bring a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its wrappers allocate every
+ * intermediate with torch.empty).  Same arguments, same kernels and bit for bit the same results as bimamba2_fwd, but
+ * `workspace` / `workspace_bytes` are ignored: the intermediates that the caller does not bring live in a buffer of
+ * BIMAMBA2_STATIC_SCRATCH_BYTES that is part of the library's device image (each GPU the library runs on holds one until
+ * the process ends).  Calls no hipMalloc / hipFree or any other allocating routine.  Returns BIMAMBA2_ESCRATCH when
+ * bimamba2_workspace_bytes(p, 0) exceeds the buffer.  All calls on one GPU share that GPU's buffer: calls that overlap
+ * on one GPU (two streams, two host threads) race; calls on one stream, one after the other, are safe. */
+#define BIMAMBA2_STATIC_SCRATCH_BYTES (64u << 20)
+int bimamba2_fwd_static(const bimamba2_params *p);
 
 /* Whole backward; replaces _mamba_chunk_scan_combined_bwd (src/ssd/bi/ssd_combined.py:334-475).
  * Needs: the forward inputs, dout, out_x (pre-gate output, when has_z), dx ddt dA dB dC [dD dz ddt_bias],

@@ -48,7 +48,11 @@ def test_argument_checks_return_error_codes():
     assert lib.bimamba2_fwd(ctypes.byref(_params(nheads=3))) == -1              # heads not divisible by groups
     assert lib.bimamba2_fwd(ctypes.byref(_params(dtype=7))) == -2
     assert lib.bimamba2_bwd(ctypes.byref(_params(fwd_saved=1, workspace=1, workspace_bytes=1 << 40))) == -1
-    for code in (0, -1, -2, -3, -4, -99):
+    # the forward without a workspace refuses what its built-in buffer cannot hold, before any GPU call
+    big = _params(batch=16, seqlen=65536, nheads=64, headdim=64, ngroups=1, dstate=64, chunk_size=256)
+    assert lib.bimamba2_fwd_static(ctypes.byref(big)) == -5
+    assert lib.bimamba2_fwd_static(None) == -1
+    for code in (0, -1, -2, -3, -4, -5, -99):
         assert lib.bimamba2_strerror(code)
     with pytest.raises(ValueError):
         _lib.call("bimamba2_chunk_cumsum_fwd", _params())
