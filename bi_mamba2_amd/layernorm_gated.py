@@ -123,6 +123,9 @@ class LayerNormFn(torch.autograd.Function):
                 dz.reshape(ctx.shape).to(ctx.zdtype) if dz is not None else None, None, None, None, None)
 
 
+MAX_GROUP = 8192      # columns per normalisation group (bimamba2_rmsnorm_gated_fwd / _bwd refuse more)
+
+
 def rmsnorm_fn(x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True):
     return LayerNormFn.apply(x, weight, bias, z, eps, group_size, norm_before_gate, True)
 
@@ -132,6 +135,10 @@ class RMSNorm(torch.nn.Module):
 
     def __init__(self, hidden_size, eps=1e-5, group_size=None, norm_before_gate=True, device=None, dtype=None):
         super().__init__()
+        # the kernels hold a group of at most MAX_GROUP columns per wave (the reference's Triton kernel: 64 KB per row);
+        # refuse a wider one where the module is built rather than at the first forward
+        if (group_size or hidden_size) > MAX_GROUP:
+            raise ValueError(f"RMSNorm: groups of {group_size or hidden_size} columns exceed the {MAX_GROUP} the kernels support")
         self.eps = eps
         self.weight = torch.nn.Parameter(torch.empty(hidden_size, device=device, dtype=dtype))
         self.register_parameter("bias", None)

@@ -57,6 +57,7 @@ class _Call:
         p.dt_softplus = int(bool(dt_softplus))
         p.dt_min, p.dt_max = float(dt_limit[0]), float(dt_limit[1])
         self.p, self.keep, self.device, self.dtype, self.dt_dtype = p, [], device, dtype, dt_dtype
+        self.params = []       # float32 copies of A, D, dt_bias that the parameter block points at
         self.nchunks = (seqlen + chunk_size - 1) // chunk_size
 
     # ---- raw pointer fields -------------------------------------------------------------------------
@@ -113,21 +114,26 @@ class _Call:
         self.p.dt_sb, self.p.dt_sl, self.p.dt_sh = dt.stride()
         return dt
 
+    def _param(self, field, t):
+        t = self.put(field, _f32c(t))
+        self.params.append(t)
+        return t
+
     def set_A(self, A):
-        return self.put("A", _f32c(A))
+        return self._param("A", A)
 
     def set_D(self, D):
         if D is None:
             return None
         self.p.has_D = 1
         self.p.D_has_hdim = int(D.dim() == 2)
-        return self.put("D", _f32c(D))
+        return self._param("D", D)
 
     def set_dt_bias(self, dt_bias):
         if dt_bias is None:
             return None
         self.p.has_dt_bias = 1
-        return self.put("dt_bias", _f32c(dt_bias))
+        return self._param("dt_bias", dt_bias)
 
     def _workspace_bytes(self, is_bwd):
         return int(_lib.load().bimamba2_workspace_bytes(self.p, int(is_bwd)))
@@ -164,14 +170,16 @@ class _Call:
 
     # ---- reuse of the input half of a call (the autograd function builds it once for forward and backward) ----
     def snapshot(self):
-        """The parameter block as bytes plus the small converted tensors it points at (A, D, dt_bias copies)."""
-        return bytes(self.p), [t for t in self.keep if t.numel() <= 1 << 16]
+        """The parameter block as bytes plus the converted tensors it points at (the float32 copies of A, D, dt_bias,
+        whatever their size): a call rebuilt from the snapshot uses their pointers again."""
+        return bytes(self.p), list(self.params)
 
     @classmethod
     def from_snapshot(cls, snap, x, nchunks):
         self = cls.__new__(cls)
         self.p = Params.from_buffer_copy(snap[0])
         self.keep = list(snap[1])
+        self.params = list(snap[1])
         self.device, self.dtype, self.dt_dtype = x.device, x.dtype, None
         self.nchunks = nchunks
         return self
@@ -420,8 +428,11 @@ def _bmm_chunk_bwd(B, C, dCB, dBs, dCs):
     (slices, batch, seqlen, ngroups, dstate) partial sums of _chunk_state_bwd_db / _chunk_scan_bwd_dC."""
     batch, seqlen, ngroups, dstate = B.shape
     chunk_size = dCB.shape[-1]
-    # nheads is only used to tell the kernel how many slices to add up
-    c = _Call(batch, seqlen, ngroups * 4 * dBs.shape[0], 1, ngroups, dstate, chunk_size, B.dtype, B.device)
+    # nheads is only used to tell the kernel how many slices to add up: _slices(nheads, ngroups) must give them back
+    assert dCs.shape[0] == dBs.shape[0]
+    nheads = ngroups * 8 * dBs.shape[0]
+    assert _slices(nheads, ngroups) == dBs.shape[0]
+    c = _Call(batch, seqlen, nheads, 1, ngroups, dstate, chunk_size, B.dtype, B.device)
     c.set_B(B); c.set_C(C)
     c.put("dCB", dCB, torch.float32); c.put("dCBT", dCB.transpose(-1, -2).contiguous(), torch.float32)
     c.put("dBs", dBs, torch.float32); c.put("dCs", dCs, torch.float32)
@@ -429,6 +440,32 @@ def _bmm_chunk_bwd(B, C, dCB, dBs, dCs):
     dC = torch.zeros(B.shape, device=B.device, dtype=B.dtype); c.put("dC", dC)
     c.run("bimamba2_bmm_chunk_bwd")
     return dB, dC
+
+
+def _chunk_cumsum_bwd(da_intra, u_f, u_b, v_f, v_b, ddA_chunk_f, ddA_chunk_b, ddt_direct, dt, A, dt_bias=None,
+                      dt_softplus=False, dt_limit=(0.0, _INF)):
+    """Assembles d(dt * A) from its pieces and takes it through the dt transform: the reference's host-side scans
+    (src/ssd/bi/ssd_combined.py:456-466) and its _chunk_cumsum_bwd (src/ssd/bi/ssd_chunk_state.py:727-761) in one kernel.
+    da_intra: per-tile vectors of _chunk_scan_bwd_dcb; u_*: of _chunk_scan_bwd_dC; v_*: of _chunk_state_bwd_db;
+    ddA_chunk_*: (batch, nheads, nchunks) of _state_passing_bwd; ddt_direct: of _chunk_scan_chunk_state_bwd_dx; dt: the raw
+    (batch, seqlen, nheads) input.  -> ddt (like dt), dA (nheads,), ddt_bias (nheads,) or None."""
+    batch, seqlen, nheads = dt.shape
+    _, _, nchunks, chunk_size = ddt_direct.shape
+    assert u_f.shape == ddt_direct.shape and v_f.shape == ddt_direct.shape
+    assert ddA_chunk_f.shape == (batch, nheads, nchunks) and ddA_chunk_b.shape == ddA_chunk_f.shape
+    # headdim = dstate = 1: one partial sum per chunk in ddA_chunk_*
+    c = _Call(batch, seqlen, nheads, 1, 1, 1, chunk_size, torch.float32, dt.device, dt.dtype, dt_softplus, dt_limit)
+    c.set_dt(dt); c.set_A(A); c.set_dt_bias(dt_bias)
+    for field, t in (("da_intra", da_intra), ("u_f", u_f), ("u_b", u_b), ("v_f", v_f), ("v_b", v_b),
+                     ("ddA_chunk_f", ddA_chunk_f.reshape(batch, nheads, nchunks, 1)),
+                     ("ddA_chunk_b", ddA_chunk_b.reshape(batch, nheads, nchunks, 1)), ("ddt_direct", ddt_direct)):
+        c.put(field, t.contiguous(), torch.float32)
+    ddt = c.new("ddt", dt.shape, dt.dtype)
+    dA = c.new("dA", (nheads,))
+    ddt_bias = c.new("ddt_bias", (nheads,)) if dt_bias is not None else None
+    c.new("red", (2 * batch * nchunks * nheads,))
+    c.run("bimamba2_chunk_cumsum_bwd")
+    return ddt, dA, ddt_bias
 
 
 # =============================================================================================================
@@ -582,6 +619,10 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
         sshape = (batch, nheads, headdim, B.shape[3])
         dinit = tuple(c.new(f, sshape) if t is not None else None
                       for f, t in zip(("dinitial_f", "dinitial_b"), initial_states))
+    if blob is not None and x.element_size() == 2 and (dout.data_ptr() % 16 or any(s % 8 for s in dout.stride()[:3])):
+        # the forward kept the 16-bit copies of the entering states only, which the kernels for aligned operands know:
+        # a gradient view that breaks their alignment (e.g. a slice of a wider tensor at an odd offset) is copied
+        dout = dout.contiguous()
     c.set_dout(dout)
     if blob is not None:
         _point_into(c, blob, snap[2], snap[3])

@@ -49,7 +49,11 @@ enum {
 #define BIMAMBA2_MAX_HEADDIM 128
 #define BIMAMBA2_MAX_DSTATE 256
 
-#define BIMAMBA2_SEQ_CUT (-64.0f)   /* added to the decay exponent across a change of seq_idx: e^-64 = 1.6e-28 */
+/* Added to the decay exponent across a change of seq_idx: every factor across a boundary carries e^-20 = 2e-9, below
+ * float32 resolution next to the terms it is added to.  The cumulative sums of a chunk grow by this much per boundary
+ * inside it, and their float32 resolution with them: relative accuracy of the in-sequence decays about 1.2e-6 per boundary
+ * in the chunk (the float32 contract of 1e-4 holds up to about 40 boundaries per chunk). */
+#define BIMAMBA2_SEQ_CUT (-20.0f)
 
 typedef struct bimamba2_params {
     /* problem */

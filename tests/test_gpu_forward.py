@@ -58,8 +58,9 @@ def test_forward_stages(ops, shape, dtype):
     out, out_x = ops._chunk_scan_fwd(CB, d["x"], dt_out, csf, csb, d["C"], pf, pb, D=d["D"], z=d["z"])
     out_ref, outx_ref = O.stage_chunk_scan(CB.double().cpu(), r["x"], dt64, csf64, csb64, r["C"], pf.double().cpu(),
                                            pb.double().cpu(), r["D"], r["z"])
-    assert_close(out_x, outx_ref, dtype, "out_x")
-    assert_close(out, out_ref, dtype, "out")
+    big = N > 64      # dot products over 128 state columns of 16-bit operands: outputs of RMS ~ 10
+    assert_close(out_x, outx_ref, dtype, "out_x", scaled=big)
+    assert_close(out, out_ref, dtype, "out", scaled=big)
 
 
 # the reference's own end-to-end forward grid (tests/test_fwd_scan.py:8-16 there): z = None, D = None
@@ -100,7 +101,7 @@ def test_forward_end_to_end(ops, case):
     ref = O.bimamba2_sequential(r["x"], r["dt"], r["A"], r["B"], r["C"], D=r["D"], z=r["z"], dt_bias=r["dt_bias"],
                                 dt_softplus=sp, dt_limit=lim)
     assert out.dtype == dtype and ff.dtype == torch.float32
-    assert_close(out, ref[0], dtype, "out")
+    assert_close(out, ref[0], dtype, "out", scaled=not sp)      # raw dt without softplus: outputs far from unit scale
     assert_close(ff, ref[2], dtype, "final_f")
     assert_close(fb, ref[3], dtype, "final_b")
 
@@ -142,12 +143,12 @@ def test_stages_rebuild_cb_when_it_is_not_given(ops, dtype):
     assert_close(dx2, dx1.double().cpu(), dtype, "dx without CB")
     # positions past the end of the sequence are not written by either path
     valid = (torch.arange(ddt1.shape[2])[:, None] * Q + torch.arange(Q)[None, :] < L).to(ddt1.device)
-    assert_close(torch.where(valid, ddt2, 0.0), torch.where(valid, ddt1, 0.0).double().cpu(), dtype, "ddt_direct without CB")
-    assert_close(dD2, dD1.double().cpu(), dtype, "dD without CB")
+    assert_close(torch.where(valid, ddt2, 0.0), torch.where(valid, ddt1, 0.0).double().cpu(), dtype, "ddt_direct without CB", scaled=True)
+    assert_close(dD2, dD1.double().cpu(), dtype, "dD without CB", scaled=True)
     dCB1, da1 = ops._chunk_scan_bwd_dcb(d["x"], dt_out, csf, csb, dout, CB, ngroups=G)
     dCB2, da2 = ops._chunk_scan_bwd_dcb(d["x"], dt_out, csf, csb, dout, None, ngroups=G, B=d["B"], C=d["C"])
-    assert_close(dCB2, dCB1.double().cpu(), dtype, "dCB without CB")
-    assert_close(da2, da1.double().cpu(), dtype, "da_intra without CB")
+    assert_close(dCB2, dCB1.double().cpu(), dtype, "dCB without CB", scaled=True)
+    assert_close(da2, da1.double().cpu(), dtype, "da_intra without CB", scaled=True)
     # shapes whose kernels cannot rebuild CB refuse a missing CB instead of reading a null pointer
     with pytest.raises(ValueError):
         ops._chunk_scan_fwd(None, d["x"].float(), dt_out, csf, csb, d["C"].float(), pf, pb, B=d["B"].float())

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import bimamba2_oracle as O
-from tests.helpers import assert_close, make_case, to64, to_dev
+from tests.helpers import assert_close, is_reduced, make_case, to64, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -53,14 +53,16 @@ def test_initial_states_and_final_state_gradients(ops, case, keep, monkeypatch):
     ro, _, rff, rfb = O.bimamba2_sequential(r["x"], r["dt"], r["A"], r["B"], r["C"], D=r["D"], z=r["z"], dt_bias=r["dt_bias"],
                                             dt_softplus=True, initial_states_f=ri["f"], initial_states_b=ri["b"])
     torch.autograd.backward([ro, rff, rfb], [dout.double(), cot["f"].double(), cot["b"].double()])
-    assert_close(out, ro, dtype, "out")
-    assert_close(ff, rff, dtype, "final_f")
-    assert_close(fb, rfb, dtype, "final_b")
+    # the initial states (RMS 0.5 over dstate columns) lift the 16-bit cases' outputs well above unit scale
+    big = dtype != torch.float32
+    assert_close(out, ro, dtype, "out", scaled=big)
+    assert_close(ff, rff, dtype, "final_f", scaled=big)
+    assert_close(fb, rfb, dtype, "final_b", scaled=big)
     for k in ("x", "B", "C", "z", "dt", "A", "D", "dt_bias"):
         if r[k] is not None:
-            assert_close(leaves[k].grad, r[k].grad, dtype, "d" + k)
-    assert_close(di["f"].grad, ri["f"].grad, dtype, "dinitial_f")
-    assert_close(di["b"].grad, ri["b"].grad, dtype, "dinitial_b")
+            assert_close(leaves[k].grad, r[k].grad, dtype, "d" + k, scaled=big or is_reduced("d" + k, dtype))
+    assert_close(di["f"].grad, ri["f"].grad, dtype, "dinitial_f", scaled=big)
+    assert_close(di["b"].grad, ri["b"].grad, dtype, "dinitial_b", scaled=big)
 
 
 def test_cut_sequence_equals_the_whole(ops):

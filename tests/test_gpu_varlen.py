@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import bimamba2_oracle as O
-from tests.helpers import assert_close, make_case, to64, to_dev
+from tests.helpers import assert_close, is_reduced, make_case, to64, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -29,6 +29,10 @@ CASES = [
     (2, 100, 4, 16, 2, 8, 32, torch.float32, False, [(17, 32, 33, 64), ()]),
     (2, 300, 4, 64, 2, 64, 128, torch.bfloat16, True, [(128, 200), (1, 255, 256, 299)]),
     (1, 512, 8, 64, 1, 64, 256, torch.bfloat16, False, [(100, 256, 300)]),
+    # many short sequences inside one chunk: 32 (float32) resp. 42 (bf16) boundaries per 256 positions, every one adding its cut to the
+    # chunk's cumulative sums
+    (2, 512, 4, 32, 2, 16, 256, torch.float32, False, [tuple(range(8, 264, 8)), tuple(range(4, 512, 8))]),
+    (1, 512, 4, 64, 1, 64, 256, torch.bfloat16, True, [tuple(range(6, 510, 6))]),
 ]
 
 
@@ -47,10 +51,13 @@ def test_packed_sequences_forward_and_backward(ops, case):
     ro = O.bimamba2_sequential(r["x"], r["dt"], r["A"], r["B"], r["C"], D=r["D"], z=r["z"], dt_bias=r["dt_bias"],
                                dt_softplus=True, seq_idx=si.long())[0]
     ro.backward(dout.double())
-    assert_close(out, ro, dtype, "out")
+    # 16-bit cases: outputs up to 40 from operands rounded to 8 bits of mantissa leave a few elements per 100000 beyond the
+    # plain bound (the same without seq_idx)
+    big = dtype != torch.float32
+    assert_close(out, ro, dtype, "out", scaled=big)
     for k in ("x", "B", "C", "z", "dt", "A", "D", "dt_bias"):
         if r[k] is not None:
-            assert_close(leaves[k].grad, r[k].grad, dtype, "d" + k)
+            assert_close(leaves[k].grad, r[k].grad, dtype, "d" + k, scaled=is_reduced("d" + k, dtype))
 
 
 def test_packed_equals_one_by_one(ops):

@@ -125,6 +125,22 @@ def test_gradients_of_forms_agree():
         torch.testing.assert_close(a[k], b[k], rtol=1e-10, atol=1e-10, msg=lambda m: f"{k}: {m}")
 
 
+def test_gradients_through_the_stage_functions_agree_with_the_closed_form():
+    """The GPU tests of the backward stages take torch.autograd through the stage_* functions as the expected value: here
+    the gradients through their composition (ragged last chunk, grouped heads) are held against the closed form's."""
+    inp = to64(make_case(2, 70, 4, 4, 2, 4, with_z=True, D_has_hdim=True))
+    dout = torch.randn(inp["x"].shape, dtype=torch.float64, generator=torch.Generator().manual_seed(4))
+    names = ("x", "dt", "A", "B", "C", "D", "z", "dt_bias")
+    leaves = {k: inp[k].clone().requires_grad_(True) for k in names}
+    out = O.bimamba2_staged(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], 32, D=leaves["D"], z=leaves["z"],
+                            dt_bias=leaves["dt_bias"], dt_softplus=True)[0]
+    out.backward(dout)
+    ref = O.bimamba2_grads(dout, inp["x"], inp["dt"], inp["A"], inp["B"], inp["C"], D=inp["D"], z=inp["z"],
+                           dt_bias=inp["dt_bias"], dt_softplus=True, form="quadratic")
+    for k in names:
+        torch.testing.assert_close(leaves[k].grad, ref["d" + k], rtol=1e-10, atol=1e-10, msg=lambda m: f"{k}: {m}")
+
+
 def test_causal_operator_against_the_plain_recurrence():
     """ssd_causal (what the single-direction comparator is checked against) against the token-by-token recurrence
     h_t = e^{dt_t A} h_{t-1} + dt_t x_t (x) B_t,  y_t = C_t . h_t + D x_t  written out here, and: the two causal passes
