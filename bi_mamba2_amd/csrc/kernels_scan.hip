@@ -721,6 +721,13 @@ static int launch_scan_t(const bimamba2_params *p) {
     const void *c16f = BWD ? p->dstates16_f : p->states16_f, *c16b = BWD ? p->dstates16_b : p->states16_b;
     if (c16f && (!al16(c16f) || !al16(c16b) || !(p->causal || c16b))) return BIMAMBA2_EINVAL;
     if constexpr (sizeof(T) == 2 && NJMAX == 4) {
+#ifndef BM2_SCAN_V1
+        // the shapes of the 16-bit kernel with transposed products and a raw operand tile: it needs the 16-bit copies of the
+        // entering states (the composites keep them at these shapes) and no CB
+        if (c16f && (BWD ? p->CBT : p->CB) == nullptr && scan_recomputes_cb(p, BWD) && (P == 64 || P == 128) && N == 64 &&
+            (p->causal || c16b))
+            return launch_chunk_scan16(p, BWD);
+#endif
         if (p->causal) {                                // single-direction comparator: the fused kernels only
             if (!scan_recomputes_cb(p, BWD)) return BIMAMBA2_EUNSUPPORTED;
             if (qt == 1) hipLaunchKernelGGL((chunk_scan_kernel<T, 1, 4, BWD, true, 2, true>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);

@@ -14,6 +14,8 @@ int launch_chunk_state(const bimamba2_params *p, bool dstates, bool cumsum = fal
 bool chunk_state_does_cumsum(const bimamba2_params *p);
 int launch_state_passing_fwd(const bimamba2_params *p);
 int launch_chunk_scan(const bimamba2_params *p, bool bwd);
+// the 16-bit kernel of kernels_scan16.hip (launch_chunk_scan picks it where it applies)
+int launch_chunk_scan16(const bimamba2_params *p, bool bwd);
 // true when that launch recomputes CB (bwd: CB^T) from the C and B rows instead of reading it
 bool scan_recomputes_cb(const bimamba2_params *p, bool bwd);
 // true when the dCB launch can rebuild its CB tiles from the C and B rows (then CB may be NULL)
