@@ -131,6 +131,10 @@ template <int OFF> __device__ __forceinline__ void raw_lds_write_at(unsigned add
     static_assert(OFF >= 0 && OFF < 65536, "DS offset field is 16 bits");
     asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
 }
+template <int OFF> __device__ __forceinline__ void raw_lds_write16_at(unsigned addr, _Float16 v) {
+    static_assert(OFF >= 0 && OFF < 65536, "DS offset field is 16 bits");
+    asm volatile("ds_write_b16 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
+}
 template <int OFF> __device__ __forceinline__ void raw_lds_write128_at(unsigned addr, f32x4 v) {
     static_assert(OFF >= 0 && OFF < 65536, "DS offset field is 16 bits");
     asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
@@ -403,6 +407,14 @@ __device__ __forceinline__ float row16_sum(float v) {
     v += dpp_mov<0x124>(v);  // row_ror:4
     v += dpp_mov<0x122>(v);  // row_ror:2
     v += dpp_mov<0x121>(v);  // row_ror:1
+    return v;
+}
+// the largest of the 16 lanes' values, likewise
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_mov<0x128>(v));
+    v = fmaxf(v, dpp_mov<0x124>(v));
+    v = fmaxf(v, dpp_mov<0x122>(v));
+    v = fmaxf(v, dpp_mov<0x121>(v));
     return v;
 }
 // inclusive prefix / suffix sums over the 64 lanes

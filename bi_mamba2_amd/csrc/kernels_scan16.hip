@@ -1,21 +1,36 @@
 // The chunk-scan kernel (forward output) and its mirror (dx in the backward pass) for 16-bit inputs on gfx950, for the
-// shapes every BASELINE configuration with dstate 64 has: headdim a multiple of 64, dstate 64, chunk_size a multiple of 32,
+// shapes the benchmark configurations with dstate 64 have: headdim a multiple of 64, dstate 64, chunk_size a multiple of 32,
 // 16-byte aligned operands, the states entering the chunks kept in their 16-bit copies.
 //
-// The math is that of chunk_scan_kernel (kernels_scan.hip); what differs is how little of the work is vector ALU work,
-// which is what bounds that kernel (counters: VALU busy 53 % of its duration, MFMA 19 %, LDS 29 %):
-//  * the K operand of the big product (x, resp. dy: 256 x 64 elements) goes from global memory straight into LDS as it
-//    lies in memory (direct loads, no registers, no staging code) and its MFMA fragments are LDS transpose reads;
+// The math is that of chunk_scan_kernel (kernels_scan.hip).  That kernel runs one workgroup per (batch, chunk, head): it
+// asks for its operands, waits, computes, asks for its epilogue operands, waits, stores - with two workgroups per CU the
+// memory system idles while they compute and the ALUs idle while they wait (counters: VALU busy 53 %, MFMA 19 %, 60 % of
+// the copy bandwidth).  Here ONE workgroup of 16 waves owns a CU and walks through several heads of one (batch, chunk):
+//  * everything a head needs - its x (resp. dy) tile, its two state tiles, its decay vectors, its z (resp. x) rows - travels
+//    from global memory straight into LDS (direct loads: no registers, no staging code) one head ahead of its use
+//    (double-buffered; the z / x rows of the head in hand arrive while its K loop runs), so nothing but the first head's
+//    operands is ever waited for.  The requests for the next head go out a part at a time during the K loop (issued in one
+//    go behind the previous head's stores they fill the memory pipeline's queue and the wave stalls at the issue), and
+//    between the requests and the wait in front of the epilogue there is no vector memory operation and no LDS access the
+//    compiler knows of: it would make either wait for everything in flight (hence the raw_lds_* accessors);
+//  * the heads of a group share C.B^T: each wave computes the CB (resp. CB^T) entries of its 16 rows x 256 columns once and
+//    keeps them in 32 registers as float16 pairs, scaled by a power of two that is common to the workgroup so that the
+//    largest entry sits at 2^14 (float16 keeps 11 bits of mantissa, three more than the bf16 the masked entries are
+//    rounded to for the MFMA anyway; the scale rules out overflow); the K loop has neither a ring of K rows nor a barrier
+//    nor CB MFMAs;
+//  * away from the diagonal the decay factor of (row r, column k) separates into a factor of the row and the column's
+//    16-block and a factor of the column; the column factors are kept as float16 as well (scaled per block into [0.5, 1),
+//    the exponent going to the row factor), so a K step multiplies them onto the CB entries two at a time and then
+//    applies the row factor with the conversion to float32 in the same instruction: 2 instructions per entry instead of 3.5
+//    (the kernel is bound by VALU issue: 63 % busy against 16 % for the MFMA pipe);
+//  * the K operand lies in LDS as it lies in memory and its MFMA fragments are LDS transpose reads;
 //  * the products are computed transposed, D[p][r] = sum_k X[k][p] A[r][k]: operand fragments are the same registers as
 //    for D[r][p] with the two MFMA operands swapped, but a lane then holds four consecutive headdim columns of ONE row
 //    per 16-column tile.  Which headdim column an MFMA row stands for is free (it is decided where the operand
 //    fragments are read), and is chosen so that the tiles 2t and 2t + 1 together give a lane EIGHT consecutive columns,
-//    32 t + 8 (lane / 16) ..: out / out_x / dx leave as 16-byte stores and x / z / dy arrive as 16-byte loads without the
-//    accumulators passing through LDS, and the per-row factors are one value per lane;
-//  * the D term's rows are 16-byte LDS reads of the raw tile;
-//  * the state tiles arrive by direct loads as well; one barrier in front of the K loop, none behind it (waves leave the
-//    loop and write their rows independently);
-//  * the K loop is unrolled over its (at most 8) steps, so ring slots, table offsets and fragment offsets are immediates.
+//    32 t + 8 (lane / 16) ..: out / out_x / dx leave as 16-byte stores and z / x / dy arrive as 16-byte LDS reads without
+//    the accumulators passing through LDS, and the per-row factors are one value per lane;
+//  * the K loop is unrolled over its (at most 8) steps: table and fragment offsets are immediates.
 //
 //   forward (BWD = false), rows r = output positions t, k = source positions s:
 //     acc[r,p] = e^{cs_f[r]} C_r.prev_f[p,:] + e^{cs_b[r]} C_r.prev_b[p,:]
@@ -35,18 +50,31 @@ namespace bm2 {
 namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr int S16_WAVES = 8, S16_THREADS = 64 * S16_WAVES;
-constexpr int S16_KRING = 4;                       // slots of the K-row ring: requests run three K steps ahead
+constexpr int S16_WAVES = 16, S16_THREADS = 64 * S16_WAVES;
+constexpr int S16_ROWS = 16 * S16_WAVES;          // rows the workgroup covers (>= chunk_size)
+constexpr int S16_NSTEP = S16_ROWS / 32;          // K steps at most
+constexpr int S16_MAX_HEADS = 4;                  // heads a workgroup walks through at most
 
-// byte offset of the four elements (r, n .. n + 3), n a multiple of 4, in a raw [rows][64] 16-bit tile whose 16-byte chunks
-// are swizzled by tile64_swz (the layout tile64_request leaves)
+// LDS map (bytes)
+constexpr int S16_XR = 0;                                     // 2 x raw K-operand tile (x, resp. dy): [256][64] 16-bit, tile64 swizzle
+constexpr int S16_ST = S16_XR + 2 * 32768;                    // 2 x 2 state tiles [p][n], 16-byte chunks ^ (p % 8)
+constexpr int S16_KT = S16_ST + 2 * 2 * 8192;                 // K rows (B, resp. C) of the chunk, chunks ^ (row % 8); afterwards
+                                                              // the z (resp. x) rows of the head in hand, tile64 swizzle
+constexpr int S16_RAW = S16_KT + 32768;                       // 2 x (cs_f, cs_b, dt) of a head as they lie in memory
+constexpr int S16_TAB = S16_RAW + 2 * 3 * 1024;               // lo, up, glo, gup, dtl of the head in hand
+constexpr int S16_RED = S16_TAB + 5 * 1024;                   // mirror: per-wave column sums of dy * x
+constexpr int S16_DT = S16_RED + S16_WAVES * 64 * 4;           // D of the workgroup's heads, one value per headdim column
+constexpr int S16_LDS = S16_DT + S16_MAX_HEADS * 64 * 4;
+
+// byte offset of the elements (r, n ..), n a multiple of 4, in a raw [rows][64] 16-bit tile whose 16-byte chunks are swizzled
+// by tile64_swz (the layout tile64_request leaves)
 __device__ __forceinline__ int tile64_row_offset(int r, int n) {
     return r * 128 + ((((n >> 3) ^ tile64_swz(r)) << 4) | ((n & 4) << 1));
 }
 
 // headdim column (inside the workgroup's 64) that row m of the 16-row MFMA tile j stands for: 32 (j/2) + 8 (m/4) + 4 (j%2) + m%4.
 // Output rows m = 4 g + i of lane group g are then the columns 32 t + 8 g + i (tile 2t) and 32 t + 8 g + 4 + i (tile 2t + 1).
-__device__ __forceinline__ int s16_col(int j, int m) { return 32 * (j >> 1) + 8 * (m >> 2) + 4 * (j & 1) + (m & 3); }
+__device__ __forceinline__ constexpr int s16_col(int j, int m) { return 32 * (j >> 1) + 8 * (m >> 2) + 4 * (j & 1) + (m & 3); }
 
 // f(integral_constant<int, I>) for I = 0 .. N - 1, until it returns false: a loop whose index is a constant expression inside
 // the body (LDS offsets become immediates)
@@ -56,397 +84,566 @@ template <int I, int N, class F> __device__ __forceinline__ void static_for(F &&
     }
 }
 
+// load16_to_lds(base + off) with the address in the scalar-base form: `base` wave-uniform, `off` this lane's 32-bit byte
+// offset.  The offset passes through an empty asm right in front of the load, which keeps the 64-bit add next to the load
+// (hoisted into another block it could not be folded into the instruction and would cost two registers per address).
+__device__ __forceinline__ void load16_to_lds_at(const char *base, unsigned off, void *lds_wave_base) {
+    asm volatile("" : "+v"(off));
+    load16_to_lds(base + off, lds_wave_base);
+}
+
+// A wave-uniform pointer, made visibly so (through 64-bit address arithmetic the compiler loses sight of it and would build
+// the address per lane): base + 32-bit lane offset then takes the scalar-base form of the memory instructions.
+__device__ __forceinline__ const char *uniform_ptr(const void *ptr) {
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const char *>(((uint64_t)hi << 32) | lo);
+}
+
 }  // namespace
 
-// QT: 16-row tiles per wave (8 waves: the workgroup covers 128 * QT rows >= chunk_size).  UNI: the single-direction
-// (causal) operator: the reverse direction's state product, the K steps on the far side of the diagonal and the far half of
-// the diagonal step are left out.
-template <typename T, int QT, bool BWD, bool UNI>
-__global__ __launch_bounds__(S16_THREADS, 4) void chunk_scan16_kernel(const bimamba2_params p, int nc, int npt) {
+// UNI: the single-direction (causal) operator: the reverse direction's state product, the K steps on the far side of the
+// diagonal and the far half of the diagonal step are left out.
+// hpw: heads per workgroup (divides nheads / ngroups, <= S16_MAX_HEADS); blockIdx.x = ((pt * nslices + slice) * nbc + bc).
+template <typename T, bool BWD, bool UNI>
+__global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba2_params p, int nc, int npt, int hpw) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
     static_assert(sizeof(T) == 2, "16-bit operands");
-    constexpr int KSTEP = 32;
-    constexpr int QP = S16_WAVES * 16 * QT;        // rows the workgroup covers
-    constexpr int NSTEP = QP / KSTEP;              // K steps at most
-    __shared__ __attribute__((aligned(16))) T xr[QP * 64];                     // raw K-operand tile (x, resp. dy), swizzled
-    __shared__ __attribute__((aligned(16))) T krl[S16_KRING * 32 * 64];        // ring of K rows (B, resp. C) for the CB tiles
-    __shared__ __attribute__((aligned(16))) T sF[64 * 64], sB[UNI ? 8 : 64 * 64];   // state tiles [p][n], 16-byte chunks ^ (p % 8)
-    __shared__ float lo[QP], up[QP];               // decay exponents (times log2 e), see below
-    __shared__ float glo[QP], gup[QP];             // their column factors relative to the edge of the 16-block
-    __shared__ float dtl[QP];                      // forward: dt of the columns; mirror: 1 inside the sequence, 0 behind it
-    __shared__ float red[BWD ? S16_WAVES : 1][64];
+    constexpr int KSTEP = 32, NSTEP = S16_NSTEP;
+    // (aligned: the fragment addresses below flip bit 6 of an absolute LDS address)
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[S16_LDS];
+    const unsigned sbase = lds_addr(smem);
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lr = lane & 15, lg = lane >> 4;
-    // linear block id -> (pt, h, bc) with bc fastest: consecutive ids are dealt round-robin to the 8 XCDs, so all heads of
-    // one (batch, chunk), which share the B and C rows, stay on one XCD's L2
+    // consecutive block ids are dealt round-robin to the 8 XCDs: bc fastest keeps the workgroups of one (batch, chunk), which
+    // share the B and C rows, on one XCD's L2
     const int nbc = p.batch * nc;
-    const int bc = blockIdx.x % nbc, hp = blockIdx.x / nbc, pt = hp % npt, h = hp / npt;
+    const int bc = blockIdx.x % nbc, sp = blockIdx.x / nbc, nslices = p.nheads / hpw, slice = sp % nslices, pt = sp / nslices;
     const int c = bc % nc, b = bc / nc;
-    const int g = h / (p.nheads / p.ngroups);
+    const int h0 = slice * hpw;
+    const int g = h0 / (p.nheads / p.ngroups);
     const int Q = p.chunk_size, P = p.headdim, H = p.nheads;
     const int limit = min(Q, p.seqlen - c * Q);
     const int nsteps = (limit + KSTEP - 1) / KSTEP;
     const int p0 = pt * 64;
-    const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
-    const float *csf = p.cs_f + o, *csb = p.cs_b + o, *dto = p.dt_out + o;
-    const float d_head = (p.has_D && !p.D_has_hdim) ? p.D[h] : 0.f;
+    const int wr0 = wave * 16;                     // this wave's rows wr0 .. wr0 + 15
+    const bool active = wr0 < limit;               // (uniform) waves whose rows lie behind the end only help with the loads
+    const int r_own = wr0 + lr, rc_own = min(r_own, limit - 1);
 
-    // ---- every request of the prologue goes out before anything is waited for ----
-    // K rows of the first ring slots: wave w brings rows 4w..4w+3 of a step; unit u = 32*w + lane (lane < 32) is row u/8,
-    // chunk position u%8, which holds the row's 16-byte chunk (u%8) ^ (row % 8)
-    const char *krbase;
-    unsigned krs_bytes;
-    if (BWD) { krs_bytes = (unsigned)p.C_sl * sizeof(T); krbase = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * p.C_sl + g * p.C_sg); }
-    else { krs_bytes = (unsigned)p.B_sl * sizeof(T); krbase = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * p.B_sl + g * p.B_sg); }
-    {
-        const uint64_t kb64 = reinterpret_cast<uint64_t>(krbase);
-        const uint32_t klo = __builtin_amdgcn_readfirstlane((uint32_t)kb64), khi = __builtin_amdgcn_readfirstlane((uint32_t)(kb64 >> 32));
-        krbase = reinterpret_cast<const char *>(((uint64_t)khi << 32) | klo);
-    }
-    const int kr_row = wave * 4 + ((lane & 31) >> 3);                           // this lane's row inside a step
-    const unsigned kr_col = (((lane & 7) ^ (kr_row & 7)) * 16);
-    auto kr_issue = [&](int step) {
-        if (lane < 32) {
-            const unsigned off = (unsigned)min(step * 32 + kr_row, limit - 1) * krs_bytes + kr_col;
-            load16_to_lds(krbase + off, krl + (step % S16_KRING) * (32 * 64) + wave * 256);
+    // Every global address below is a wave-uniform 64-bit base (scalar registers) plus a 32-bit byte offset of the lane (the
+    // launcher checks that 256 rows of every row stride fit 32 bits): lane parts are few and cheap to keep.
+    // rows u*8 + lane/8 (u = 2 wave, 2 wave + 1) of a 256-row tile, 16-byte chunk (lane%8) ^ swizzle(row) at chunk position lane%8
+    // The lane parts are recomputed from the lane number wherever they are needed (`ln` is made opaque there: kept across
+    // the head loop they would be spilled, and a reload from scratch memory between two requests waits for the first one).
+    const unsigned ks_bytes = (unsigned)((!BWD ? p.x_sl : p.has_z ? (int64_t)H * P : p.dout_sl) * (int64_t)sizeof(T));
+    const unsigned s2_bytes = (unsigned)((BWD ? p.x_sl : p.z_sl) * (int64_t)sizeof(T));
+    // rows wave*16 + ln/8 (+8) of a 256-row tile with row stride `rs` bytes: 16-byte chunk (ln%8) ^ swizzle(row) at position ln%8
+    auto tile_off = [&](int ln, int half, unsigned rs) __attribute__((always_inline)) {
+        const int row = wave * 16 + half * 8 + (ln >> 3);
+        return (unsigned)min(row, limit - 1) * rs + (unsigned)(((ln & 7) ^ tile64_swz(row)) << 4);
+    };
+
+    // ---- requests of a head: its K-operand tile (parts 0, 1), its two state tiles (2), its decay vectors (3) -> buffer `buf`.
+    // In parts, so that the K loop can hand them to the memory pipeline one at a time: issued in one go behind the previous
+    // head's output stores they fill its queue, and a wave whose request does not fit waits there instead of computing.
+    auto request_part = [&](int h, int buf, int part) __attribute__((always_inline)) {
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        if (part < 2) {
+            const char *kp;
+            if (!BWD) kp = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh + p0);
+            else if (p.has_z) kp = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * H * P + (int64_t)h * P + p0);
+            else kp = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * p.dout_sl + h * p.dout_sh + p0);
+            kp = uniform_ptr(kp);
+            // (rows behind the last K step are never read; their requests go to the clamped, valid row all the same)
+            load16_to_lds_at(kp, tile_off(ln, part, ks_bytes), smem + S16_XR + buf * 32768 + wave * 2048 + part * 1024);
+        } else if (part == 2) {
+            const int dir = wave >> 3;
+            if (!(UNI && dir)) {
+                const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * 64 + (int64_t)p0 * 64;
+                const T *src = reinterpret_cast<const T *>(BWD ? (dir ? p.dstates16_b : p.dstates16_f) : (dir ? p.states16_b : p.states16_f));
+                // thread t of a half brings row t/8, chunk position t%8 <- chunk (t%8) ^ (row%8)
+                const int row = (wave & 7) * 8 + (ln >> 3);
+                const unsigned soff = (unsigned)((row * 64 + (((ln & 7) ^ (row & 7)) << 3)) * sizeof(T));
+                load16_to_lds_at(uniform_ptr(src + so), soff, smem + S16_ST + (buf * 2 + dir) * 8192 + (wave & 7) * 1024);
+            }
+        } else if (wave < 3) {
+            // cs_f, cs_b, dt (waves 0, 1, 2): 256 floats each (entries past chunk_size are never used: clamped to stay inside)
+            const float *src = (wave == 0 ? p.cs_f : wave == 1 ? p.cs_b : p.dt_out) + (((int64_t)b * H + h) * nc + c) * Q;
+            load16_to_lds_at(uniform_ptr(src), (unsigned)min(ln * 4, Q - 4) * 4u, smem + S16_RAW + (buf * 3 + wave) * 1024);
         }
     };
+    auto request_head = [&](int h, int buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int st = 0; st < S16_KRING - 1; ++st)
-        if (st < nsteps) kr_issue(st);
-    // the K operand of the big product, as it lies in memory
-    const T *kp;
-    int64_t ks;
-    if (!BWD) { ks = p.x_sl; kp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * ks + h * p.x_sh; }
-    else if (p.has_z) { ks = (int64_t)H * P; kp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * ks + (int64_t)h * P; }
-    else { ks = p.dout_sl; kp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * ks + h * p.dout_sh; }
-    tile64_request(xr, kp + p0, ks, nsteps * KSTEP, limit, wave, S16_WAVES, lane);
-    // the two state tiles: thread t brings row t/8, chunk position t%8 <- chunk (t%8) ^ (row%8)
+        for (int part = 0; part < 4; ++part) request_part(h, buf, part);
+    };
+    // requests of a head this wave issues (the vmcnt a wait for something older has to leave outstanding)
+    const int head_requests = 2 + ((UNI && wave >= 8) ? 0 : 1) + (wave < 3 ? 1 : 0);
+
+    // ---- prologue: the K rows of the chunk (B, resp. C), this lane's own rows (C, resp. B), the first head's operands.  The
+    // products below wait for the first two only; the head's operands land meanwhile.  (LDS accesses are raw from here on.)
     {
-        const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * 64 + (int64_t)p0 * 64;
-        const int row = threadIdx.x >> 3, ch = (threadIdx.x & 7) ^ (row & 7);
-        const T *s16f = reinterpret_cast<const T *>(BWD ? p.dstates16_f : p.states16_f) + so + row * 64 + ch * 8;
-        load16_to_lds(s16f, sF + wave * 512);
-        if (!UNI) {
-            const T *s16b = reinterpret_cast<const T *>(BWD ? p.dstates16_b : p.states16_b) + so + row * 64 + ch * 8;
-            load16_to_lds(s16b, sB + wave * 512);
+        const T *kr;
+        int64_t krs;
+        if (BWD) { krs = p.C_sl; kr = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * krs + g * p.C_sg; }
+        else { krs = p.B_sl; kr = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * krs + g * p.B_sg; }
+#pragma unroll
+        for (int uu = 0; uu < 2; ++uu) {
+            const int u = wave * 2 + uu, row = u * 8 + (lane >> 3);
+            if (u * 8 < nsteps * KSTEP)
+                load16_to_lds_at(uniform_ptr(kr), (unsigned)min(row, limit - 1) * (unsigned)(krs * sizeof(T)) + (((lane & 7) ^ (row & 7)) << 4), smem + S16_KT + u * 1024);
         }
     }
-    // this lane's rows of the other matrix (forward: C, mirror: B) in operand layout: rows wr0 + 16 rt + lr
-    const int wr0 = wave * 16 * QT;
-    const T *ap;
-    int64_t as;
-    if (BWD) { as = p.B_sl; ap = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * as + g * p.B_sg; }
-    else { as = p.C_sl; ap = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * as + g * p.C_sg; }
-    Frag own[QT][2];
+    Frag own[2];
+    {
+        const T *ap;
+        int64_t as;
+        if (BWD) { as = p.B_sl; ap = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * as + g * p.B_sg; }
+        else { as = p.C_sl; ap = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * as + g * p.C_sg; }
 #pragma unroll
-    for (int rt = 0; rt < QT; ++rt)
-#pragma unroll
-        for (int f = 0; f < 2; ++f) own[rt][f] = M::load(ap + (int64_t)min(wr0 + rt * 16 + lr, limit - 1) * as + f * KSTEP + lg * 8);
-    // forward: k<r uses lo[r]-lo[k] with lo = cs_f, k>r uses up[r]-up[k] with up = cs_b
-    // mirror : k<r uses e^{cs_b[k]-cs_b[r]} -> lo = -cs_b;  k>r uses e^{cs_f[k]-cs_f[r]} -> up = -cs_f
-    // Away from the diagonal the factor separates: with m = lo at the last position of k's block of 16 (which lies
-    // between k and r), 2^{lo[r]-lo[k]} = 2^{lo[r]-m} * glo[k], glo[k] = 2^{m-lo[k]}, both factors <= 1 for A <= 0;
-    // likewise gup[k] = 2^{up[first of k's block] - up[k]}.  The column factors also carry dt[k] (forward) and the zero
-    // of the rows behind the end of the sequence, which the raw tile holds as copies of its last row.
-    for (int q = threadIdx.x; q < QP; q += S16_THREADS) {
-        const int qq = min(q, Q - 1), qe = min(q | 15, Q - 1), qs = min(q & ~15, Q - 1);
-        const float f = csf[qq] * LOG2E, r = csb[qq] * LOG2E;
-        const float fe = (BWD ? -csb[qe] : csf[qe]) * LOG2E, rs = (BWD ? -csf[qs] : csb[qs]) * LOG2E;
-        const float dtq = q < limit ? (BWD ? 1.f : dto[qq]) : 0.f;
-        const float l = BWD ? -r : f, u = BWD ? -f : r;
-        lo[q] = l;
-        up[q] = u;
-        glo[q] = __builtin_amdgcn_exp2f(fe - l) * dtq;
-        gup[q] = __builtin_amdgcn_exp2f(rs - u) * dtq;
-        dtl[q] = dtq;
+        for (int f = 0; f < 2; ++f) own[f] = M::load(ap + (int64_t)rc_own * as + f * KSTEP + lg * 8);
     }
-    const float e_f = BWD ? csf[Q - 1] * LOG2E : 0.f, e_b = BWD ? csb[0] * LOG2E : 0.f;   // mirror: the far ends of the chunk
-    wait_vmcnt<0>();
-    __syncthreads();
-
-    // ---- part 1: states.  D[p][r] = sum_n S[p][n] Own[r][n], scaled by this lane's row factor, one direction after the other
-    f32x4 acc[QT][4];
-    float lor[QT], upr[QT];
-#pragma unroll
-    for (int rt = 0; rt < QT; ++rt) {
-        lor[rt] = lo[wr0 + rt * 16 + lr];
-        upr[rt] = up[wr0 + rt * 16 + lr];
+    float d_val = 0.f;                             // D of head h0 + tid / 64, headdim column tid % 64
+    if ((int)threadIdx.x < hpw * 64 && p.has_D) {
+        const int hh = h0 + ((int)threadIdx.x >> 6), col = threadIdx.x & 63;
+        d_val = p.D_has_hdim ? p.D[hh * P + p0 + col] : p.D[hh];
     }
-#pragma unroll
-    for (int dir = 0; dir < (UNI ? 1 : 2); ++dir) {
-        const T *st = dir ? sB : sF;
-        f32x4 tmp[QT][4] = {};
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            Frag sf[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int pr = s16_col(j, lr);     // the state row (headdim column) this lane's MFMA row stands for
-                sf[j] = M::load(st + pr * 64 + (((s * 4 + lg) ^ (pr & 7)) << 3));
-            }
-#pragma unroll
-            for (int rt = 0; rt < QT; ++rt)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) tmp[rt][j] = M::mma(sf[j], own[rt][s], tmp[rt][j]);
-        }
-#pragma unroll
-        for (int rt = 0; rt < QT; ++rt) {
-            // forward: e^{cs_f[r]} = 2^{lo[r]}, e^{cs_b[r]} = 2^{up[r]}; mirror: e^{cs_f[Q-1]-cs_f[r]} = 2^{e_f+up[r]}, e^{cs_b[0]-cs_b[r]} = 2^{e_b+lo[r]}
-            const float e = __builtin_amdgcn_exp2f(BWD ? (dir ? e_b + lor[rt] : e_f + upr[rt]) : (dir ? upr[rt] : lor[rt]));
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[rt][j] = dir ? tmp[rt][j] * e + acc[rt][j] : tmp[rt][j] * e;
-        }
-    }
-
-    // ---- part 2: inside the chunk.  Per K step of 32 columns: the CB (resp. CB^T) tiles of this wave's rows from its own
-    // rows and the step's K rows (arranged so that the product comes out in operand layout: D[m][n] = sum_d Krow[k(m)][d]
+    request_head(h0, 0);
+    // everything older than this wave's last two requests has landed (a wave issues at least two per head): the K rows it
+    // brought, its own rows, its D values
+    wait_vmcnt<2>();
+    if ((int)threadIdx.x < hpw * 64) raw_lds_write_at<0>(sbase + S16_DT + threadIdx.x * 4, d_val);
+    raw_lds_wait();
+    raw_lds_barrier();
+    // CB (resp. CB^T) of this wave's rows against every column of the chunk, in operand layout: D[m][n] = sum_d Krow[k(m)][d]
     // Own[n][d] with k(m) = k0 + 8*(m/4) + m%4 leaves lane (l%16 = row, l/16 = g) with columns k0 + 8g + 0..3, the second
-    // product with +4), times the decay factors, times the K operand.
+    // product (k(m) + 4) with columns k0 + 8g + 4..7.  Fragment (hh, f): K row krow + 4*hh of the step, 16-byte chunk lg + 4*f,
+    // stored at chunk ^ (row % 8); with krow % 8 = lr % 4 that is element kfb + 256*hh + 32*(f ^ hh) of the step's 32 rows.
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    unsigned cbh[NSTEP][4];                        // step s: columns k0 + 8 lg + {0,1}, {2,3}, {4,5}, {6,7} of row wr0 + lr (float16 pairs)
+    float cb_unscale;                              // 1 / (the power of two the entries were scaled by)
     {
-        // fragment (hh, f): K row krow + 4*hh of the step, 16-byte chunk lg + 4*f, stored at chunk ^ (row % 8); with
-        // krow % 8 = lr % 4 that is element kfb + 256*hh + 32*(f ^ hh) of the slot
+        f32x4 cb1[NSTEP], cb2[NSTEP];
         const int kfb = (8 * (lr >> 2) + (lr & 3)) * 64 + (lg ^ (lr & 3)) * 8;
-        const unsigned krl_a = lds_addr(krl) + kfb * 2;
-        // K-operand fragments: LDS transpose reads of the raw tile, rows k0 + 8 lg + lr/4 (+4); source lane s of a 16-lane group
-        // supplies the four columns s16_col(j, 4 (s%4)) .., which lanes 4 (s%4) .. + 3 of the group receive
-        // (rows k + 4: the swizzle flips bit 2 of the chunk position, i.e. byte bit 6, and the row adds 512 bytes)
-        unsigned xo_lo[4];
-        {
-            const int kk = 8 * lg + (lr >> 2);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) xo_lo[j] = lds_addr(xr) + tile64_tr_offset(kk, s16_col(j, 4 * (lr & 3)));
-        }
-        const unsigned lg32 = lg * 32;             // this lane's 8 columns inside a step of the float tables
-        const unsigned glo_a = lds_addr(glo) + lg32, gup_a = lds_addr(gup) + lg32, lo_a = lds_addr(lo) + lg32, up_a = lds_addr(up) + lg32;
-        const unsigned dtl_a = lds_addr(dtl) + lg32;
-        // reference points of the column factors: lo at the last, up at the first position of this lane's block of 16
-        const unsigned mlo_a = lds_addr(lo) + ((lg * 8) | 15) * 4, mup_a = lds_addr(up) + ((lg * 8) & ~15) * 4;
-        auto k_step = [&](auto STEP) __attribute__((always_inline)) -> bool {
-            constexpr int step = decltype(STEP)::value;
-            if (step >= nsteps) return false;
-            constexpr int k0 = step * KSTEP;
-            // this wave's request for the step has landed: one request per step, up to KRING - 2 newer ones
-            const int newer = min(S16_KRING - 2, nsteps - 1 - step);
-            if (newer >= 2) wait_vmcnt<2>();
-            else if (newer == 1) wait_vmcnt<1>();
-            else wait_vmcnt<0>();
-            raw_lds_barrier();                     // ... and everybody else's; the slot of step - 1 is free again
-            if (step + S16_KRING - 1 < nsteps) kr_issue(step + S16_KRING - 1);
-            // the wave's rows [wr0, wr0 + 16*QT) meet the step's columns [k0, k0 + 32) in one step only
-            const int cls = (k0 + KSTEP - 1 < wr0) ? 0 : (k0 > wr0 + QT * 16 - 1) ? 1 : 2;   // below, above, across the diagonal
-            if (UNI && cls == (BWD ? 0 : 1)) return true;                                      // far side of the diagonal
-            constexpr int SLOT = (step % S16_KRING) * (32 * 64 * 2);
-            f32x4 cb1[QT], cb2[QT];
-            {
-                Frag kf00 = raw_lds_read_at<Frag, SLOT>(krl_a), kf01 = raw_lds_read_at<Frag, SLOT + 64>(krl_a);
-                Frag kf10 = raw_lds_read_at<Frag, SLOT + 512 + 64>(krl_a), kf11 = raw_lds_read_at<Frag, SLOT + 512>(krl_a);
+        const unsigned kt = sbase + S16_KT + kfb * 2;
+        static_for<0, NSTEP>([&](auto S) __attribute__((always_inline)) {
+            constexpr int s = decltype(S)::value;
+            cb1[s] = cb2[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (active && s < nsteps) {
+                Frag kf00 = raw_lds_read_at<Frag, s * 4096>(kt), kf01 = raw_lds_read_at<Frag, s * 4096 + 64>(kt);
+                Frag kf10 = raw_lds_read_at<Frag, s * 4096 + 512 + 64>(kt), kf11 = raw_lds_read_at<Frag, s * 4096 + 512>(kt);
                 raw_lds_wait();
                 raw_lds_use(kf00); raw_lds_use(kf01); raw_lds_use(kf10); raw_lds_use(kf11);
-#pragma unroll
-                for (int rt = 0; rt < QT; ++rt) {
-                    cb1[rt] = M::mma(kf00, own[rt][0], f32x4{0.f, 0.f, 0.f, 0.f});
-                    cb2[rt] = M::mma(kf10, own[rt][0], f32x4{0.f, 0.f, 0.f, 0.f});
-                    cb1[rt] = M::mma(kf01, own[rt][1], cb1[rt]);
-                    cb2[rt] = M::mma(kf11, own[rt][1], cb2[rt]);
-                }
-            }
-            const int kb = k0 + lg * 8;
-            constexpr int TB = step * (KSTEP * 4);     // byte offset of the step inside the float tables
-            Frag af[QT];
-            if (cls != 2) {
-                const unsigned ta = cls == 0 ? glo_a : gup_a;
-                f32x4 ga0 = raw_lds_read_at<f32x4, TB>(ta), ga1 = raw_lds_read_at<f32x4, TB + 16>(ta);
-                float mref = raw_lds_read_at<float, TB>(cls == 0 ? mlo_a : mup_a);
-                raw_lds_wait();
-                raw_lds_use(ga0); raw_lds_use(ga1); raw_lds_use(mref);
-#pragma unroll
-                for (int rt = 0; rt < QT; ++rt) {
-                    const float rf = __builtin_amdgcn_exp2f((cls == 0 ? lor[rt] : upr[rt]) - mref);
-                    float v[8];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { v[i] = cb1[rt][i] * rf * ga0[i]; v[i + 4] = cb2[rt][i] * rf * ga1[i]; }
-                    af[rt] = M::pack(v);
-                }
-            } else {
-                // the one step across the diagonal: element by element
-                f32x4 l0 = raw_lds_read_at<f32x4, TB>(lo_a), l1 = raw_lds_read_at<f32x4, TB + 16>(lo_a);
-                f32x4 u0 = raw_lds_read_at<f32x4, TB>(up_a), u1 = raw_lds_read_at<f32x4, TB + 16>(up_a);
-                f32x4 d0 = raw_lds_read_at<f32x4, TB>(dtl_a), d1 = raw_lds_read_at<f32x4, TB + 16>(dtl_a);
-                raw_lds_wait();
-                raw_lds_use(l0); raw_lds_use(l1); raw_lds_use(u0); raw_lds_use(u1); raw_lds_use(d0); raw_lds_use(d1);
-#pragma unroll
-                for (int rt = 0; rt < QT; ++rt) {
-                    const int r = wr0 + rt * 16 + lr;
-                    float v[8];
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        const int k = kb + i;
-                        const float lk = i < 4 ? l0[i & 3] : l1[i & 3], uk = i < 4 ? u0[i & 3] : u1[i & 3];
-                        const float e = k < r ? lor[rt] - lk : upr[rt] - uk;
-                        float w = (k == r) ? (UNI ? 1.f : 2.f) : __builtin_amdgcn_exp2f(e);
-                        if (UNI && (BWD ? k < r : k > r)) w = 0.f;
-                        w *= i < 4 ? d0[i & 3] : d1[i & 3];
-                        v[i] = (i < 4 ? cb1[rt][i & 3] : cb2[rt][i & 3]) * w;
-                    }
-                    af[rt] = M::pack(v);
-                }
-            }
-            // ---- the product with the K operand, transposed: D[p][r] += X[k][p] A[r][k]; two column tiles at a time
-            constexpr int XS = step * (KSTEP * 128);
-#pragma unroll
-            for (int jj = 0; jj < 4; jj += 2) {
-                const i16x4 a0 = raw_lds_tr16_read_at<XS>(xo_lo[jj]), a1 = raw_lds_tr16_read_at<XS + 512>(xo_lo[jj] ^ 64u);
-                const i16x4 b0 = raw_lds_tr16_read_at<XS>(xo_lo[jj + 1]), b1 = raw_lds_tr16_read_at<XS + 512>(xo_lo[jj + 1] ^ 64u);
-                raw_lds_wait();
-                i16x8 fa = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7), fb = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
-                raw_lds_use(fa); raw_lds_use(fb);
-                const Frag xa = __builtin_bit_cast(Frag, fa), xb = __builtin_bit_cast(Frag, fb);
-#pragma unroll
-                for (int rt = 0; rt < QT; ++rt) {
-                    acc[rt][jj] = M::mma(xa, af[rt], acc[rt][jj]);
-                    acc[rt][jj + 1] = M::mma(xb, af[rt], acc[rt][jj + 1]);
-                }
+                cb1[s] = M::mma(kf00, own[0], cb1[s]);
+                cb2[s] = M::mma(kf10, own[0], cb2[s]);
+                cb1[s] = M::mma(kf01, own[1], cb1[s]);
+                cb2[s] = M::mma(kf11, own[1], cb2[s]);
             }
             return true;
-        };
-        static_for<0, NSTEP>(k_step);
-        wait_vmcnt<0>();
+        });
+        // the largest entry of the workgroup decides the scale
+        float mx = 0.f;
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(fabsf(cb1[s][i]), fabsf(cb2[s][i])));
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+        if (lane == 0) raw_lds_write_at<0>(sbase + S16_RED + wave * 4, mx);
+        raw_lds_wait();
+        wait_vmcnt<0>();                           // the first head's operands (this wave's share; the barrier makes it everybody's)
+        raw_lds_barrier();                         // (everybody is done with the K rows as well: their place takes the z / x rows)
+        {
+            float wm = raw_lds_read_at<float, 0>(sbase + S16_RED + (lane & (S16_WAVES - 1)) * 4);
+            raw_lds_wait();
+            raw_lds_use(wm);
+            mx = wm;
+#pragma unroll
+            for (int d = S16_WAVES / 2; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+        }
+        // scale = 2^(14 - e), e the exponent of the maximum (1 for an all-zero or non-finite block)
+        const int ex = (int)((__float_as_uint(mx) >> 23) & 255u);
+        const bool ok = ex > 0 && ex < 255;
+        const float scale = ok ? __uint_as_float((unsigned)min(254, 127 + 14 + 127 - ex) << 23) : 1.f;
+        cb_unscale = ok ? __uint_as_float((unsigned)max(1, 127 - 14 - 127 + ex) << 23) : 1.f;
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+            cbh[s][0] = __builtin_bit_cast(unsigned, half2_t{(_Float16)(cb1[s][0] * scale), (_Float16)(cb1[s][1] * scale)});
+            cbh[s][1] = __builtin_bit_cast(unsigned, half2_t{(_Float16)(cb1[s][2] * scale), (_Float16)(cb1[s][3] * scale)});
+            cbh[s][2] = __builtin_bit_cast(unsigned, half2_t{(_Float16)(cb2[s][0] * scale), (_Float16)(cb2[s][1] * scale)});
+            cbh[s][3] = __builtin_bit_cast(unsigned, half2_t{(_Float16)(cb2[s][2] * scale), (_Float16)(cb2[s][3] * scale)});
+        }
     }
 
-    // ---- epilogue.  acc[rt][2t][i], acc[rt][2t+1][i] = row wr0 + 16 rt + lr, headdim columns p0 + 32 t + 8 lg + i, + 4 + i ----
+    // per-lane LDS addresses
+    const unsigned tab = sbase + S16_TAB;          // lo +0, up +1024, glo +2048 (mlo +2560), gup +3072 (mup +3584), dtl +4096
+    const unsigned lg32 = lg * 32;                 // this lane's 8 columns inside a step of the float tables
+    // column factors of this lane's 8 columns (8 float16 = 16 bytes) and the reference exponent of their block of 16
+    unsigned g_l = tab + 2048 + lg * 16, m_l = tab + 2048 + 512 + (lg >> 1) * 4;
+    unsigned tab_l = tab + lg32;                   // lo of this lane's columns; up +1024, glo +2048, gup +3072, dtl +4096
+    // K-operand fragments: LDS transpose reads of the raw tile, rows k0 + 8 lg + lr/4 (+4); source lane s of a 16-lane group
+    // supplies the four columns s16_col(j, 4 (s%4)) .., which lanes 4 (s%4) .. + 3 of the group receive
+    // (rows k + 4: the swizzle flips bit 2 of the chunk position, i.e. byte bit 6, and the row adds 512 bytes).
+    // The addresses follow the buffer of the head in hand.
+    unsigned xo[4];
+    {
+        const int kk = 8 * lg + (lr >> 2);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xo[j] = sbase + S16_XR + tile64_tr_offset(kk, s16_col(j, 4 * (lr & 3)));
+    }
     const int cq = 8 * lg;                         // first of this lane's eight columns inside a 32-column half
-    const bool need_d = p.has_D;
-    // operands of all row tiles first (the D term's rows - forward: x, mirror: dy - from the raw tile; z resp. x from memory)
-    Vec16<T> kx[QT][2], g2[QT][2];
-    const bool want2 = BWD || p.has_z;
+
+    auto cb_at = [&](int s, int col) __attribute__((always_inline)) { return (float)__builtin_bit_cast(half2_t, cbh[s][col >> 1])[col & 1]; };
+    int r_lane = r_own;
+    for (int hi = 0; hi < hpw; ++hi) {
+        int h = h0 + hi;
+        // (opaque: seen as a function of the loop counter, the head's base addresses become per-lane running pointers)
+        asm volatile("" : "+s"(h));
+        const int cur = hi & 1;
+        // What does not change from head to head (the packed CB entries, the lane's row) is made opaque here: hoisted out of
+        // the loop, the unpacked entries and the diagonal steps' comparison masks would take a few hundred registers.
 #pragma unroll
-    for (int rt = 0; rt < QT; ++rt) {
-        if (wr0 + rt * 16 >= limit) break;         // (uniform) the whole row tile lies behind the end of the sequence
-        const int rc = min(wr0 + rt * 16 + lr, limit - 1);
-        if (need_d || BWD) {
+        for (int s = 0; s < NSTEP; ++s)
 #pragma unroll
-            for (int t = 0; t < 2; ++t) kx[rt][t] = *reinterpret_cast<const Vec16<T> *>(reinterpret_cast<const char *>(xr) + tile64_row_offset(rc, t * 32 + cq));
+            for (int k = 0; k < 4; ++k) asm volatile("" : "+v"(cbh[s][k]));
+        asm volatile("" : "+v"(r_lane));
+        asm volatile("" : "+v"(tab_l));
+        asm volatile("" : "+v"(g_l));
+        asm volatile("" : "+v"(m_l));
+        int wr0_l = wr0;
+        asm volatile("" : "+s"(wr0_l));
+        unsigned sb = sbase;                       // (addresses used once per head are rebuilt from this, not kept across the loop)
+        asm volatile("" : "+s"(sb));
+        // From here to the end of the loop every LDS access is a raw one (the compiler makes an LDS access it knows of, and a
+        // register it believes a load still owes, wait for EVERY vector memory operation in flight: the requests below and
+        // the previous head's output stores, which are meant to drain while this head is worked on), and there is no global
+        // load besides the requests.
+        // ---- requests: this head's z (resp. x) rows, each wave its own 16; the next head's operands go out during the K
+        // loop, four parts at the first four steps (waves without rows in the chunk have no K loop: theirs go out here)
+        const bool more = hi + 1 < hpw;
+        int hn = h + 1;
+        asm volatile("" : "+s"(hn));
+        if (more && !active) request_head(hn, cur ^ 1);
+        if (BWD || p.has_z) {
+            const char *row2 = uniform_ptr(
+                BWD ? reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh + p0
+                    : reinterpret_cast<const T *>(p.z) + b * p.z_sb + (int64_t)c * Q * p.z_sl + h * p.z_sh + p0);
+            if (active) {
+                int ln = lane;
+                asm volatile("" : "+v"(ln));
+                load16_to_lds_at(row2, tile_off(ln, 0, s2_bytes), smem + S16_KT + wave * 2048);
+                load16_to_lds_at(row2, tile_off(ln, 1, s2_bytes), smem + S16_KT + wave * 2048 + 1024);
+            }
         }
-        if (want2) {
-            const T *row2 = BWD ? reinterpret_cast<const T *>(p.x) + b * p.x_sb + ((int64_t)c * Q + rc) * p.x_sl + h * p.x_sh
-                                : reinterpret_cast<const T *>(p.z) + b * p.z_sb + ((int64_t)c * Q + rc) * p.z_sl + h * p.z_sh;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) g2[rt][t] = *reinterpret_cast<const Vec16<T> *>(row2 + p0 + cq + t * 32);
+        // ---- tables of this head
+        // forward: k<r uses lo[r]-lo[k] with lo = cs_f, k>r uses up[r]-up[k] with up = cs_b
+        // mirror : k<r uses e^{cs_b[k]-cs_b[r]} -> lo = -cs_b;  k>r uses e^{cs_f[k]-cs_f[r]} -> up = -cs_f
+        // Away from the diagonal the factor separates: with m = lo at the last position of k's block of 16 (which lies
+        // between k and r), 2^{lo[r]-lo[k]} = 2^{lo[r]-m} * glo[k], glo[k] = 2^{m-lo[k]}, both factors <= 1 for A <= 0;
+        // likewise gup[k] = 2^{up[first of k's block] - up[k]}.  The column factors also carry dt[k] (forward) and the zero
+        // of the rows behind the end of the sequence, which the raw tile holds as copies of its last row.
+        const unsigned raw_a = sb + S16_RAW + cur * 3072;        // cs_f +0, cs_b +1024, dt +2048
+        if (threadIdx.x < S16_ROWS) {
+            int q = threadIdx.x;
+            asm volatile("" : "+v"(q));             // (the addresses below are rebuilt per head, not kept across the loop)
+            const int qq = min(q, Q - 1), qe = min(q | 15, Q - 1), qs = min(q & ~15, Q - 1);
+            float f = raw_lds_read_at<float, 0>(raw_a + qq * 4), r = raw_lds_read_at<float, 1024>(raw_a + qq * 4);
+            float fe = BWD ? raw_lds_read_at<float, 1024>(raw_a + qe * 4) : raw_lds_read_at<float, 0>(raw_a + qe * 4);
+            float rs = BWD ? raw_lds_read_at<float, 0>(raw_a + qs * 4) : raw_lds_read_at<float, 1024>(raw_a + qs * 4);
+            float dtq = BWD ? 1.f : raw_lds_read_at<float, 2048>(raw_a + qq * 4);
+            raw_lds_wait();
+            raw_lds_use(f); raw_lds_use(r); raw_lds_use(fe); raw_lds_use(rs); raw_lds_use(dtq);
+            f *= LOG2E; r *= LOG2E;
+            fe *= BWD ? -LOG2E : LOG2E; rs *= BWD ? -LOG2E : LOG2E;
+            if (q >= limit) dtq = 0.f;
+            const float l = BWD ? -r : f, u = BWD ? -f : r;
+            const unsigned ta = sb + S16_TAB + q * 4;
+            raw_lds_write_at<0>(ta, l);
+            raw_lds_write_at<1024>(ta, u);
+            raw_lds_write_at<4096>(ta, dtq);
+            // the column factors as float16, scaled by a power of two per block of 16 (this thread's 16-lane row) that brings
+            // the block's largest one into [0.5, 1) (the scaled CB entries stay below 2^15, so the products stay finite): the K loop multiplies them onto the float16 CB entries two at a time.
+            // The block's exponent goes into its reference point, i.e. into the row factor.
+            const float gl = __builtin_amdgcn_exp2f(fe - l) * dtq, gu = __builtin_amdgcn_exp2f(rs - u) * dtq;
+            const unsigned exl = (__float_as_uint(row16_max(gl)) >> 23) & 255u, exu = (__float_as_uint(row16_max(gu)) >> 23) & 255u;
+            const bool okl = exl > 0 && exl < 254, oku = exu > 0 && exu < 254;       // (zero or denormal maximum: left as it is)
+            const _Float16 hl = (_Float16)(okl ? gl * __uint_as_float((253u - exl) << 23) : gl);
+            const _Float16 hu = (_Float16)(oku ? gu * __uint_as_float((253u - exu) << 23) : gu);
+            const unsigned tg = sb + S16_TAB + q * 2;
+            raw_lds_write16_at<2048>(tg, hl);
+            raw_lds_write16_at<3072>(tg, hu);
+            if ((q & 15) == 0) {
+                const unsigned tm = sb + S16_TAB + (q >> 4) * 4;
+                raw_lds_write_at<2048 + 512>(tm, fe - (okl ? (float)((int)exl - 126) : 0.f));
+                raw_lds_write_at<3072 + 512>(tm, rs - (oku ? (float)((int)exu - 126) : 0.f));
+            }
         }
-    }
-    float dtr[QT];                                 // mirror: dt of this lane's rows
-    if (BWD) {
-#pragma unroll
-        for (int rt = 0; rt < QT; ++rt) dtr[rt] = dto[min(wr0 + rt * 16 + lr, Q - 1)];
-    }
-    float dcol[2][8];                              // D of this lane's columns
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) dcol[t][e] = d_head;
-        if (p.has_D && p.D_has_hdim) {
-            const float4 d0 = *reinterpret_cast<const float4 *>(p.D + h * P + p0 + t * 32 + cq), d1 = *reinterpret_cast<const float4 *>(p.D + h * P + p0 + t * 32 + cq + 4);
-            dcol[t][0] = d0.x; dcol[t][1] = d0.y; dcol[t][2] = d0.z; dcol[t][3] = d0.w;
-            dcol[t][4] = d1.x; dcol[t][5] = d1.y; dcol[t][6] = d1.z; dcol[t][7] = d1.w;
+        // mirror: the far ends of the chunk and dt of this lane's row
+        float e_f = 0.f, e_b = 0.f;
+        if (BWD) {
+            e_f = raw_lds_read_at<float, 0>(raw_a + (Q - 1) * 4);
+            e_b = raw_lds_read_at<float, 1024>(raw_a);
+            raw_lds_wait();
+            raw_lds_use(e_f); raw_lds_use(e_b);
+            e_f *= LOG2E; e_b *= LOG2E;
         }
-    }
+        raw_lds_wait();
+        raw_lds_barrier();                         // #1: the tables are there (everybody's requests for this head landed before #2)
+
+        f32x4 acc[4];
+        if (active) {
+            float lor = raw_lds_read_at<float, 0>(tab + r_own * 4), upr = raw_lds_read_at<float, 1024>(tab + r_own * 4);
+            // ---- part 1: states.  D[p][r] = sum_n S[p][n] Own[r][n], scaled by this lane's row factor, one direction after the other
 #pragma unroll
-    for (int rt = 0; rt < QT; ++rt) {
-        if (wr0 + rt * 16 >= limit) break;
-        const int r = wr0 + rt * 16 + lr, rc = min(r, limit - 1);
-        const bool live = r < limit;
-        const int64_t orow = (((int64_t)b * p.seqlen + (int64_t)c * Q + rc) * H + h) * P + p0 + cq;
-        float rsum = 0.f;
+            for (int dir = 0; dir < (UNI ? 1 : 2); ++dir) {
+                f32x4 tmp[4];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            float a[8];
+                for (int j = 0; j < 4; ++j) tmp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int e = 0; e < 8; ++e) a[e] = acc[rt][2 * t + (e >> 2)][e & 3];
-            if (!BWD) {
-                if (need_d) {
+                for (int jj = 0; jj < 4; jj += 2) {
+                    Frag sf[2][2];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) a[e] = __builtin_fmaf(dcol[t][e], to_f(kx[rt][t].v[e]), a[e]);
-                }
-                if (p.has_z) {
-                    if (p.out_x && live) {
-                        Vec16<T> ox;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) ox.v[e] = from_f<T>(a[e]);
-                        *reinterpret_cast<Vec16<T> *>(reinterpret_cast<T *>(p.out_x) + orow + t * 32) = ox;
+                    for (int j = 0; j < 2; ++j) {
+                        // row s16_col(jj + j, lr) of the tile, chunk (4 s + lg) ^ (row % 8)
+                        const int pr = s16_col(jj + j, lr);
+                        const unsigned ra = sbase + S16_ST + (cur * 2 + dir) * 8192 + pr * 128;
+                        sf[j][0] = raw_lds_read_at<Frag, 0>(ra + ((lg ^ (pr & 7)) << 4));
+                        sf[j][1] = raw_lds_read_at<Frag, 0>(ra + (((4 + lg) ^ (pr & 7)) << 4));
                     }
+                    raw_lds_wait();
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) a[e] *= silu_f(to_f(g2[rt][t].v[e]));
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int s = 0; s < 2; ++s) {
+                            raw_lds_use(sf[j][s]);
+                            tmp[jj + j] = M::mma(sf[j][s], own[s], tmp[jj + j]);
+                        }
                 }
-                if (live) {
+                raw_lds_use(lor); raw_lds_use(upr);
+                // forward: e^{cs_f[r]} = 2^{lo[r]}, e^{cs_b[r]} = 2^{up[r]}; mirror: e^{cs_f[Q-1]-cs_f[r]} = 2^{e_f+up[r]}, e^{cs_b[0]-cs_b[r]} = 2^{e_b+lo[r]}
+                const float e = __builtin_amdgcn_exp2f(BWD ? (dir ? e_b + lor : e_f + upr) : (dir ? upr : lor));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = dir ? tmp[j] * e + acc[j] : tmp[j] * e;
+            }
+            // ---- part 2: inside the chunk.  Per K step of 32 columns: CB (resp. CB^T) times the decay factors, times the K operand
+            auto k_step = [&](auto STEP) __attribute__((always_inline)) -> bool {
+                constexpr int step = decltype(STEP)::value;
+                if (step < 4 && more) request_part(hn, cur ^ 1, step);
+                if (step >= nsteps) return true;
+                constexpr int k0 = step * KSTEP;
+                // the wave's rows [wr0, wr0 + 16) meet the step's columns [k0, k0 + 32) in one step only
+                const int cls = (k0 + KSTEP - 1 < wr0_l) ? 0 : (k0 > wr0_l + 15) ? 1 : 2;   // below, above, across the diagonal
+                if (UNI && cls == (BWD ? 0 : 1)) return true;                              // far side of the diagonal
+                constexpr int TB = step * (KSTEP * 4);     // byte offset of the step inside the float tables
+                Frag af;
+                if (cls != 2) {
+                    const unsigned sel = cls == 0 ? 0u : 1024u;
+                    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+                    u32x4 gq = raw_lds_read_at<u32x4, step * 64>(g_l + sel);
+                    float mref = raw_lds_read_at<float, step * 8>(m_l + sel);
+                    raw_lds_wait();
+                    raw_lds_use(gq); raw_lds_use(mref);
+                    const float rf = __builtin_amdgcn_exp2f((cls == 0 ? lor : upr) - mref) * cb_unscale;
+                    float v[8];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        // two entries times their column factors in float16, then each times the row factor in float32
+                        // (vector element copied to a scalar first: __builtin_bit_cast applied to the element itself reads element 0)
+                        const unsigned gk = gq[k];
+                        const half2_t t = __builtin_bit_cast(half2_t, cbh[step][k]) * __builtin_bit_cast(half2_t, gk);
+                        v[2 * k] = __builtin_fmaf((float)t[0], rf, 0.f);
+                        v[2 * k + 1] = __builtin_fmaf((float)t[1], rf, 0.f);
+                    }
+                    af = M::pack(v);
+                } else {
+                    // the one step across the diagonal: element by element, four columns at a time
+                    const unsigned la = tab_l;
+                    const int kb = k0 + lg * 8;
+                    float v[8];
+#pragma unroll
+                    for (int hh = 0; hh < 2; ++hh) {
+                        f32x4 l0 = hh ? raw_lds_read_at<f32x4, TB + 16>(la) : raw_lds_read_at<f32x4, TB>(la);
+                        f32x4 u0 = hh ? raw_lds_read_at<f32x4, TB + 1024 + 16>(la) : raw_lds_read_at<f32x4, TB + 1024>(la);
+                        f32x4 d0 = hh ? raw_lds_read_at<f32x4, TB + 4096 + 16>(la) : raw_lds_read_at<f32x4, TB + 4096>(la);
+                        raw_lds_wait();
+                        raw_lds_use(l0); raw_lds_use(u0); raw_lds_use(d0);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int k = kb + hh * 4 + i;
+                            const float e = k < r_lane ? lor - l0[i] : upr - u0[i];
+                            float w = (k == r_lane) ? (UNI ? 1.f : 2.f) : __builtin_amdgcn_exp2f(e);
+                            if (UNI && (BWD ? k < r_lane : k > r_lane)) w = 0.f;
+                            v[hh * 4 + i] = cb_at(step, hh * 4 + i) * (w * d0[i] * cb_unscale);
+                        }
+                    }
+                    af = M::pack(v);
+                }
+                // ---- the product with the K operand, transposed: D[p][r] += X[k][p] A[r][k]; two column tiles at a time
+                constexpr int XS = step * (KSTEP * 128);
+#pragma unroll
+                for (int jj = 0; jj < 4; jj += 2) {
+                    const i16x4 a0 = raw_lds_tr16_read_at<XS>(xo[jj]), a1 = raw_lds_tr16_read_at<XS + 512>(xo[jj] ^ 64u);
+                    const i16x4 b0 = raw_lds_tr16_read_at<XS>(xo[jj + 1]), b1 = raw_lds_tr16_read_at<XS + 512>(xo[jj + 1] ^ 64u);
+                    raw_lds_wait();
+                    i16x8 fa = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7), fb = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
+                    raw_lds_use(fa); raw_lds_use(fb);
+                    acc[jj] = M::mma(__builtin_bit_cast(Frag, fa), af, acc[jj]);
+                    acc[jj + 1] = M::mma(__builtin_bit_cast(Frag, fb), af, acc[jj + 1]);
+                }
+                return true;
+            };
+            static_for<0, NSTEP>(k_step);
+        }
+        // this wave's z (resp. x) rows have landed: everything but the requests for the next head, which are younger
+        if (!more) wait_vmcnt<0>();
+        else if (head_requests == 2) wait_vmcnt<2>();
+        else if (head_requests == 3) wait_vmcnt<3>();
+        else wait_vmcnt<4>();
+        // ---- epilogue.  acc[2t][i], acc[2t+1][i] = row wr0 + lr, headdim columns p0 + 32 t + 8 lg + i, + 4 + i ----
+        f32x4 res_a[2], res_b[2];                  // packed results of the two column halves: out / dx, and out_x
+        float rsum = 0.f;
+        const bool live = r_own < limit;
+        if (active) {
+            const bool need_d = p.has_D;
+            const unsigned d_a = sb + S16_DT + hi * 256 + cq * 4;
+            float dtr = 0.f;                       // mirror: dt of this lane's row
+            if (BWD) dtr = raw_lds_read_at<float, 2048>(raw_a + min(r_lane, Q - 1) * 4);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                // the D term's row (forward: x, mirror: dy) from the raw tile, z (resp. x) from the rows this wave brought
+                const unsigned eo = sb + tile64_row_offset(min(r_lane, limit - 1), t * 32 + cq);
+                f32x4 kx4 = {0.f, 0.f, 0.f, 0.f}, g24 = {0.f, 0.f, 0.f, 0.f}, d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+                if (need_d || BWD) kx4 = raw_lds_read_at<f32x4, S16_XR>(eo + cur * 32768);
+                if (BWD || p.has_z) g24 = raw_lds_read_at<f32x4, 0>(eo + S16_KT);
+                if (need_d) {
+                    d0 = t ? raw_lds_read_at<f32x4, 128>(d_a) : raw_lds_read_at<f32x4, 0>(d_a);
+                    d1 = t ? raw_lds_read_at<f32x4, 144>(d_a) : raw_lds_read_at<f32x4, 16>(d_a);
+                }
+                raw_lds_wait();
+                raw_lds_use(kx4); raw_lds_use(g24); raw_lds_use(d0); raw_lds_use(d1);
+                const Vec16<T> kx = __builtin_bit_cast(Vec16<T>, kx4), g2 = __builtin_bit_cast(Vec16<T>, g24);
+                const float dcol[8] = {d0[0], d0[1], d0[2], d0[3], d1[0], d1[1], d1[2], d1[3]};
+                float a[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a[e] = acc[2 * t + (e >> 2)][e & 3];
+                if (!BWD) {
+                    if (need_d) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) a[e] = __builtin_fmaf(dcol[e], to_f(kx.v[e]), a[e]);
+                    }
+                    if (p.has_z) {
+                        if (p.out_x) {
+                            Vec16<T> ox;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) ox.v[e] = from_f<T>(a[e]);
+                            res_b[t] = __builtin_bit_cast(f32x4, ox);
+                        }
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) a[e] *= silu_f(to_f(g2.v[e]));
+                    }
                     Vec16<T> ov;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) ov.v[e] = from_f<T>(a[e]);
-                    // out is not read again by any kernel of the pass: past the caches
-                    __builtin_nontemporal_store(__builtin_bit_cast(f32x4, ov), reinterpret_cast<f32x4 *>(reinterpret_cast<T *>(p.out) + orow + t * 32));
-                }
-            } else {
-                Vec16<T> ov;
+                    res_a[t] = __builtin_bit_cast(f32x4, ov);
+                } else {
+                    Vec16<T> ov;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float xv = to_f(g2[rt][t].v[e]), yv = to_f(kx[rt][t].v[e]);
-                    rsum = __builtin_fmaf(a[e], xv, rsum);
-                    float dxv = a[e] * dtr[rt];
-                    if (need_d) dxv = __builtin_fmaf(dcol[t][e], yv, dxv);
-                    ov.v[e] = from_f<T>(dxv);
-                    // dD: kept in the accumulator's place (it is dead from here on); rows behind the end count nothing
-                    acc[rt][2 * t + (e >> 2)][e & 3] = live ? yv * xv : 0.f;
+                    for (int e = 0; e < 8; ++e) {
+                        const float xv = to_f(g2.v[e]), yv = to_f(kx.v[e]);
+                        rsum = __builtin_fmaf(a[e], xv, rsum);
+                        float dxv = a[e] * dtr;
+                        if (need_d) dxv = __builtin_fmaf(dcol[e], yv, dxv);
+                        ov.v[e] = from_f<T>(dxv);
+                        // dD: kept in the accumulator's place (it is dead from here on); rows behind the end count nothing
+                        acc[2 * t + (e >> 2)][e & 3] = live ? yv * xv : 0.f;
+                    }
+                    res_a[t] = __builtin_bit_cast(f32x4, ov);
                 }
-                if (live) __builtin_nontemporal_store(__builtin_bit_cast(f32x4, ov), reinterpret_cast<f32x4 *>(reinterpret_cast<T *>(p.dx) + orow + t * 32));
             }
         }
-        if (BWD) {
-            // the four lanes lr, lr + 16, lr + 32, lr + 48 hold the four column groups of a row
-            rsum += __shfl_xor(rsum, 16, 64);
-            rsum += __shfl_xor(rsum, 32, 64);
-            if (lg == 0 && live) {
-                if (npt == 1) p.ddt_direct[o + r] = rsum;
-                else atomicAdd(p.ddt_direct + o + r, rsum);   // several headdim tiles share a row
+        // The next head's operands (this wave's share) have landed; waited for here, in front of this head's stores: a wait
+        // behind them would be for the stores as well.
+        wait_vmcnt<0>();
+        if (active) {
+            // output rows: uniform base of the (chunk, head) + this lane's row and column group
+            int hh = h;
+            asm volatile("" : "+s"(hh));            // (addresses are built here, not kept from the top of the loop)
+            const int64_t obase = (((int64_t)b * p.seqlen + (int64_t)c * Q) * H + hh) * P + p0;
+            const unsigned orow = (unsigned)min(r_lane, limit - 1) * (unsigned)(H * P) + cq;
+            if (live) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    if (!BWD && p.has_z && p.out_x) *reinterpret_cast<f32x4 *>(reinterpret_cast<T *>(p.out_x) + obase + (orow + t * 32)) = res_b[t];
+                    // out (resp. dx) is not read again by any kernel of the pass: past the caches
+                    __builtin_nontemporal_store(res_a[t], reinterpret_cast<f32x4 *>(reinterpret_cast<T *>(BWD ? p.dx : p.out) + obase + (orow + t * 32)));
+                }
+            }
+            if (BWD) {
+                // the four lanes lr, lr + 16, lr + 32, lr + 48 hold the four column groups of a row
+                // (lane indices rebuilt here: kept from the prologue's shuffles they would be spilled)
+                int ln = lane;
+                asm volatile("" : "+v"(ln));
+                rsum += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((ln ^ 16) << 2, __builtin_bit_cast(int, rsum)));
+                rsum += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((ln ^ 32) << 2, __builtin_bit_cast(int, rsum)));
+                if (lg == 0 && live) {
+                    float *dst = p.ddt_direct + ((((int64_t)b * H + hh) * nc + c) * Q + r_lane);
+                    if (npt == 1) *dst = rsum;
+                    else atomicAdd(dst, rsum);   // several headdim tiles share a row
+                }
             }
         }
-    }
-    if (BWD && p.has_D) {
-        // dD partial of this (b, c, h): column sums of dy * x over the rows; a lane holds columns s16_col(j, 4 lg + i) of the
-        // rows lr (+16): add the row tiles, then the 16 lanes of a row group, then the waves
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float v = 0.f;
-#pragma unroll
-                for (int rt = 0; rt < QT; ++rt)
-                    if (wr0 + rt * 16 < limit) v += acc[rt][j][i];
-                v = row16_sum(v);
-                if (lr == 0) red[wave][s16_col(j, 4 * lg + i)] = v;
-            }
-        __syncthreads();
-        if (threadIdx.x < 64) {
+        if (BWD && p.has_D) {
+            // dD partial of this (b, c, h): column sums of dy * x over the rows; a lane holds columns s16_col(j, 4 lg + i) of
+            // row lr: add the 16 lanes of a row group, then the waves
+            const unsigned red_a = sb + S16_RED + (wave * 64 + 8 * lg) * 4;
+            static_for<0, 16>([&](auto JI) __attribute__((always_inline)) {
+                constexpr int j = decltype(JI)::value >> 2, i = decltype(JI)::value & 3;
+                const float v = row16_sum(active ? acc[j][i] : 0.f);
+                if (lr == 0) raw_lds_write_at<s16_col(j, i) * 4>(red_a, v);   // s16_col(j, 4 lg + i) = s16_col(j, i) + 8 lg
+                return true;
+            });
+        }
+        // #2: everybody is done with this head's tiles, tables and z rows (a bare barrier: the stores just issued need not
+        // have completed)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        raw_lds_barrier();
+        if (BWD && p.has_D && threadIdx.x < 64) {
+            float pv[S16_WAVES];
+            const unsigned red_a = sb + S16_RED + threadIdx.x * 4;
+            static_for<0, S16_WAVES>([&](auto WV) __attribute__((always_inline)) {
+                pv[decltype(WV)::value] = raw_lds_read_at<float, decltype(WV)::value * 256>(red_a);
+                return true;
+            });
+            raw_lds_wait();
             float v = 0.f;
 #pragma unroll
-            for (int wv = 0; wv < S16_WAVES; ++wv) v += red[wv][threadIdx.x];
+            for (int wv = 0; wv < S16_WAVES; ++wv) { raw_lds_use(pv[wv]); v += pv[wv]; }
             p.red[((int64_t)(b * nc + c) * H + h) * P + p0 + threadIdx.x] = v;   // partials [(b, c)][h][P]
         }
+        // the fragment addresses move on to the other buffer
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xo[j] = cur ? xo[j] - 32768u : xo[j] + 32768u;
     }
+}
+
+// heads a workgroup of the kernel above walks through: the largest divisor of the heads per group that is <= S16_MAX_HEADS
+static int scan16_heads_per_block(const bimamba2_params *p) {
+    const int hpg = p->nheads / p->ngroups;
+    for (int k = S16_MAX_HEADS; k > 1; --k)
+        if (hpg % k == 0) return k;
+    return 1;
 }
 
 // Launches the kernel above; the caller (launch_chunk_scan) has checked that the problem is one of its shapes:
 // scan_recomputes_cb(), 16-bit copies of the entering states present and 16-byte aligned.
 template <typename T, bool BWD>
 static int launch_scan16_t(const bimamba2_params *p, int nc) {
-    const int npt = p->headdim / 64;
-    dim3 grid(p->batch * nc * p->nheads * npt);
+    const int npt = p->headdim / 64, hpw = scan16_heads_per_block(p);
+    dim3 grid(p->batch * nc * (p->nheads / hpw) * npt);
     hipStream_t s = reinterpret_cast<hipStream_t>(p->stream);
-    const bool one = p->chunk_size <= 128;
-#define BM2_S16(QTV, UNIV) hipLaunchKernelGGL((chunk_scan16_kernel<T, QTV, BWD, UNIV>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt)
-    if (p->causal) { if (one) BM2_S16(1, true); else BM2_S16(2, true); }
-    else { if (one) BM2_S16(1, false); else BM2_S16(2, false); }
-#undef BM2_S16
+    if (p->causal) hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, true>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
+    else hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, false>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
     return check_launch();
 }
 
@@ -458,3 +655,4 @@ int launch_chunk_scan16(const bimamba2_params *p, bool bwd) {
 }
 
 }  // namespace bm2
+

@@ -92,12 +92,12 @@ def test_backward_with_recomputation(ops, case, monkeypatch):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_sixteen_bit_state_copies_change_nothing_but_the_chunk_decay_gradient(ops, dtype):
+def test_sixteen_bit_state_copies_against_float32_states(ops, dtype):
     """Where the kernels can, the composites keep the states entering the chunks (and their gradients) in copies of the
-    input's 16-bit type instead of float32.  Every kernel that reads them rounded them to that type for its MFMA before,
-    so out, dx, dz, dB and dC must come out bit for bit as with float32 states; only the gradient of the chunk decays
-    (a float32 dot product with the entering states inside the backward state passing, which feeds ddt and dA) sees
-    the rounding.  The float32 side: forward with the states returned as tensors, which switches the copies off."""
+    input's 16-bit type instead of float32, and the scan kernels that know the copies run.  Every kernel that reads the
+    entering states rounds them to that type for its MFMA anyway, so both ways must agree within the tolerance of the type
+    (different kernels with different rounding points: not bit for bit).  The float32 side: forward with the states returned as tensors, which switches
+    the copies off."""
     import ctypes
     from bi_mamba2_amd import _lib
     Q = 256
@@ -115,15 +115,14 @@ def test_sixteen_bit_state_copies_change_nothing_but_the_chunk_decay_gradient(op
     res_c = ops._mamba_chunk_scan_combined_fwd(*args, **kw, return_intermediates=False, keep_for_bwd=True)
     assert res_c[9][2][3] == ops._BLOB_FIELDS_COPIES
     res_f = ops._mamba_chunk_scan_combined_fwd(*args, **kw, return_intermediates=True, keep_for_bwd=True)
-    assert torch.equal(res_c[0], res_f[0]) and torch.equal(res_c[1], res_f[1])
+    # (two 16-bit results against each other, each with its own rounding: absolute tolerance in units of the RMS)
+    assert_close(res_c[0], res_f[0].double(), dtype, "out", scaled=True)
+    assert_close(res_c[1], res_f[1].double(), dtype, "out_x", scaled=True)
     g_c = ops._mamba_chunk_scan_combined_bwd(dout, *args[:5], res_c[1], Q, **kw, saved=res_c[9])
     g_f = ops._mamba_chunk_scan_combined_bwd(dout, *args[:5], res_f[1], Q, **kw, saved=res_f[9])
     names = ("dx", "ddt", "dA", "dB", "dC", "dD", "dz", "ddt_bias")
     for name, a, b in zip(names, g_c, g_f):
-        if name in ("ddt", "dA", "ddt_bias"):
-            assert_close(a, b.double(), dtype, name, scaled=True)
-        else:
-            assert torch.equal(a, b), name
+        assert_close(a, b.double(), dtype, name, scaled=True)
 
 
 def test_backward_takes_a_misaligned_gradient_view(ops):
