@@ -183,14 +183,32 @@ def make_inputs(batch, seqlen, nheads, headdim, ngroups, dstate, dtype, with_z, 
     return dict(x=x, dt=dt, A=A, B=B, C=C, D=D, z=z, dt_bias=dt_bias)
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(w, budget_s=15.0):
     """The oracle's naive flip-and-sum path (chunked causal SSD twice) in float32 PyTorch on the host cores,
-    forward + backward, on one batch row of the same workload, repeated for about 15 s."""
+    forward + backward, on one batch row of the same workload, repeated for about 15 s.  Threads: the cores this process
+    may use - its affinity mask, capped by OMP_NUM_THREADS where the machine's operator sets it (a GPU's share of a
+    multi-GPU host; os.cpu_count() counts the whole host) - all three numbers are reported."""
     import torch
     from oracle import bimamba2_oracle as O
 
-    cores = min(16, os.cpu_count() or 1)
-    torch.set_num_threads(cores)
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    cap = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    torch.set_num_threads(min(usable, cap) if cap > 0 else usable)
+    cores = torch.get_num_threads()
     heads = w["nheads"]
     inp = make_inputs(1, w["seqlen"], heads, w["headdim"], 1, w["dstate"], torch.float32, True)
 
@@ -211,8 +229,138 @@ def cpu_baseline(w, budget_s=15.0):
     med = times[len(times) // 2]
     value = w["seqlen"] / med / 1e6
     return {"value": value, "unit": "Mtokens/s", "cores": cores, "kind": "port",
+            "os_cpu_count": os.cpu_count(), "affinity_cores": usable, "omp_num_threads_env": cap or None,
+            "torch_num_threads": cores, "cpu_model": cpu_model(),
             "sample": f"batch 1 (of {w['batch']}) x seqlen {w['seqlen']} x {heads} heads, float32, fwd+bwd via autograd, "
                       f"median of {len(times)} runs = {med * 1e3:.1f} ms"}
+
+
+# The other benchmark configurations (the headline stays WORKLOAD): name -> (shape, z gate, backward too)
+OTHER_CONFIGS = {
+    "config1_fwd": (dict(batch=4, seqlen=2048, nheads=32, headdim=64, ngroups=1, dstate=64, chunk_size=256), True, False),
+    "config2_fwd": (dict(batch=2, seqlen=16384, nheads=48, headdim=64, ngroups=1, dstate=128, chunk_size=256), False, False),
+    "config3_fwd_bwd": (dict(batch=4, seqlen=4096, nheads=32, headdim=64, ngroups=8, dstate=64, chunk_size=256), True, True),
+}
+
+
+def graphed(fn):
+    """fn recorded once into a HIP graph (torch.cuda.CUDAGraph); returns the replay callable."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    return graph.replay
+
+
+def timed(fn, n):
+    import torch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / n
+
+
+def config_line(name, dev, steps, warmup):
+    """One of the other configurations: forward (and backward) of the operator as a HIP graph replay, bf16, synthetic
+    inputs; ms per pass, tokens/s and the fraction of the HBM roofline on the operator's algorithmic bytes."""
+    import torch
+    from bi_mamba2_amd import ops
+    w, has_z, bwd = OTHER_CONFIGS[name]
+    dtype, e = torch.bfloat16, 2
+    inp = make_inputs(w["batch"], w["seqlen"], w["nheads"], w["headdim"], w["ngroups"], w["dstate"], dtype, has_z)
+    leaves = {k: (v.to(dev).requires_grad_(bwd) if v is not None else None) for k, v in inp.items()}
+    kw = dict(D=leaves["D"], z=leaves["z"], dt_bias=leaves["dt_bias"], dt_softplus=True)
+    args = (leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], w["chunk_size"])
+    if bwd:
+        dout = torch.randn(inp["x"].shape, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
+        grad_inputs = [v for v in leaves.values() if v is not None]
+
+        def fn():
+            torch.autograd.grad(ops.bimamba_chunk_scan_combined(*args, **kw), grad_inputs, dout)
+    else:
+        def fn():
+            with torch.no_grad():
+                ops.bimamba_chunk_scan_combined(*args, **kw)
+    replay = graphed(fn)
+    for _ in range(warmup):
+        replay()
+    t = timed(replay, steps)
+    fwd_b, bwd_b = whole_op_bytes(w, e, has_z)
+    nbytes = fwd_b + (bwd_b if bwd else 0)
+    tokens = w["batch"] * w["seqlen"]
+    return {"workload": {**w, "has_z": has_z, "dtype": "bf16"}, "pass": "fwd+bwd" if bwd else "fwd",
+            "ms": round(t * 1e3, 4), "Mtokens_s": round(tokens / t / 1e6, 2), "alg_MB": round(nbytes / 1e6, 1),
+            "hbm_roofline_us": round(nbytes / (HBM_PEAK_GBS * 1e9) * 1e6, 1),
+            "hbm_frac": round(nbytes / t / (HBM_PEAK_GBS * 1e9), 4)}
+
+
+def layer_line(dev, steps, warmup):
+    """The BiMamba2 layer (in_proj GEMM, non-causal depthwise conv + SiLU, the bidirectional SSD, gated RMSNorm, out_proj
+    GEMM) forward + backward at batch 16 x seqlen 1024, d_model 768, bf16, weights as the constructor draws them; and
+    the operator alone at the layer's shape, for its share."""
+    import torch
+    from bi_mamba2_amd import ops
+    from bi_mamba2_amd.modules import BiMamba2
+    torch.manual_seed(0)
+    dtype = torch.bfloat16
+    m = BiMamba2(d_model=768, d_state=64, d_conv=7, expand=2, headdim=64, ngroups=1, chunk_size=256).to(dev).to(dtype)
+    u = torch.randn(16, 1024, 768, device=dev, dtype=dtype, requires_grad=True)
+    dy = torch.randn(16, 1024, 768, device=dev, dtype=dtype)
+    params = [p for n, p in m.named_parameters() if n != "fc_D.weight"]
+
+    def step():
+        torch.autograd.grad(m(u), [u] + params, dy)
+
+    def fwd():
+        with torch.no_grad():
+            m(u)
+    for _ in range(warmup):
+        step()
+    t_eager = timed(step, steps)
+    launch = "eager"
+    t = t_eager
+    try:
+        replay = graphed(step)
+        for _ in range(warmup):
+            replay()
+        t, launch = timed(replay, steps), "HIP graph replay"
+    except RuntimeError as exc:
+        sys.stderr.write(f"bench.py: the layer step was not captured ({exc}); reporting the eager step\n")
+    for _ in range(warmup):
+        fwd()
+    t_fwd = timed(fwd, steps)
+    # the operator alone at the layer's shape
+    w = dict(batch=16, seqlen=1024, nheads=24, headdim=64, ngroups=1, dstate=64, chunk_size=256)
+    inp = make_inputs(w["batch"], w["seqlen"], w["nheads"], w["headdim"], 1, w["dstate"], dtype, False)
+    leaves = {k: (v.to(dev).requires_grad_(True) if v is not None else None) for k, v in inp.items()}
+    dout = torch.randn(inp["x"].shape, generator=torch.Generator().manual_seed(1)).to(dtype).to(dev)
+    gi = [v for v in leaves.values() if v is not None]
+
+    def op_step():
+        out = ops.bimamba_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], 256,
+                                              D=leaves["D"], dt_bias=leaves["dt_bias"], dt_softplus=True)
+        torch.autograd.grad(out, gi, dout)
+    op_replay = graphed(op_step)
+    for _ in range(warmup):
+        op_replay()
+    t_op = timed(op_replay, steps)
+    tokens = 16 * 1024
+    return {"workload": "BiMamba2 layer fwd+bwd: batch 16 x seqlen 1024, d_model 768, d_state 64, d_conv 7, expand 2, "
+                        "headdim 64 (24 heads), ngroups 1, chunk 256, bf16, random-init weights",
+            "launch": launch, "ms_per_step": round(t * 1e3, 4), "Mtokens_s": round(tokens / t / 1e6, 2),
+            "eager_ms_per_step": round(t_eager * 1e3, 4), "fwd_ms": round(t_fwd * 1e3, 4),
+            "operator_ms_per_step": round(t_op * 1e3, 4), "operator_share": round(t_op / t, 3),
+            "rest": "in_proj / out_proj GEMMs (torch, hipBLASLt), conv1d + SiLU and gated RMSNorm (this library's kernels), "
+                    "splits and the dt_bias / A_log parameter maps (torch)"}
 
 
 def main():
@@ -224,7 +372,10 @@ def main():
     ap.add_argument("--no-z", action="store_true", help="benchmark without the z gate")
     ap.add_argument("--eager", action="store_true", help="time the eagerly launched step instead of its HIP graph replay")
     ap.add_argument("--no-extras", action="store_true",
-                    help="skip the causal comparator and the layer's norm / conv legs (keeps a profile of the run to the operator)")
+                    help="skip the causal comparator, the other configurations and the layer's legs (keeps a profile of the run to "
+                         "the operator)")
+    ap.add_argument("--config", choices=["target"] + sorted(OTHER_CONFIGS) + ["layer_config4"], default="target",
+                    help="target (default): the headline workload with every leg; another name: only that configuration's leg")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build measures the operator on ONE GPU; --gpus must be 1 "
@@ -237,6 +388,10 @@ def main():
     _lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    if args.config != "target":
+        line = layer_line(dev, args.steps, args.warmup) if args.config == "layer_config4" else config_line(args.config, dev, args.steps, args.warmup)
+        print(json.dumps({args.config: line}))
+        return
     w = WORKLOAD
     dtype, e = torch.bfloat16, 2
     has_z = not args.no_z
@@ -258,33 +413,11 @@ def main():
                                             w["chunk_size"], D=leaves["D"], z=leaves["z"], dt_bias=leaves["dt_bias"],
                                             dt_softplus=True)
 
-    def timed(fn, n):
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(n):
-            fn()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / n
-
     def causal_step():
         out = ops.causal_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"],
                                              w["chunk_size"], D=leaves["D"], z=leaves["z"], dt_bias=leaves["dt_bias"],
                                              dt_softplus=True)
         torch.autograd.grad(out, grad_inputs, dout)
-
-    def graphed(fn):
-        """fn recorded once into a HIP graph (torch.cuda.CUDAGraph); returns the replay callable."""
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(3):
-                fn()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            fn()
-        return graph.replay
 
     # The step is timed twice: launched eagerly through autograd (what a caller of the Python function gets; the host
     # needs 0.18-0.35 ms for it depending on the box, which is more than the GPU needs on the slower hosts), and recorded
@@ -448,9 +581,12 @@ def main():
             "ms_per_step": t_causal * 1e3, "Mtokens_s": tokens / t_causal / 1e6,
             "bidirectional_over_causal": t_step / t_causal,
             "what": "single-direction SSD (y = SS(x) + D x, z gate) forward + backward from the same kernels with the "
-                    "reverse direction compiled out, same shape and dtypes"}
+                    "reverse direction compiled out, same shape and dtypes; the scan kernels skip the K steps (and the "
+                    "reverse state tiles) the single direction does not use but still load the whole K-operand tile"}
         result["gated_rmsnorm"] = rmsnorm_line(w, dtype, dev, max(10, args.steps))
         result["conv1d_silu"] = conv_line(w, dtype, dev, max(10, args.steps))
+        result["configs"] = {name: config_line(name, dev, max(10, args.steps // 2), 3) for name in OTHER_CONFIGS}
+        result["layer_config4"] = layer_line(dev, max(10, args.steps // 2), 3)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(result))
