@@ -1196,12 +1196,7 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_kernel(const bimamba2_params
 #pragma unroll
                         for (int j = 0; j < 4; ++j) acc[j][i] = 0.f;
                     }
-#ifndef BM2_DBG_SKIPFIN
                 finish_head(it / nkc);
-#else
-#pragma unroll
-                for (int j = 0; j < 4; ++j) dcb[j] += acc[j];
-#endif
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
@@ -1277,11 +1272,6 @@ constexpr int DCB_SLOT_B = DCB_CS_OFF + 5 * 64 * 4;
 constexpr int DCB_PART_OFF = DCB_RING * DCB_SLOT_B;        // per-wave column sums (f: 0-3, b: 4-7), row sums (f: 8, b: 9)
 constexpr int DCB_PART_B = 10 * 64 * 4;
 
-#ifdef BM2_DBG_TIME
-#define TSR(k) do { long long _t = wall_clock64(); ph[k] += _t - tlast; tlast = _t; } while (0)
-#else
-#define TSR(k)
-#endif
 
 // UNI: the single-direction operator - tiles above the diagonal are empty, tiles on it keep the forward half.
 // bid / gdx / gdz: block index and grid extents (x: batch * chunks * groups, y: tiles, z: head slices)
@@ -1402,10 +1392,6 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
         }
         // settle these register loads here: inside the loop a wait for them would drain the ring's requests as well
         wait_vmcnt<0>();
-#ifdef BM2_DBG_TIME
-        long long ph[12] = {}, tlast = wall_clock64();
-        const long long tstart = tlast;
-#endif
         int slot = 0, slot2 = (DCB_RING - 1) % DCB_RING, kc = 0, par = 0;
         float *tv = tv0 + (wave & 1) * 64 + lane;
         // the sums of a head are written out one iteration later, after the barrier that the next step needs anyway
@@ -1446,7 +1432,6 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
             constexpr int KIND = decltype(KC)::value;
             constexpr bool DIAG = KIND >= 0;
         for (int it = 0; it < nit; ++it) {
-            TSR(0);
             // with two slots nothing but step `it` is outstanding here; with more, the requests of step `it` went out before
             // those of the step after it (waves 0 and 1 make five requests per step, the others four)
             if (DCB_RING > 2 && it + 1 < nit) {
@@ -1455,14 +1440,12 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
             } else {
                 wait_vmcnt<0>();
             }
-            TSR(1);
             raw_lds_barrier();     // step `it` has landed for everybody; every wave is done with the slot and the sums of step it - 1
             if (it + DCB_RING - 1 < nit) issue(slot2);
             if (pending) {
                 write_out(par ^ 1);
                 pending = false;
             }
-            TSR(2);
             const unsigned sb = sbase + slot * DCB_SLOT_B;
             Frag af[NKS], bf[4][NKS];
 #pragma unroll
@@ -1474,7 +1457,6 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                 bf[3][ks] = raw_lds_read_at<Frag, 6144>(sb + b_off[ks]);
             }
             raw_lds_wait();
-            TSR(3);
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
                 raw_lds_use(af[ks]);
@@ -1484,10 +1466,6 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                     acc[j] = M::mma(af[ks], bf[j][ks], acc[j]);
                 }
             }
-#ifdef BM2_DBG_TIME
-            asm volatile("" ::"v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3]));
-#endif
-            TSR(4);
             if (++kc == nkc) {
                 kc = 0;
                 // ---- decay vectors of this head
@@ -1505,7 +1483,6 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                 raw_lds_use(cft_); raw_lds_use(cbt_); raw_lds_use(mf); raw_lds_use(mb);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) { raw_lds_use(cfs[j]); raw_lds_use(cbs[j]); raw_lds_use(dts[j]); }
-                TSR(5);
                 if (rows_left < 4) {
                     // rows past the end of the sequence were read from a valid row: drop them
 #pragma unroll
@@ -1569,10 +1546,6 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
 #pragma unroll
                     for (int i = 0; i < 4; ++i) { rowF[i] = __builtin_fmaf(rpf[i], Ef[i], df[i]); rowB[i] = __builtin_fmaf(rpb[i], Eb[i], db[i]); }
                 }
-#ifdef BM2_DBG_TIME
-                asm volatile("" ::"v"(colF[0]), "v"(colF[1]), "v"(colF[2]), "v"(colF[3]), "v"(rowF[0]), "v"(rowF[1]), "v"(rowF[2]), "v"(rowF[3]));
-#endif
-                TSR(6);
                 // ---- hand the sums to the other waves through LDS (double-buffered by head parity)
                 const unsigned pb = sbase + DCB_PART_OFF + par * DCB_PART_B;
                 {
@@ -1605,12 +1578,10 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                     }
                 }
                 raw_lds_wait();
-                TSR(7);
                 pending = true;            // written out after the next barrier (or after the loop)
                 par ^= 1;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-                TSR(9);
             }
             slot = slot + 1 == DCB_RING ? 0 : slot + 1;
             slot2 = slot2 + 1 == DCB_RING ? 0 : slot2 + 1;
@@ -1625,13 +1596,6 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
             raw_lds_barrier();
             write_out(par ^ 1);
         }
-#ifdef BM2_DBG_TIME
-        if (threadIdx.x == 0) {
-            long long *lg2 = reinterpret_cast<long long *>(p.workspace) + (bid.y * gdx + bid.x) * 16;
-            for (int k = 0; k < 10; ++k) lg2[k] = ph[k];
-            lg2[10] = tstart; lg2[11] = tlast;
-        }
-#endif
     }
     const int64_t oo = ((int64_t)bid.z * gdx + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
     float *out = p.dCB + oo, *outT = p.dCBT + oo;

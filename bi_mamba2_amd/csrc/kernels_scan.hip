@@ -75,14 +75,6 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     const int64_t o = (((int64_t)b * H + h) * nc + c) * Q;
     const float *csf = p.cs_f + o, *csb = p.cs_b + o, *dto = p.dt_out + o;
     const float d_head = (p.has_D && !p.D_has_hdim) ? p.D[h] : 0.f;   // read here: in the epilogue its latency would be exposed
-
-#ifdef BM2_DBG_TIME
-    long long *tlog = reinterpret_cast<long long *>(p.workspace) + ((int64_t)blockIdx.x * SCAN_WAVES + wave) * 8;
-#define TSTAMP(i) if (lane == 0) tlog[i] = wall_clock64();
-#else
-#define TSTAMP(i)
-#endif
-    TSTAMP(0)
     // NF > 0: the K rows of part 2 (forward: B rows, mirror: C rows) travel straight into a ring of LDS slots, KRING - 1
     // K steps (of 32 rows) ahead of their use: a global access takes microseconds when the memory system is busy.  Wave w brings rows 4w..4w+3 of the step: unit u = 32*w + lane (lane < 32) is row
     // u/8, chunk position u%8, which holds the row's 16-byte chunk (u%8) ^ (row % 8).
@@ -180,7 +172,6 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
         load_arows(0);
     }
     f32x4 acc[QT][NJ] = {};
-    TSTAMP(1)
 
     // ---- part 1: states.  A = (C or B rows) * row scale, K = dstate; B operand = state tiles [p][n] in LDS ----
     {
@@ -235,7 +226,6 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                 }
             }
             __syncthreads();
-            TSTAMP(2)
 #pragma unroll
             for (int dir = 0; dir < (UNI ? 1 : 2); ++dir) {
                 const T *st = dir ? sB : sF;
@@ -271,7 +261,6 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             tile_load_kcontig<T, float, PW, NW>(sF, stf + n0, N, P - p0, N - n0, Ident());
             tile_load_kcontig<T, float, PW, NW>(sB, stb + n0, N, P - p0, N - n0, Ident());
             __syncthreads();
-            TSTAMP(2)
 #pragma unroll
             for (int s = 0; s < NW / KSTEP; ++s) {
                 if (n0 + s * KSTEP >= N) break;
@@ -348,9 +337,6 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     };
     typedef std::integral_constant<int, 0> B0;
     typedef std::integral_constant<int, 1> B1;
-
-    TSTAMP(3)
-#ifndef BM2_DBG_SKIP2
     // ---- part 2: inside the chunk.  A built in registers from CB (forward) or CB^T (mirror); the CB rows of
     // the next K step are requested before the current step is consumed (two register buffers) ----
     {
@@ -543,7 +529,6 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
             }
         }
     }
-#endif
 
     // ---- epilogue.  Each wave passes its 16-row accumulator tiles through a private LDS patch so that out, out_x,
     // dx are written (and x, z, dy were read) as 16-byte vectors along headdim ----
@@ -571,9 +556,7 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     for (int rt = 0; rt < QT; ++rt) {
         if ((wave * QT + rt) * 16 < limit) epi_issue(rt);
     }
-    TSTAMP(4)
     __syncthreads();   // every wave is done with xT: the operand images become the staging area
-    TSTAMP(5)
     float *stg = reinterpret_cast<float *>(shared_u) + wave * 16 * SLD;
     float dsum[VS];
 #pragma unroll
@@ -647,7 +630,6 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
     for (int rt = 0; rt < QT; ++rt) {
         if ((wave * QT + rt) * 16 < limit) epi_consume(rt);
     }
-    TSTAMP(6)
     if (BWD && p.has_D) {
         // dsum[i]: this lane's share of column (lane % CPR)*VS + i; add the lanes that hold other rows
 #pragma unroll
