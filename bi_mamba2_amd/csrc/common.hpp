@@ -18,6 +18,8 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr int NTHREADS = 256;
 constexpr int BK = 32;          // K extent of one LDS tile
 
+constexpr float LOG2E = 1.4426950408889634f;       // exponentials are taken as 2^(x * LOG2E): one v_exp_f32
+
 __device__ __forceinline__ float to_f(float v) { return v; }
 __device__ __forceinline__ float to_f(bf16_t v) { return static_cast<float>(v); }
 __device__ __forceinline__ float to_f(f16_t v) { return static_cast<float>(v); }
@@ -398,8 +400,11 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
     return v;
 }
+// (row rotations only: every lane has a source, and with bound_ctrl set the compiler folds the move into the
+// instruction that uses it - v_add_f32_dpp instead of v_mov_b32_dpp + v_add_f32)
 template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+    static_assert(CTRL >= 0x121 && CTRL <= 0x12f, "row_ror only");
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 // sum over the 16 lanes that share l/16 (one row group of an MFMA output tile); every lane gets the sum
 __device__ __forceinline__ float row16_sum(float v) {

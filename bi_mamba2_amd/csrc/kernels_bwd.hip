@@ -1441,11 +1441,13 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                 wait_vmcnt<0>();
             }
             raw_lds_barrier();     // step `it` has landed for everybody; every wave is done with the slot and the sums of step it - 1
-            if (it + DCB_RING - 1 < nit) issue(slot2);
+            // (the store of the sums goes out before the requests: the wait at the top of the next step counts on the
+            // requests of the step after it being this wave's youngest operations)
             if (pending) {
                 write_out(par ^ 1);
                 pending = false;
             }
+            if (it + DCB_RING - 1 < nit) issue(slot2);
             const unsigned sb = sbase + slot * DCB_SLOT_B;
             Frag af[NKS], bf[4][NKS];
 #pragma unroll
@@ -1457,13 +1459,16 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                 bf[3][ks] = raw_lds_read_at<Frag, 6144>(sb + b_off[ks]);
             }
             raw_lds_wait();
+            // (the first product of a head starts from a literal zero: no registers to clear between heads)
+            const bool first = kc == 0;
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
                 raw_lds_use(af[ks]);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     raw_lds_use(bf[j][ks]);
-                    acc[j] = M::mma(af[ks], bf[j][ks], acc[j]);
+                    if (ks == 0 && first) acc[j] = M::mma(af[ks], bf[j][ks], f32x4{0.f, 0.f, 0.f, 0.f});
+                    else acc[j] = M::mma(af[ks], bf[j][ks], acc[j]);
                 }
             }
             if (++kc == nkc) {
@@ -1509,10 +1514,11 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                 if constexpr (!DIAG) {
                     const bool lower = st < tt;                // forward direction below the diagonal, reverse above it
                     float E[4], rp[4] = {0.f, 0.f, 0.f, 0.f};
+                    const float ml = (lower ? mf : mb) * LOG2E;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) E[i] = __expf(lower ? cft_[i] - mf : cbt_[i] - mb);
+                    for (int i = 0; i < 4; ++i) E[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(lower ? cft_[i] : cbt_[i], LOG2E, -ml));
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) sep_block(j, E, dts[j] * __expf(lower ? mf - cfs[j] : mb - cbs[j]), colF[j], rp);
+                    for (int j = 0; j < 4; ++j) sep_block(j, E, dts[j] * __builtin_amdgcn_exp2f(__builtin_fmaf(lower ? cfs[j] : cbs[j], -LOG2E, ml)), colF[j], rp);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) rowF[i] = rp[i] * E[i];
                 } else {
@@ -1580,8 +1586,6 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                 raw_lds_wait();
                 pending = true;            // written out after the next barrier (or after the loop)
                 par ^= 1;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
             slot = slot + 1 == DCB_RING ? 0 : slot + 1;
             slot2 = slot2 + 1 == DCB_RING ? 0 : slot2 + 1;

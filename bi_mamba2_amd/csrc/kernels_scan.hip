@@ -23,7 +23,6 @@ namespace bm2 {
 static inline int nchunks(const bimamba2_params *p) { return (p->seqlen + p->chunk_size - 1) / p->chunk_size; }
 static inline hipStream_t stream_of(const bimamba2_params *p) { return reinterpret_cast<hipStream_t>(p->stream); }
 
-constexpr float LOG2E = 1.4426950408889634f;
 
 constexpr int SCAN_WAVES = 8, SCAN_THREADS = 64 * SCAN_WAVES;
 

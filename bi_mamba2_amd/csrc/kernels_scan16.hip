@@ -49,7 +49,6 @@ namespace bm2 {
 
 namespace {
 
-constexpr float LOG2E = 1.4426950408889634f;
 constexpr int S16_WAVES = 16, S16_THREADS = 64 * S16_WAVES;
 constexpr int S16_ROWS = 16 * S16_WAVES;          // rows the workgroup covers (>= chunk_size)
 constexpr int S16_NSTEP = S16_ROWS / 32;          // K steps at most
