@@ -40,6 +40,7 @@
 //     acc[r,p] = e^{cs_f[Q-1]-cs_f[r]} B_r.dS_f[p,:] + e^{cs_b[0]-cs_b[r]} B_r.dS_b[p,:]
 //              + sum_k CBT[r,k] m'(r,k) dy[k,p],       m' = e^{cs_f[k]-cs_f[r]} (k>r), e^{cs_b[k]-cs_b[r]} (k<r), 2 (k=r)
 //     dx = acc dt[r] + D dy[r,p];  ddt_direct[r] = sum_p acc x[r,p];  dD partial = sum_r dy x
+#include <atomic>
 #include <type_traits>
 
 #include "common.hpp"
@@ -626,19 +627,42 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
     }
 }
 
-// heads a workgroup of the kernel above walks through: the largest divisor of the heads per group that is <= S16_MAX_HEADS
-static int scan16_heads_per_block(const bimamba2_params *p) {
-    const int hpg = p->nheads / p->ngroups;
-    for (int k = S16_MAX_HEADS; k > 1; --k)
-        if (hpg % k == 0) return k;
-    return 1;
+// CUs of the current device (one workgroup of the kernel above fills a CU), asked for once per device
+static int cu_count() {
+    constexpr int MAXD = 64;
+    static std::atomic<int> cached[MAXD];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAXD) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+// Heads a workgroup of the kernel above walks through: a divisor k <= S16_MAX_HEADS of the heads per group, chosen for the
+// shortest launch.  The grid runs in rounds of one workgroup per CU, and a workgroup takes a fixed start (launch, first
+// loads, CB: about 0.8 of a head's time) plus k heads: rounds(k) * (0.8 + k) is what is compared, the larger k on a tie.
+static int scan16_heads_per_block(const bimamba2_params *p, int nc) {
+    const int hpg = p->nheads / p->ngroups, cus = cu_count();
+    const long long units = (long long)p->batch * nc * (p->headdim / 64) * p->nheads;
+    int best = 1;
+    double best_cost = 0;
+    for (int k = 1; k <= S16_MAX_HEADS; ++k) {
+        if (hpg % k) continue;
+        const long long rounds = (units / k + cus - 1) / cus;
+        const double cost = rounds * (0.8 + k);
+        if (k == 1 || cost <= best_cost) { best = k; best_cost = cost; }
+    }
+    return best;
 }
 
 // Launches the kernel above; the caller (launch_chunk_scan) has checked that the problem is one of its shapes:
 // scan_recomputes_cb(), 16-bit copies of the entering states present and 16-byte aligned.
 template <typename T, bool BWD>
 static int launch_scan16_t(const bimamba2_params *p, int nc) {
-    const int npt = p->headdim / 64, hpw = scan16_heads_per_block(p);
+    const int npt = p->headdim / 64, hpw = scan16_heads_per_block(p, nc);
     dim3 grid(p->batch * nc * (p->nheads / hpw) * npt);
     hipStream_t s = reinterpret_cast<hipStream_t>(p->stream);
     if (p->causal) hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, true>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
