@@ -735,7 +735,9 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
         }
     }
     f32x4 tf[QT][4], tb[QT][4];
-    auto step_body = [&](int step, Frag (&af)[QT][NKS]) {
+    // SLOT = step % RING as a compile-time value: the slot's offset goes into the offset field of the LDS reads
+    auto step_body = [&](int step, Frag (&af)[QT][NKS], auto SLOT) {
+        constexpr int RB = decltype(SLOT)::value * NDIR * TILE_B;
         const int hh = hh0 + step / nkc, kc = step % nkc;
         // this wave's requests of the step have landed (those of the next step may be outstanding) ...
         if (step + 1 < nsteps) wait_vmcnt<PER_STEP>();
@@ -766,48 +768,63 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
         raw_lds_wait();
         raw_lds_barrier();
         }
-        if (kc == 0) {
-#pragma unroll
-            for (int q = 0; q < QT; ++q)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) { tf[q][j] = f32x4{0.f, 0.f, 0.f, 0.f}; tb[q][j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-        }
+        // (the first products of a head start from a literal zero: no registers to clear between heads)
+        const bool first = kc == 0;
 #pragma unroll
         for (int q = 0; q < QT; ++q)
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) raw_lds_use(af[q][ks]);
         const unsigned ib = buf * NDIR * IMG_B;
-        const unsigned rb = ((step % RING) * NDIR) * TILE_B;
+        if constexpr (S16) {
+            // both K halves' fragments are asked for at once; the products of the first half run while the second half's
+            // reads are still under way (LDS reads return in order: "at most NR outstanding" = the first half is there)
+            static_assert(NKS == 2, "two K halves");
+            constexpr int NR = UNI ? 8 : 16;                   // LDS reads per K half
+            i16x4 flo[NKS][4], fhi[NKS][4], blo[NKS][4], bhi[NKS][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                flo[0][j] = raw_lds_tr16_read_at<RB>(tr_lo[j]); fhi[0][j] = raw_lds_tr16_read_at<RB>(tr_hi[j]);
+                if (!UNI) { blo[0][j] = raw_lds_tr16_read_at<RB + TILE_B>(tr_lo[j]); bhi[0][j] = raw_lds_tr16_read_at<RB + TILE_B>(tr_hi[j]); }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                flo[1][j] = raw_lds_tr16_read_at<RB + 4096>(tr_lo[j]); fhi[1][j] = raw_lds_tr16_read_at<RB + 4096>(tr_hi[j]);
+                if (!UNI) { blo[1][j] = raw_lds_tr16_read_at<RB + TILE_B + 4096>(tr_lo[j]); bhi[1][j] = raw_lds_tr16_read_at<RB + TILE_B + 4096>(tr_hi[j]); }
+            }
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                // lgkmcnt(min(NR, 15)), vmcnt and expcnt left alone (the counter has four bits: 15 is its largest value)
+                if (ks == 0) __builtin_amdgcn_s_waitcnt(0xC07F | ((NR < 15 ? NR : 15) << 8));
+                else raw_lds_wait();
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    raw_lds_use(flo[ks][j]); raw_lds_use(fhi[ks][j]);
+                    const Frag bff = __builtin_bit_cast(Frag, __builtin_shufflevector(flo[ks][j], fhi[ks][j], 0, 1, 2, 3, 4, 5, 6, 7));
+                    Frag bfb = bff;
+                    if (!UNI) {
+                        raw_lds_use(blo[ks][j]); raw_lds_use(bhi[ks][j]);
+                        bfb = __builtin_bit_cast(Frag, __builtin_shufflevector(blo[ks][j], bhi[ks][j], 0, 1, 2, 3, 4, 5, 6, 7));
+                    }
+#pragma unroll
+                    for (int q = 0; q < QT; ++q) {
+                        if (ks == 0 && first) {
+                            tf[q][j] = M::mma(af[q][ks], bff, f32x4{0.f, 0.f, 0.f, 0.f});
+                            if (!UNI) tb[q][j] = M::mma(af[q][ks], bfb, f32x4{0.f, 0.f, 0.f, 0.f});
+                        } else {
+                            tf[q][j] = M::mma(af[q][ks], bff, tf[q][j]);
+                            if (!UNI) tb[q][j] = M::mma(af[q][ks], bfb, tb[q][j]);
+                        }
+                    }
+                }
+            }
+        } else {
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
             Frag bff[4], bfb[4];
-            if constexpr (S16) {
-                i16x4 flo[4], fhi[4], blo[4], bhi[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if (ks == 0) { flo[j] = raw_lds_tr16_read_at<0>(tr_lo[j] + rb); fhi[j] = raw_lds_tr16_read_at<0>(tr_hi[j] + rb); }
-                    else { flo[j] = raw_lds_tr16_read_at<4096>(tr_lo[j] + rb); fhi[j] = raw_lds_tr16_read_at<4096>(tr_hi[j] + rb); }
-                    if (!UNI) {
-                        if (ks == 0) { blo[j] = raw_lds_tr16_read_at<TILE_B>(tr_lo[j] + rb); bhi[j] = raw_lds_tr16_read_at<TILE_B>(tr_hi[j] + rb); }
-                        else { blo[j] = raw_lds_tr16_read_at<TILE_B + 4096>(tr_lo[j] + rb); bhi[j] = raw_lds_tr16_read_at<TILE_B + 4096>(tr_hi[j] + rb); }
-                    }
-                }
-                raw_lds_wait();
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    raw_lds_use(flo[j]); raw_lds_use(fhi[j]);
-                    bff[j] = __builtin_bit_cast(Frag, __builtin_shufflevector(flo[j], fhi[j], 0, 1, 2, 3, 4, 5, 6, 7));
-                    if (!UNI) {
-                        raw_lds_use(blo[j]); raw_lds_use(bhi[j]);
-                        bfb[j] = __builtin_bit_cast(Frag, __builtin_shufflevector(blo[j], bhi[j], 0, 1, 2, 3, 4, 5, 6, 7));
-                    }
-                }
-            } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 bff[j] = raw_lds_read_at<Frag, 0>(img_r[ks][j] + ib);
                 if (!UNI) bfb[j] = raw_lds_read_at<Frag, IMG_B>(img_r[ks][j] + ib);
-            }
             }
             raw_lds_wait();
 #pragma unroll
@@ -816,10 +833,16 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
                 if (!UNI) raw_lds_use(bfb[j]);
 #pragma unroll
                 for (int q = 0; q < QT; ++q) {
-                    tf[q][j] = M::mma(af[q][ks], bff[j], tf[q][j]);
-                    if (!UNI) tb[q][j] = M::mma(af[q][ks], bfb[j], tb[q][j]);
+                    if (ks == 0 && first) {
+                        tf[q][j] = M::mma(af[q][ks], bff[j], f32x4{0.f, 0.f, 0.f, 0.f});
+                        if (!UNI) tb[q][j] = M::mma(af[q][ks], bfb[j], f32x4{0.f, 0.f, 0.f, 0.f});
+                    } else {
+                        tf[q][j] = M::mma(af[q][ks], bff[j], tf[q][j]);
+                        if (!UNI) tb[q][j] = M::mma(af[q][ks], bfb[j], tb[q][j]);
+                    }
                 }
             }
+        }
         }
         // the fragments of step + 2 take the place of the ones just used
         if (step + 2 < nsteps) issue_frags(step + 2, af);
@@ -852,9 +875,14 @@ __global__ __launch_bounds__(DBDC_THREADS) void bwd_dbdc_dma_kernel(const bimamb
             }
         }
     };
-    for (int step = 0; step < nsteps; step += 2) {
-        step_body(step, afA);
-        if (step + 1 < nsteps) step_body(step + 1, afB);
+    static_assert(RING == 3, "six steps = one round of ring slots and of the two fragment sets");
+    for (int step = 0; step < nsteps; step += 6) {
+        step_body(step, afA, std::integral_constant<int, 0>());
+        if (step + 1 < nsteps) step_body(step + 1, afB, std::integral_constant<int, 1>());
+        if (step + 2 < nsteps) step_body(step + 2, afA, std::integral_constant<int, 2>());
+        if (step + 3 < nsteps) step_body(step + 3, afB, std::integral_constant<int, 0>());
+        if (step + 4 < nsteps) step_body(step + 4, afA, std::integral_constant<int, 1>());
+        if (step + 5 < nsteps) step_body(step + 5, afB, std::integral_constant<int, 2>());
     }
     raw_lds_wait();
     __syncthreads();                                           // nothing is in flight any more: ordinary code again
