@@ -352,6 +352,9 @@ int bimamba2_bwd(const bimamba2_params *p) {
         TRY(forward_cumsum_and_states(&q));
         TRY(bimamba2_state_passing_fwd(&q));
     }
+    // dCB / dCBT in the 16-bit element type where this call owns them and the two launches that write and read them are the
+    // merged ones (their reader rounds them to that type for its MFMA anyway)
+    const bool dcb16 = !p->dCB && !p->dCBT && bwd_dcb_sp_merged(&q) && bwd_tail_merged(&q);
     const bool need_cbt = !scan_recomputes_cb(&q, true), need_cb = need_cbt || !dcb_recomputes_cb(&q);
     if (need_cb) TRY(bimamba2_bmm_chunk_fwd(&q));  // CB for the dCB kernel, CB^T for the dx kernel, unless they rebuild it
     else q.CB = nullptr;
@@ -365,7 +368,7 @@ int bimamba2_bwd(const bimamba2_params *p) {
         REQUIRE(q.x); REQUIRE(q.dt_out); REQUIRE(q.cs_f); REQUIRE(q.cs_b); REQUIRE(q.dCB); REQUIRE(q.dCBT); REQUIRE(q.da_intra);
         REQUIRE(q.dstates_f); REQUIRE(q.ddA_chunk_f); REQUIRE(q.ddA_chunk_b);
         if (q.has_z) REQUIRE(q.dout_x); else REQUIRE(q.dout);
-        TRY(launch_bwd_dcb_sp(&q));
+        TRY(launch_bwd_dcb_sp(&q, dcb16));
     } else {
         TRY(bimamba2_chunk_scan_bwd_dcb(&q));
         TRY(bimamba2_chunk_scan_bwd_dstates(&q));
@@ -396,7 +399,7 @@ int bimamba2_bwd(const bimamba2_params *p) {
         qc.red = q.red + (size_t)q.batch * nchunks(&q) * q.nheads * q.headdim;
         REQUIRE(q.ddt); REQUIRE(q.dA); REQUIRE(q.dB); REQUIRE(q.dC);
         if (bwd_tail_merged(&q)) {
-            TRY(launch_bwd_tail(&qc, &jobs));
+            TRY(launch_bwd_tail(&qc, &jobs, dcb16));
         } else {
             TRY(bimamba2_bmm_chunk_bwd(&q));
             TRY(launch_chunk_cumsum_bwd(&qc, &jobs));

@@ -1304,7 +1304,7 @@ constexpr int DCB_PART_B = 10 * 64 * 4;
 // UNI: the single-direction operator - tiles above the diagonal are empty, tiles on it keep the forward half.
 // bid / gdx / gdz: block index and grid extents (x: batch * chunks * groups, y: tiles, z: head slices)
 template <typename T, bool UNI>
-__device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int nc, int nqt, BlockId bid, int gdx, int gdz) {
+__device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int nc, int nqt, BlockId bid, int gdx, int gdz, bool out16 = false) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
     static_assert(sizeof(T) == 2, "ring variant is for 16-bit operands");
@@ -1630,6 +1630,23 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
         }
     }
     const int64_t oo = ((int64_t)bid.z * gdx + (int64_t)(b * nc + c) * p.ngroups + g) * Q * Q;
+    if (out16) {
+        // dCB / dCBT in the element type of the inputs (inside bimamba2_bwd, one head slice: their one reader rounds them to
+        // that type for its MFMA anyway, so nothing changes but the bytes moved)
+        T *out = reinterpret_cast<T *>(p.dCB) + oo, *outT = reinterpret_cast<T *>(p.dCBT) + oo;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int s = s0 + j * 16 + lr;
+            T v4[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v4[i] = from_f<T>(dcb[j][i]);
+                out[(int64_t)(t0 + trow + i) * Q + s] = v4[i];
+            }
+            *reinterpret_cast<uint2 *>(outT + (int64_t)s * Q + t0 + trow) = *reinterpret_cast<const uint2 *>(v4);
+        }
+        return;
+    }
     float *out = p.dCB + oo, *outT = p.dCBT + oo;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -1651,10 +1668,10 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
 // dCB tiles in the order of their own grid (so they are placed first, two per CU as when alone), the rest are the state
 // passing's blocks, which take what is left of each CU.
 template <typename T, bool UNI>
-__global__ __launch_bounds__(NTHREADS) void bwd_dcb_sp_kernel(const bimamba2_params p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir) {
+__global__ __launch_bounds__(NTHREADS) void bwd_dcb_sp_kernel(const bimamba2_params p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir, bool out16) {
     const int id = blockIdx.x;
     if (id < ndcb) {
-        bwd_dcb_ring_body<T, UNI>(p, nc, nqt, BlockId{id % gdx, id / gdx, 0}, gdx, 1);
+        bwd_dcb_ring_body<T, UNI>(p, nc, nqt, BlockId{id % gdx, id / gdx, 0}, gdx, 1, out16);
     } else {
         const int k = id - ndcb;                  // grid (nsplit, nheads, batch * ndir) of the state passing
         state_passing_bwd_vec_body<T, true, true>(p, nc, nsplit, ndir, BlockId{k % nsplit, (k / nsplit) % p.nheads, k / (nsplit * p.nheads)});
@@ -1717,15 +1734,15 @@ bool bwd_dcb_sp_merged(const bimamba2_params *p) {
 }
 
 // bimamba2_chunk_scan_bwd_dcb and bimamba2_state_passing_bwd in one launch (the caller checked bwd_dcb_sp_merged())
-int launch_bwd_dcb_sp(const bimamba2_params *p) {
+int launch_bwd_dcb_sp(const bimamba2_params *p, bool out16) {
     const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64, PN = p->headdim * p->dstate;
     const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS), ndir = p->causal ? 1 : 2;
     const int gdx = p->batch * nc * p->ngroups, ndcb = gdx * nqt * nqt, nsp = nsplit * p->nheads * p->batch * ndir;
     dim3 grid(ndcb + nsp);
 #define BM2_DS(TT)                                                                                                                     \
     do {                                                                                                                               \
-        if (p->causal) hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir);  \
-        else hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir);           \
+        if (p->causal) hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);  \
+        else hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);           \
     } while (0)
     if (p->dtype == BIMAMBA2_BF16) BM2_DS(bf16_t); else BM2_DS(f16_t);
 #undef BM2_DS
@@ -1751,7 +1768,7 @@ int launch_bwd_dcb(const bimamba2_params *p) {
 
 
 template <typename T, int QP, bool FAST>
-__device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int nc, int nslices, BlockId bid) {
+__device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int nc, int nslices, BlockId bid, bool in16 = false) {
     typedef Mma<T> M;
     constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
     constexpr int LDX = QP + 16 / (int)sizeof(T);
@@ -1776,11 +1793,19 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
     __shared__ __attribute__((aligned(16))) float stg[64 * SLD];
     if constexpr (FAST) {
         constexpr int NS = QP / KSTEP, NIT = 64 * (64 / VS) / NTHREADS, MAXSL = 8;
+        // in16: dCB / dCBT hold elements of type T (written that way by the dCB kernel inside bimamba2_bwd): a row piece is
+        // the MFMA operand as it lies in memory
         float4 raw[NS][2];
+        if (in16) {
+            const T *arow16 = reinterpret_cast<const T *>(which == 0 ? p.dCBT : p.dCB) + (int64_t)bcg * Q * Q + (int64_t)min(r0 + wave * 16 + lr, Q - 1) * Q;
 #pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            raw[s][0] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL);
-            raw[s][1] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL + 4);
+            for (int s = 0; s < NS; ++s) raw[s][0] = *reinterpret_cast<const float4 *>(arow16 + s * KSTEP + lg * KPL);
+        } else {
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                raw[s][0] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL);
+                raw[s][1] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL + 4);
+            }
         }
         // slices: the first half is requested here, the second half after the products, into the registers of the row pieces
         // (keeps the kernel at two workgroups per CU)
@@ -1807,7 +1832,9 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
         for (int s = 0; s < NS; ++s) {
             if (s * KSTEP < limit) {
                 float v[KPL] = {raw[s][0].x, raw[s][0].y, raw[s][0].z, raw[s][0].w, raw[s][1].x, raw[s][1].y, raw[s][1].z, raw[s][1].w};
-                const typename M::Frag af = M::pack(v);
+                typename M::Frag af;
+                if constexpr (sizeof(typename M::Frag) == 16) af = in16 ? __builtin_bit_cast(typename M::Frag, raw[s][0]) : M::pack(v);
+                else af = M::pack(v);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[j] = M::mma(af, M::load(kT + xt_index<T, LDX>(j * 16 + lr, s * KSTEP + lg * KPL)), acc[j]);
             }
@@ -2109,11 +2136,11 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
 // other, both are short and latency-bound, and together they fit the machine in one wave of workgroups.
 template <typename T, typename DT>
 __global__ __launch_bounds__(NTHREADS) void bwd_tail_kernel(const bimamba2_params p, int nc, int nslices, int nqt, int nsplit, int nbmm,
-                                                            int bmm_gy, int cs_gx) {
+                                                            int bmm_gy, int cs_gx, bool in16) {
     const int id = blockIdx.x;
     if (id < nbmm) {
         // bmm grid (1, bmm_gy, z)
-        bmm_chunk_bwd_body<T, 256, true>(p, nc, nslices, BlockId{0, id % bmm_gy, id / bmm_gy});
+        bmm_chunk_bwd_body<T, 256, true>(p, nc, nslices, BlockId{0, id % bmm_gy, id / bmm_gy}, in16);
     } else {
         const int k = id - nbmm;                  // cumsum grid (cs_gx, nc, batch)
         chunk_cumsum_bwd_body<DT>(p, nc, nqt, nsplit, BlockId{k % cs_gx, (k / cs_gx) % nc, k / (cs_gx * nc)});
@@ -2133,15 +2160,15 @@ static bool bmm_bwd_fast(const bimamba2_params *p) {
 bool bwd_tail_merged(const bimamba2_params *p) { return bmm_bwd_fast(p) && p->chunk_size == 256 && p->dstate == 64; }
 
 template <typename T>
-static int launch_bwd_tail_t(const bimamba2_params *p, int nc, int nqt, int nsplit) {
+static int launch_bwd_tail_t(const bimamba2_params *p, int nc, int nqt, int nsplit, bool in16) {
     const int bmm_gy = (p->chunk_size + 63) / 64, nbmm = bmm_gy * p->batch * nc * p->ngroups * 2;
     const int cs_gx = (p->nheads + 3) / 4, ncs = cs_gx * nc * p->batch;
     dim3 grid(nbmm + ncs);
     const int nsl = dbdc_slices(p);
     switch (p->dt_dtype) {
-        case BIMAMBA2_F32: hipLaunchKernelGGL((bwd_tail_kernel<T, float>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx); break;
-        case BIMAMBA2_BF16: hipLaunchKernelGGL((bwd_tail_kernel<T, bf16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx); break;
-        case BIMAMBA2_F16: hipLaunchKernelGGL((bwd_tail_kernel<T, f16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx); break;
+        case BIMAMBA2_F32: hipLaunchKernelGGL((bwd_tail_kernel<T, float>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx, in16); break;
+        case BIMAMBA2_BF16: hipLaunchKernelGGL((bwd_tail_kernel<T, bf16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx, in16); break;
+        case BIMAMBA2_F16: hipLaunchKernelGGL((bwd_tail_kernel<T, f16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx, in16); break;
         default: return BIMAMBA2_EUNSUPPORTED;
     }
     return check_launch();
@@ -2149,11 +2176,11 @@ static int launch_bwd_tail_t(const bimamba2_params *p, int nc, int nqt, int nspl
 
 // bmm_chunk_bwd + chunk_cumsum_bwd in one launch (the caller checked bwd_tail_merged()); reductions as in
 // launch_chunk_cumsum_bwd
-int launch_bwd_tail(const bimamba2_params *p, ReduceJobs *defer) {
+int launch_bwd_tail(const bimamba2_params *p, ReduceJobs *defer, bool in16) {
     const int nc = nchunks(p), nqt = (p->chunk_size + 63) / 64;
     const int PN = p->headdim * p->dstate;
     const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS);
-    int rc = p->dtype == BIMAMBA2_BF16 ? launch_bwd_tail_t<bf16_t>(p, nc, nqt, nsplit) : launch_bwd_tail_t<f16_t>(p, nc, nqt, nsplit);
+    int rc = p->dtype == BIMAMBA2_BF16 ? launch_bwd_tail_t<bf16_t>(p, nc, nqt, nsplit, in16) : launch_bwd_tail_t<f16_t>(p, nc, nqt, nsplit, in16);
     if (rc) return rc;
     const int ni = p->batch * nc;
     defer->job[defer->n++] = ReduceJob{p->red, p->dA, ni, p->nheads, 1};

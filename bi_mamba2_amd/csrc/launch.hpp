@@ -36,9 +36,11 @@ int launch_chunk_cumsum_bwd(const bimamba2_params *p, ReduceJobs *defer = nullpt
 // bmm_chunk_bwd and chunk_cumsum_bwd as one launch, where bwd_tail_merged() says it exists
 // the dCB kernel and the backward state passing as one launch, where bwd_dcb_sp_merged() says it exists
 bool bwd_dcb_sp_merged(const bimamba2_params *p);
-int launch_bwd_dcb_sp(const bimamba2_params *p);
+// out16 / in16: dCB and dCBT in the element type of the inputs between the two launches (one head slice: the reader rounds
+// them to that type anyway)
+int launch_bwd_dcb_sp(const bimamba2_params *p, bool out16 = false);
 bool bwd_tail_merged(const bimamba2_params *p);
-int launch_bwd_tail(const bimamba2_params *p, ReduceJobs *defer);
+int launch_bwd_tail(const bimamba2_params *p, ReduceJobs *defer, bool in16 = false);
 int launch_fill(float *ptr, size_t n, float value, hipStream_t stream);
 // out[j] = sum_{i<ni} sum_{k<nk} in[(i*nj + j)*nk + k]
 int launch_reduce(const float *in, float *out, int ni, int nj, int nk, hipStream_t stream);
