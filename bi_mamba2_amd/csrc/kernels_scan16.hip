@@ -513,10 +513,11 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             for (int t = 0; t < 2; ++t) {
                 // the D term's row (forward: x, mirror: dy) from the raw tile, z (resp. x) from the rows this wave brought
                 const unsigned eo = sb + tile64_row_offset(min(r_lane, limit - 1), t * 32 + cq);
-                f32x4 kx4 = {0.f, 0.f, 0.f, 0.f}, g24 = {0.f, 0.f, 0.f, 0.f}, d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
-                if (need_d || BWD) kx4 = raw_lds_read_at<f32x4, S16_XR>(eo + cur * 32768);
-                if (BWD || p.has_z) g24 = raw_lds_read_at<f32x4, 0>(eo + S16_KT);
-                if (need_d) {
+                // (read whether used or not: the addresses are valid, and a conditional read needs its registers cleared first)
+                f32x4 kx4 = raw_lds_read_at<f32x4, S16_XR>(eo + cur * 32768);
+                f32x4 g24 = raw_lds_read_at<f32x4, 0>(eo + S16_KT);
+                f32x4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+                if (!BWD || need_d) {                  // (the mirror is out of registers: there the read stays conditional)
                     d0 = t ? raw_lds_read_at<f32x4, 128>(d_a) : raw_lds_read_at<f32x4, 0>(d_a);
                     d1 = t ? raw_lds_read_at<f32x4, 144>(d_a) : raw_lds_read_at<f32x4, 16>(d_a);
                 }
