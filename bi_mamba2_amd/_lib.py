@@ -59,10 +59,10 @@ class NormParams(ctypes.Structure):
     """Mirror of ``struct bimamba2_norm_params`` (gated RMSNorm)."""
     _fields_ = (
         [("rows", _i64), ("cols", _i32), ("group_size", _i32), ("dtype", _i32), ("has_z", _i32), ("has_bias", _i32),
-         ("norm_before_gate", _i32), ("eps", _f32), ("reserved0", _i32)]
+         ("norm_before_gate", _i32), ("eps", _f32), ("layer_norm", _i32)]
         + [(n, _i64) for n in ("x_rs", "z_rs", "out_rs", "dout_rs", "dx_rs", "dz_rs")]
         + [(n, _vp) for n in ("x", "z", "weight", "bias", "out", "rstd", "dout", "dx", "dz", "dweight", "dbias", "workspace")]
-        + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
+        + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp), ("mean", _vp)]
     )
 
 

@@ -435,6 +435,7 @@ int bimamba2_rmsnorm_gated_fwd(const bimamba2_norm_params *p) {
 int bimamba2_rmsnorm_gated_bwd(const bimamba2_norm_params *p) {
     TRY(check_norm(p));
     REQUIRE(p->dout); REQUIRE(p->rstd); REQUIRE(p->dx); REQUIRE(p->dweight);
+    if (p->layer_norm) REQUIRE(p->mean);
     if (p->has_z) REQUIRE(p->dz);
     if (p->has_bias) REQUIRE(p->dbias);
     if (!p->workspace || p->workspace_bytes < norm_workspace_bytes(p)) return BIMAMBA2_EWORKSPACE;

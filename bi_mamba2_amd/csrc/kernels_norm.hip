@@ -2,8 +2,10 @@
 // layer):   xg = x            (norm_before_gate)   or  x * silu(z)
 //           y  = xg * rstd * weight (+ bias),  rstd = 1 / sqrt(mean_group(xg^2) + eps)
 //           out = y * silu(z) (norm_before_gate)   or  y
+// and, with layer_norm set, the LayerNorm of the same reference kernels (IS_RMS_NORM = False): xg is centred by its group
+// mean first, xc = xg - mean_group(xg), rstd = 1 / sqrt(mean_group(xc^2) + eps), y = xc * rstd * weight (+ bias).
 // Math of rms_norm_ref (src/ssd/bi/layernorm_gated.py:18-39 of the reference); replaces its kernels
-// _layer_norm_fwd_1pass_kernel (:45-105) and _layer_norm_bwd_kernel (:155-268) for the RMS case.
+// _layer_norm_fwd_1pass_kernel (:45-105) and _layer_norm_bwd_kernel (:155-268).
 //
 // Pure HBM traffic: one wave owns one (row, group); lane l owns the 8-element pieces l, l + 64, ... of the group (16-byte
 // accesses when the rows allow it).  Forward keeps the group in registers between the two passes.  Backward re-reads it
@@ -91,6 +93,20 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_fwd_kernel(const bimam
 #pragma unroll
         for (int k = 0; k < NCH; ++k) load8(w + (k * 64 + lane) * 8, true, 8, wk[FULL ? k : 0]);
     }
+    if (p.layer_norm) {
+        float sm = 0.f;
+#pragma unroll
+        for (int k = 0; k < NCH; ++k)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sm += xv[k][i];
+        const float mean = wave_sum(sm) / gs;
+        if (lane == 0 && p.mean) p.mean[item] = mean;
+#pragma unroll
+        for (int k = 0; k < NCH; ++k)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (FULL || (k * 64 + lane) * 8 + i < gs) xv[k][i] -= mean;      // (columns past the group stay zero)
+    }
 #pragma unroll
     for (int k = 0; k < NCH; ++k)
 #pragma unroll
@@ -158,7 +174,8 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
         T *dx = reinterpret_cast<T *>(p.dx) + row * p.dx_rs + g * gs;
         T *dz = p.has_z ? reinterpret_cast<T *>(p.dz) + row * p.dz_rs + g * gs : nullptr;
         const float rstd = p.rstd[row * ngroups + g];
-        // Per element: xhat = xg * rstd, wdy = weight * dy' (dy' = dy * silu(z) when the gate comes last), and for a gate
+        const float mean = p.layer_norm ? p.mean[row * ngroups + g] : 0.f;
+        // Per element: xhat = (xg - mean) * rstd, wdy = weight * dy' (dy' = dy * silu(z) when the gate comes last), and for a gate
         // that comes first sl = silu(z), g2 = x * dsilu(z).  Groups of up to 2048 columns keep them in registers between
         // the two passes; wider ones read the row again (from cache) and recompute.
         constexpr bool HOLD = NCH <= 4;
@@ -180,7 +197,8 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
                 }
                 slv[i] = si;
                 g2v[i] = xv[i] * ds;
-                xhat[i] = (gate_first ? xv[i] * si : xv[i]) * rstd;
+                xhat[i] = ((gate_first ? xv[i] * si : xv[i]) - mean) * rstd;
+                if (!FULL && c + i >= gs) xhat[i] = 0.f;                   // (matters with a mean only)
                 if (gate_last) {
                     dzv[i] = dy[i] * (xhat[i] * wv[i] + (HAS_BIAS && first ? bv[i] : 0.f)) * ds;
                     dy[i] *= si;
@@ -193,8 +211,9 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
             }
             if (gate_last && first) store8(dz + c, vec, FULL ? 8 : gs - c, dzv);
         };
-        // pass 1: c1 = mean(xhat * wdy), weight / bias gradients, and dz when the gate comes last
-        float c1 = 0.f;
+        // pass 1: c1 = mean(xhat * wdy) (and c2 = mean(wdy) for the LayerNorm), weight / bias gradients, and dz when the gate
+        // comes last
+        float c1 = 0.f, c2 = 0.f;
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
             const int c = (k * 64 + lane) * 8;
@@ -204,10 +223,12 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 c1 += xhat[i] * wdy[i];
+                c2 += wdy[i];
                 if (HOLD) { xh[k][i] = xhat[i]; wd[k][i] = wdy[i]; sl[k][i] = slv[i]; g2[k][i] = g2v[i]; }
             }
         }
         c1 = wave_sum(c1) / gs;
+        c2 = p.layer_norm ? wave_sum(c2) / gs : 0.f;
         // pass 2: dx, and dz when the gate comes first
 #pragma unroll
         for (int k = 0; k < NCH; ++k) {
@@ -222,7 +243,7 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float dxg = (wdy[i] - xhat[i] * c1) * rstd;
+                const float dxg = (wdy[i] - xhat[i] * c1 - c2) * rstd;
                 dxv[i] = gate_first ? dxg * slv[i] : dxg;
                 dzv[i] = dxg * g2v[i];
             }

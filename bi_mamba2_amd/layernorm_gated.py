@@ -1,9 +1,10 @@
-"""Gated RMSNorm on the HIP kernels, with the reference's names (src/ssd/bi/layernorm_gated.py of Hprairie/Bi-Mamba2):
-``rmsnorm_fn`` (:383-384 there), the ``RMSNorm`` module (:415-437) and the autograd function behind them
-(``LayerNormFn``, :333-376, with is_rms_norm=True).
+"""Gated RMSNorm / LayerNorm on the HIP kernels, with the reference's names (src/ssd/bi/layernorm_gated.py of
+Hprairie/Bi-Mamba2): ``rmsnorm_fn`` (:383-384 there) and ``layernorm_fn`` (:380-381), the ``RMSNorm`` (:415-437) and
+``LayerNorm`` (:388-412) modules and the autograd function behind them (``LayerNormFn``, :333-376).
 
     xg  = x                    if norm_before_gate else x * silu(z)
-    y   = xg / sqrt(mean_group(xg^2) + eps) * weight (+ bias)
+    xc  = xg                   (RMS norm)         or  xg - mean_group(xg)   (LayerNorm, is_rms_norm=False)
+    y   = xc / sqrt(mean_group(xc^2) + eps) * weight (+ bias)
     out = y * silu(z)          if norm_before_gate else y
 
 There is no CPU or PyTorch fallback: CPU tensors raise, a missing library raises.
@@ -34,7 +35,7 @@ def _call(entry, p, device):
         raise (ValueError if rc in (-1, -2) else RuntimeError)(f"{entry}: {msg} (code {rc})")
 
 
-def _params(x2, z2, weight, bias, eps, group_size, norm_before_gate):
+def _params(x2, z2, weight, bias, eps, group_size, norm_before_gate, is_rms_norm=True):
     if x2.dtype not in _DT:
         raise ValueError(f"unsupported dtype {x2.dtype} (need float32, bfloat16 or float16)")
     p = _lib.NormParams()
@@ -43,6 +44,7 @@ def _params(x2, z2, weight, bias, eps, group_size, norm_before_gate):
     p.dtype = _DT[x2.dtype]
     p.has_z, p.has_bias, p.norm_before_gate = int(z2 is not None), int(bias is not None), int(bool(norm_before_gate))
     p.eps = float(eps)
+    p.layer_norm = int(not is_rms_norm)
     p.x, p.x_rs = x2.data_ptr(), x2.stride(0)
     if z2 is not None:
         p.z, p.z_rs = z2.data_ptr(), z2.stride(0)
@@ -52,24 +54,32 @@ def _params(x2, z2, weight, bias, eps, group_size, norm_before_gate):
     return p
 
 
-def _layer_norm_fwd(x, weight, bias, eps, z=None, group_size=None, norm_before_gate=True):
-    """x, z: (rows, cols) with unit stride along cols; weight, bias: (cols,) float32.  -> out, rstd (rows, ngroups)."""
+def _layer_norm_fwd(x, weight, bias, eps, z=None, group_size=None, norm_before_gate=True, is_rms_norm=True):
+    """x, z: (rows, cols) with unit stride along cols; weight, bias: (cols,) float32.  -> out, rstd (rows, ngroups) for the
+    RMS norm; out, mean, rstd for the LayerNorm (is_rms_norm=False)."""
     rows, cols = x.shape
     gs = group_size if group_size is not None else cols
     assert cols % gs == 0
     assert weight.shape == (cols,) and (bias is None or bias.shape == (cols,))
     assert z is None or z.shape == x.shape
-    p = _params(x, z, weight, bias, eps, group_size, norm_before_gate)
+    p = _params(x, z, weight, bias, eps, group_size, norm_before_gate, is_rms_norm)
     out = torch.empty((rows, cols), device=x.device, dtype=x.dtype)
     rstd = torch.empty((rows, cols // gs), device=x.device, dtype=torch.float32)
     p.out, p.out_rs, p.rstd = out.data_ptr(), out.stride(0), rstd.data_ptr()
+    mean = None
+    if not is_rms_norm:
+        mean = torch.empty_like(rstd)
+        p.mean = mean.data_ptr()
     _call("bimamba2_rmsnorm_gated_fwd", p, x.device)
-    return out, rstd
+    return (out, rstd) if is_rms_norm else (out, mean, rstd)
 
 
-def _layer_norm_bwd(dy, x, weight, bias, eps, rstd, z=None, group_size=None, norm_before_gate=True):
-    """-> dx, dweight (float32), dbias (float32 or None), dz (or None)."""
-    p = _params(x, z, weight, bias, eps, group_size, norm_before_gate)
+def _layer_norm_bwd(dy, x, weight, bias, eps, rstd, z=None, group_size=None, norm_before_gate=True, mean=None):
+    """-> dx, dweight (float32), dbias (float32 or None), dz (or None).  mean: the forward's group means (LayerNorm), None
+    for the RMS norm."""
+    p = _params(x, z, weight, bias, eps, group_size, norm_before_gate, mean is None)
+    if mean is not None:
+        p.mean = mean.data_ptr()
     dx = torch.empty_like(x, memory_format=torch.contiguous_format)
     dz = torch.empty_like(x, memory_format=torch.contiguous_format) if z is not None else None
     dw = torch.empty((x.shape[1],), device=x.device, dtype=torch.float32)
@@ -88,11 +98,10 @@ def _layer_norm_bwd(dy, x, weight, bias, eps, rstd, z=None, group_size=None, nor
 
 
 class LayerNormFn(torch.autograd.Function):
-    """RMS case of the reference's function of the same name (is_rms_norm is always True here)."""
+    """The reference's function of the same name: gated RMS norm (is_rms_norm=True) or gated LayerNorm."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True, is_rms_norm=True):
-        assert is_rms_norm, "only the RMS norm is built on the HIP kernels"
+    def forward(ctx, x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True, is_rms_norm=False):
         shape = x.shape
         x2 = _rows(x, "x")
         z2 = _rows(z, "z") if z is not None else None
@@ -103,8 +112,10 @@ class LayerNormFn(torch.autograd.Function):
         w32 = weight.detach().float().contiguous()
         b32 = bias.detach().float().contiguous() if bias is not None else None
         _require_gpu(w32, "weight")
-        out, rstd = _layer_norm_fwd(x2, w32, b32, eps, z=z2, group_size=group_size, norm_before_gate=norm_before_gate)
-        ctx.save_for_backward(x2, w32, b32, rstd, z2)
+        res = _layer_norm_fwd(x2, w32, b32, eps, z=z2, group_size=group_size, norm_before_gate=norm_before_gate,
+                              is_rms_norm=is_rms_norm)
+        out, rstd, mean = res[0], res[-1], (None if is_rms_norm else res[1])
+        ctx.save_for_backward(x2, w32, b32, rstd, z2, mean)
         ctx.shape, ctx.eps, ctx.group_size, ctx.norm_before_gate = shape, eps, group_size, norm_before_gate
         ctx.wdtype = weight.dtype
         ctx.bdtype = bias.dtype if bias is not None else None
@@ -113,12 +124,12 @@ class LayerNormFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
-        x2, w32, b32, rstd, z2 = ctx.saved_tensors
+        x2, w32, b32, rstd, z2, mean = ctx.saved_tensors
         dy2 = _rows(dy, "dy")
         if dy2.dtype != x2.dtype:
             dy2 = dy2.to(x2.dtype)
         dx, dw, db, dz = _layer_norm_bwd(dy2, x2, w32, b32, ctx.eps, rstd, z=z2, group_size=ctx.group_size,
-                                         norm_before_gate=ctx.norm_before_gate)
+                                         norm_before_gate=ctx.norm_before_gate, mean=mean)
         return (dx.reshape(ctx.shape), dw.to(ctx.wdtype), db.to(ctx.bdtype) if db is not None else None,
                 dz.reshape(ctx.shape).to(ctx.zdtype) if dz is not None else None, None, None, None, None)
 
@@ -126,8 +137,36 @@ class LayerNormFn(torch.autograd.Function):
 MAX_GROUP = 8192      # columns per normalisation group (bimamba2_rmsnorm_gated_fwd / _bwd refuse more)
 
 
+def layernorm_fn(x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True, is_rms_norm=False):
+    return LayerNormFn.apply(x, weight, bias, z, eps, group_size, norm_before_gate, is_rms_norm)
+
+
 def rmsnorm_fn(x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True):
     return LayerNormFn.apply(x, weight, bias, z, eps, group_size, norm_before_gate, True)
+
+
+class LayerNorm(torch.nn.Module):
+    """Same constructor, parameters (weight and bias) and forward as the reference's module (:388-412 there)."""
+
+    def __init__(self, hidden_size, eps=1e-5, group_size=None, norm_before_gate=True, device=None, dtype=None):
+        super().__init__()
+        if (group_size or hidden_size) > MAX_GROUP:
+            raise ValueError(f"LayerNorm: groups of {group_size or hidden_size} columns exceed the {MAX_GROUP} the kernels support")
+        self.eps = eps
+        self.weight = torch.nn.Parameter(torch.empty(hidden_size, device=device, dtype=dtype))
+        self.bias = torch.nn.Parameter(torch.empty(hidden_size, device=device, dtype=dtype))
+        self.group_size = group_size
+        self.norm_before_gate = norm_before_gate
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        torch.nn.init.ones_(self.weight)
+        torch.nn.init.zeros_(self.bias)
+
+    def forward(self, x, z=None):
+        """norm(x) * silu(z) if norm_before_gate, else norm(x * silu(z)); plain norm without z."""
+        return layernorm_fn(x, self.weight, self.bias, z=z, eps=self.eps, group_size=self.group_size,
+                            norm_before_gate=self.norm_before_gate)
 
 
 class RMSNorm(torch.nn.Module):

@@ -247,7 +247,8 @@ typedef struct bimamba2_norm_params {
     int32_t dtype;              /* BIMAMBA2_*: x, z, out, dout, dx, dz */
     int32_t has_z, has_bias, norm_before_gate;
     float eps;
-    int32_t reserved0;
+    int32_t layer_norm;         /* 0: RMS norm (the BiMamba2 layer's);  1: LayerNorm - the group's mean is subtracted first
+                                   (is_rms_norm = False of the reference, same kernels there) and kept in `mean` */
     int64_t x_rs, z_rs, out_rs, dout_rs, dx_rs, dz_rs;
     const void *x, *z;
     const float *weight, *bias; /* (cols,) float32 */
@@ -259,6 +260,8 @@ typedef struct bimamba2_norm_params {
     void *workspace;            /* backward only: bimamba2_rmsnorm_gated_workspace_bytes() */
     size_t workspace_bytes;
     void *stream;               /* hipStream_t */
+    float *mean;                /* layer_norm only: (rows, cols / group_size) float32, written by the forward (optional
+                                   there), read by the backward */
 } bimamba2_norm_params;
 
 size_t bimamba2_norm_params_size(void);

@@ -14,13 +14,17 @@ import torch
 import torch.nn.functional as F
 
 
-def rms_norm_gated(x, weight, bias=None, z=None, eps=1e-6, group_size=None, norm_before_gate=True):
+def rms_norm_gated(x, weight, bias=None, z=None, eps=1e-6, group_size=None, norm_before_gate=True, is_rms_norm=True):
+    """is_rms_norm=False: the LayerNorm of the same reference kernels (IS_RMS_NORM = False,
+    src/ssd/bi/layernorm_gated.py:66-76 there) - the group mean is subtracted before the mean of squares is taken."""
     if z is not None and not norm_before_gate:
         x = x * F.silu(z)
     n = x.shape[-1]
     gs = n if group_size is None else group_size
     assert n % gs == 0
     xg = x.reshape(*x.shape[:-1], n // gs, gs)
+    if not is_rms_norm:
+        xg = xg - xg.mean(dim=-1, keepdim=True)
     rstd = 1.0 / torch.sqrt(xg.square().mean(dim=-1, keepdim=True) + eps)
     out = (xg * rstd).reshape(x.shape) * weight
     if bias is not None:

@@ -1,2 +1,2 @@
 """Drop-in for the reference module of the same path (RMS norm only): names come from bi_mamba2_amd.layernorm_gated."""
-from bi_mamba2_amd.layernorm_gated import LayerNormFn, RMSNorm, rmsnorm_fn  # noqa: F401
+from bi_mamba2_amd.layernorm_gated import LayerNorm, LayerNormFn, RMSNorm, layernorm_fn, rmsnorm_fn  # noqa: F401

@@ -1,4 +1,5 @@
-"""GPU parity of the gated RMS norm (forward and backward, through the C ABI) against the float64 oracle."""
+"""GPU parity of the gated RMS norm and of the gated LayerNorm (forward and backward, through the C ABI) against the
+float64 oracle."""
 import pytest
 import torch
 
@@ -22,23 +23,28 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("rms", [True, False], ids=["rmsnorm", "layernorm"])
 @pytest.mark.parametrize("case", CASES)
-def test_rmsnorm_gated_forward_backward(case):
-    from bi_mamba2_amd.layernorm_gated import rmsnorm_fn
+def test_rmsnorm_gated_forward_backward(case, rms):
+    from bi_mamba2_amd.layernorm_gated import layernorm_fn
     shape, gs, with_z, with_b, before, dtype = case
     g = torch.Generator().manual_seed(3)
     n = shape[-1]
-    x = torch.randn(shape, generator=g).to(dtype)
+    x = torch.randn(shape, generator=g)
+    if not rms:
+        x = x + 0.75                     # a mean worth subtracting
+    x = x.to(dtype)
     z = torch.randn(shape, generator=g).to(dtype) if with_z else None
     w = (1.0 + 0.3 * torch.randn(n, generator=g)).float()
     b = (0.2 * torch.randn(n, generator=g)).float() if with_b else None
     dy = torch.randn(shape, generator=g).to(dtype)
     leaves = [t.cuda().requires_grad_(True) if t is not None else None for t in (x, w, b, z)]
-    out = rmsnorm_fn(leaves[0], leaves[1], leaves[2], z=leaves[3], eps=1e-5, group_size=gs, norm_before_gate=before)
+    out = layernorm_fn(leaves[0], leaves[1], leaves[2], z=leaves[3], eps=1e-5, group_size=gs, norm_before_gate=before, is_rms_norm=rms)
     assert out.dtype == dtype and out.shape == tuple(shape)
     out.backward(dy.cuda())
     ref_leaves = [t.double().requires_grad_(True) if t is not None else None for t in (x, w, b, z)]
-    ref = rms_norm_gated(ref_leaves[0], ref_leaves[1], ref_leaves[2], ref_leaves[3], eps=1e-5, group_size=gs, norm_before_gate=before)
+    ref = rms_norm_gated(ref_leaves[0], ref_leaves[1], ref_leaves[2], ref_leaves[3], eps=1e-5, group_size=gs, norm_before_gate=before,
+                         is_rms_norm=rms)
     ref.backward(dy.double())
     assert_close(out, ref.detach(), dtype, "out")
     for got, r, name in zip(leaves, ref_leaves, ("dx", "dweight", "dbias", "dz")):
@@ -58,6 +64,28 @@ def test_rmsnorm_strided_rows_and_module():
     out = m(x, z)
     ref = rms_norm_gated(x.double().cpu(), m.weight.detach().double().cpu(), None, z.double().cpu(), eps=1e-5)
     assert_close(out, ref, torch.float32, "out (strided)")
+
+
+def test_layernorm_module():
+    """The LayerNorm module (weight and bias parameters), gated, against the oracle."""
+    from bi_mamba2_amd.layernorm_gated import LayerNorm
+    g = torch.Generator().manual_seed(6)
+    x, z = (torch.randn(3, 20, 96, generator=g) + 1.5).cuda(), torch.randn(3, 20, 96, generator=g).cuda()
+    m = LayerNorm(96, eps=1e-5, group_size=32, norm_before_gate=False, device="cuda")
+    with torch.no_grad():
+        m.weight.copy_(1.0 + 0.1 * torch.randn(96, generator=g))
+        m.bias.copy_(0.1 * torch.randn(96, generator=g))
+    x.requires_grad_(True)
+    out = m(x, z)
+    out.sum().backward()
+    xr = x.detach().double().cpu().requires_grad_(True)
+    wr, br = m.weight.detach().double().cpu().requires_grad_(True), m.bias.detach().double().cpu().requires_grad_(True)
+    ref = rms_norm_gated(xr, wr, br, z.double().cpu(), eps=1e-5, group_size=32, norm_before_gate=False, is_rms_norm=False)
+    ref.sum().backward()
+    assert_close(out, ref.detach(), torch.float32, "out")
+    assert_close(x.grad, xr.grad, torch.float32, "dx")
+    assert_close(m.weight.grad, wr.grad, torch.float32, "dweight")
+    assert_close(m.bias.grad, br.grad, torch.float32, "dbias")
 
 
 def test_rmsnorm_refuses_cpu_tensors_and_bad_groups():

@@ -64,3 +64,22 @@ def test_gradcheck():
     x, w, b, z = (t.requires_grad_(True) for t in (_rand(2, 8), _rand(8, seed=1), _rand(8, seed=2), _rand(2, 8, seed=3)))
     for before in (True, False):
         assert torch.autograd.gradcheck(lambda a, c, d, e: rms_norm_gated(a, c, d, e, 1e-5, 4, before), (x, w, b, z))
+
+
+# ---- the LayerNorm of the same reference kernels (is_rms_norm=False) ----
+def test_layer_norm_matches_torch_layer_norm_and_group_norm():
+    x, w, b = _rand(5, 48), _rand(48, seed=1), _rand(48, seed=2)
+    ref = F.layer_norm(x, (48,), weight=w, bias=b, eps=1e-5)
+    torch.testing.assert_close(rms_norm_gated(x, w, b, eps=1e-5, is_rms_norm=False), ref, rtol=1e-12, atol=1e-12)
+    # groups of 12 columns = torch's group norm with 4 groups over the channel axis
+    refg = F.group_norm(x, 4, weight=w, bias=b, eps=1e-5)
+    torch.testing.assert_close(rms_norm_gated(x, w, b, eps=1e-5, group_size=12, is_rms_norm=False), refg, rtol=1e-12, atol=1e-12)
+
+
+def test_layer_norm_is_shift_invariant_and_gates_by_definition():
+    x, w, z = _rand(4, 32), _rand(32, seed=1), _rand(4, 32, seed=2)
+    ln = lambda t: rms_norm_gated(t, w, eps=1e-6, is_rms_norm=False)   # noqa: E731
+    torch.testing.assert_close(ln(x + 3.25), ln(x), rtol=1e-10, atol=1e-10)          # the RMS norm is not: see below
+    assert (rms_norm_gated(x + 3.25, w, eps=1e-6) - rms_norm_gated(x, w, eps=1e-6)).abs().max() > 0.1
+    torch.testing.assert_close(rms_norm_gated(x, w, z=z, norm_before_gate=True, is_rms_norm=False), ln(x) * F.silu(z), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(rms_norm_gated(x, w, z=z, norm_before_gate=False, is_rms_norm=False), ln(x * F.silu(z)), rtol=1e-12, atol=1e-12)
