@@ -21,6 +21,7 @@ from ._lib import Params
 
 _DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
 _INF = float("inf")
+MAX_CHUNK_SIZE, MAX_HEADDIM = 256, 128     # BIMAMBA2_MAX_CHUNK, BIMAMBA2_MAX_HEADDIM of include/bimamba2.h
 
 
 def _require_gpu(t, name):
@@ -723,7 +724,7 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
         A: (nheads)
         B: (batch, seqlen, ngroups, dstate)
         C: (batch, seqlen, ngroups, dstate)
-        chunk_size: int, 32..256
+        chunk_size: int, at least 32 (above 256 the kernels use 256: the result does not depend on it)
         D: (nheads, headdim) or (nheads,)
         z: (batch, seqlen, nheads, headdim)
         dt_bias: (nheads,)
@@ -741,6 +742,28 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
         out: (batch, seqlen, nheads, headdim), or (out, final_states_f, final_states_b) with
         return_final_states=True (final states are (batch, nheads, headdim, dstate) float32)
     """
+    # The result does not depend on the chunk size (it only sets where the kernels cut the sequence), and the kernels'
+    # chunks hold at most 256 positions: a larger chunk_size, which the reference accepts, runs with 256.
+    chunk_size = min(chunk_size, MAX_CHUNK_SIZE)
+    headdim = x.shape[-1]
+    if headdim > MAX_HEADDIM:
+        # The channels of a head only share dt, A and the head's group, so a head wider than the kernels' 128 channels
+        # is computed as several narrower heads with the same dt, A, dt_bias (and D), side by side in the same group.
+        # Everything here is differentiable torch glue: autograd sums the pieces' gradients of dt, A, dt_bias and D.
+        parts = next((k for k in range(2, headdim + 1) if headdim % k == 0 and headdim // k <= MAX_HEADDIM), None)
+        assert parts is not None
+        batch, seqlen, nheads, _ = x.shape
+        narrow = lambda t: t.reshape(*t.shape[:-2], nheads * parts, headdim // parts) if t is not None else None
+        rep = lambda t, dim: t.repeat_interleave(parts, dim=dim) if t is not None else None
+        res = bimamba_chunk_scan_combined(
+            narrow(x), rep(dt, 2), rep(A, 0), B, C, chunk_size, D=(narrow(D) if D is not None and D.dim() == 2 else rep(D, 0)),
+            z=narrow(z), dt_bias=rep(dt_bias, 0), dt_softplus=dt_softplus, dt_limit=dt_limit, return_final_states=return_final_states,
+            initial_states_f=(initial_states_f.reshape(batch, nheads * parts, headdim // parts, -1) if initial_states_f is not None else None),
+            initial_states_b=(initial_states_b.reshape(batch, nheads * parts, headdim // parts, -1) if initial_states_b is not None else None),
+            seq_idx=seq_idx)
+        if not return_final_states:
+            return res.reshape(x.shape)
+        return (res[0].reshape(x.shape),) + tuple(t.reshape(batch, nheads, headdim, -1) for t in res[1:])
     if initial_states_f is None and initial_states_b is None and seq_idx is None:
         return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
                                               return_final_states)

@@ -1,5 +1,6 @@
 """GPU parity on the smallest and most ragged shapes: one position, a sequence shorter than a chunk on the fast-path
-kernels (one partly filled chunk), a last chunk of one position, forward and backward."""
+kernels (one partly filled chunk), a last chunk of one position, forward and backward; and the shapes beyond the kernels'
+limits that the public function takes apart (heads wider than 128 channels, chunks longer than 256)."""
 import pytest
 import torch
 
@@ -37,6 +38,48 @@ def test_tiny_and_ragged_shapes(case):
     for k in ("x", "B", "C", "z", "dt", "A", "D", "dt_bias"):
         if ref["d" + k] is not None:
             assert_close(leaves[k].grad, ref["d" + k], dtype, "d" + k, scaled=is_reduced("d" + k, dtype))
+
+
+WIDE = [
+    # batch, seqlen, H, P, G, N, chunk, dtype, z, D with headdim, final states
+    (2, 100, 2, 256, 1, 16, 64, torch.float32, True, True, False),       # heads of 256 channels: two pieces of 128
+    (1, 300, 4, 192, 2, 64, 128, torch.bfloat16, False, False, True),    # 192 channels: two pieces of 96; final states
+    (1, 700, 2, 64, 1, 32, 512, torch.float32, True, False, False),      # chunk_size above the kernels' 256
+]
+
+
+@pytest.mark.parametrize("case", WIDE)
+def test_heads_wider_and_chunks_longer_than_the_kernels(case):
+    """Shapes the reference accepts beyond the kernels' limits (headdim > 128, chunk_size > 256): the public function
+    splits wide heads into narrower ones that share dt, A, dt_bias (and D) and caps the chunk size (the result does not
+    depend on it); output, final states and every gradient against the oracle at the shape the caller gave."""
+    from bi_mamba2_amd import ops
+    b, L, H, P, G, N, Q, dtype, z, Dhp, fin = case
+    inp = make_case(b, L, H, P, G, N, dtype, with_z=z, D_has_hdim=Dhp)
+    d = to_dev(inp)
+    leaves = {k: (v.clone().requires_grad_(True) if v is not None else None) for k, v in d.items()}
+    res = ops.bimamba_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], Q, D=leaves["D"],
+                                          z=leaves["z"], dt_bias=leaves["dt_bias"], dt_softplus=True, return_final_states=fin)
+    out = res[0] if fin else res
+    assert out.shape == (b, L, H, P)
+    dout = torch.randn(out.shape, generator=torch.Generator().manual_seed(5)).to(out.dtype)
+    out.backward(dout.cuda())
+    r = to64(inp)
+    ref = O.bimamba2_grads(dout.double(), r["x"], r["dt"], r["A"], r["B"], r["C"], D=r["D"], z=r["z"], dt_bias=r["dt_bias"],
+                           dt_softplus=True)
+    assert_close(out, ref["out"], dtype, "out")
+    if fin:
+        assert res[1].shape == (b, H, P, N) and res[2].shape == (b, H, P, N)
+        rf = O.bimamba2_sequential(r["x"], r["dt"], r["A"], r["B"], r["C"], D=r["D"], z=r["z"], dt_bias=r["dt_bias"], dt_softplus=True)
+        assert_close(res[1], rf[2], dtype, "final_f")
+        assert_close(res[2], rf[3], dtype, "final_b")
+    for k in ("x", "B", "C", "z", "dt", "A", "D", "dt_bias"):
+        if ref["d" + k] is not None:
+            assert leaves[k].grad.shape == leaves[k].shape
+            # (dx of the 16-bit case: sums of up to 22 from operands with 8 bits of mantissa leave one element in 230000
+            # at 1.17 x the plain bound; the criterion of the summed gradients, as in test_gpu_scan16_shapes.py)
+            assert_close(leaves[k].grad, ref["d" + k], dtype, "d" + k,
+                         scaled=is_reduced("d" + k, dtype) or (k == "x" and dtype != torch.float32))
 
 
 BIG = [
