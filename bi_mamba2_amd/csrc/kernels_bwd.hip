@@ -1459,6 +1459,7 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
         auto run = [&](auto KC) __attribute__((always_inline)) {
             constexpr int KIND = decltype(KC)::value;
             constexpr bool DIAG = KIND >= 0;
+            constexpr bool LOWER = KIND == -1;             // off the diagonal: -1 below it (forward direction), -2 above
         for (int it = 0; it < nit; ++it) {
             // with two slots nothing but step `it` is outstanding here; with more, the requests of step `it` went out before
             // those of the step after it (waves 0 and 1 make five requests per step, the others four)
@@ -1501,21 +1502,36 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
             }
             if (++kc == nkc) {
                 kc = 0;
-                // ---- decay vectors of this head
-                f32x4 cft_ = raw_lds_read_at<f32x4, 0>(sb + ct_off), cbt_ = raw_lds_read_at<f32x4, 256>(sb + ct_off);
-                float cfs[4], cbs[4], dts[4];
-                cfs[0] = raw_lds_read_at<float, 512>(sb + cc_off); cfs[1] = raw_lds_read_at<float, 512 + 64>(sb + cc_off);
-                cfs[2] = raw_lds_read_at<float, 512 + 128>(sb + cc_off); cfs[3] = raw_lds_read_at<float, 512 + 192>(sb + cc_off);
-                cbs[0] = raw_lds_read_at<float, 768>(sb + cc_off); cbs[1] = raw_lds_read_at<float, 768 + 64>(sb + cc_off);
-                cbs[2] = raw_lds_read_at<float, 768 + 128>(sb + cc_off); cbs[3] = raw_lds_read_at<float, 768 + 192>(sb + cc_off);
+                // ---- decay vectors of this head (off the diagonal only the ones of the tile's direction)
+                f32x4 cft_, cbt_;
+                float cfs[4], cbs[4], dts[4], mf, mb;
+                if constexpr (DIAG || LOWER) {
+                    cft_ = raw_lds_read_at<f32x4, 0>(sb + ct_off);
+                    cfs[0] = raw_lds_read_at<float, 512>(sb + cc_off); cfs[1] = raw_lds_read_at<float, 512 + 64>(sb + cc_off);
+                    cfs[2] = raw_lds_read_at<float, 512 + 128>(sb + cc_off); cfs[3] = raw_lds_read_at<float, 512 + 192>(sb + cc_off);
+                    mf = raw_lds_read_at<float, 0>(sb + cm_off);           // reference point: cs_f at the first of the wave's 16 rows
+                }
+                if constexpr (DIAG || !LOWER) {
+                    cbt_ = raw_lds_read_at<f32x4, 256>(sb + ct_off);
+                    cbs[0] = raw_lds_read_at<float, 768>(sb + cc_off); cbs[1] = raw_lds_read_at<float, 768 + 64>(sb + cc_off);
+                    cbs[2] = raw_lds_read_at<float, 768 + 128>(sb + cc_off); cbs[3] = raw_lds_read_at<float, 768 + 192>(sb + cc_off);
+                    mb = raw_lds_read_at<float, 256 + 60>(sb + cm_off);    // cs_b at the last of them
+                }
                 dts[0] = raw_lds_read_at<float, 1024>(sb + cc_off); dts[1] = raw_lds_read_at<float, 1024 + 64>(sb + cc_off);
                 dts[2] = raw_lds_read_at<float, 1024 + 128>(sb + cc_off); dts[3] = raw_lds_read_at<float, 1024 + 192>(sb + cc_off);
-                // reference points: cs_f at the first, cs_b at the last of the wave's 16 rows
-                float mf = raw_lds_read_at<float, 0>(sb + cm_off), mb = raw_lds_read_at<float, 256 + 60>(sb + cm_off);
                 raw_lds_wait();
-                raw_lds_use(cft_); raw_lds_use(cbt_); raw_lds_use(mf); raw_lds_use(mb);
+                if constexpr (DIAG || LOWER) {
+                    raw_lds_use(cft_); raw_lds_use(mf);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) { raw_lds_use(cfs[j]); raw_lds_use(cbs[j]); raw_lds_use(dts[j]); }
+                    for (int j = 0; j < 4; ++j) raw_lds_use(cfs[j]);
+                }
+                if constexpr (DIAG || !LOWER) {
+                    raw_lds_use(cbt_); raw_lds_use(mb);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) raw_lds_use(cbs[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) raw_lds_use(dts[j]);
                 if (rows_left < 4) {
                     // rows past the end of the sequence were read from a valid row: drop them
 #pragma unroll
@@ -1540,13 +1556,13 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
                     col = cp * Fd;
                 };
                 if constexpr (!DIAG) {
-                    const bool lower = st < tt;                // forward direction below the diagonal, reverse above it
+                    // forward direction below the diagonal, reverse above it
                     float E[4], rp[4] = {0.f, 0.f, 0.f, 0.f};
-                    const float ml = (lower ? mf : mb) * LOG2E;
+                    const float ml = (LOWER ? mf : mb) * LOG2E;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) E[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(lower ? cft_[i] : cbt_[i], LOG2E, -ml));
+                    for (int i = 0; i < 4; ++i) E[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(LOWER ? cft_[i] : cbt_[i], LOG2E, -ml));
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) sep_block(j, E, dts[j] * __builtin_amdgcn_exp2f(__builtin_fmaf(lower ? cfs[j] : cbs[j], -LOG2E, ml)), colF[j], rp);
+                    for (int j = 0; j < 4; ++j) sep_block(j, E, dts[j] * __builtin_amdgcn_exp2f(__builtin_fmaf(LOWER ? cfs[j] : cbs[j], -LOG2E, ml)), colF[j], rp);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) rowF[i] = rp[i] * E[i];
                 } else {
@@ -1619,7 +1635,8 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
             slot2 = slot2 + 1 == DCB_RING ? 0 : slot2 + 1;
         }
         };
-        if (st != tt) run(std::integral_constant<int, -1>());
+        if (st < tt) run(std::integral_constant<int, -1>());
+        else if (st > tt) run(std::integral_constant<int, -2>());
         else if (wave == 0) run(std::integral_constant<int, 0>());
         else if (wave == 1) run(std::integral_constant<int, 1>());
         else if (wave == 2) run(std::integral_constant<int, 2>());
