@@ -97,15 +97,30 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dz_kernel(const bimamba2_params 
     const T *ox = reinterpret_cast<const T *>(p.out_x);
     T *dz = reinterpret_cast<T *>(p.dz);
     T *dox = reinterpret_cast<T *>(p.dout_x);
+    // z and dout laid out like out_x (rows of headdim one behind the other, headdim a multiple of the vector): a vector
+    // unit's offset is the same in all of them and no index has to be taken apart (three 64-bit divisions per unit, most of
+    // the kernel's instructions otherwise)
+    const bool packed = P % VS == 0 && p.z_sh == P && p.z_sl == (int64_t)p.nheads * P && p.z_sb == (int64_t)p.seqlen * p.nheads * P &&
+                        p.dout_sh == P && p.dout_sl == p.z_sl && p.dout_sb == p.z_sb;
     for (int64_t idx = blockIdx.x * (int64_t)NTHREADS + threadIdx.x; idx < nrows * pv; idx += (int64_t)gridDim.x * NTHREADS) {
-        const int64_t row = idx / pv;
-        const int c0 = (int)(idx - row * pv) * VS;
-        const int h = (int)(row % p.nheads);
-        const int64_t bl = row / p.nheads;
-        const int l = (int)(bl % p.seqlen), b = (int)(bl / p.seqlen);
-        const T *zp = zb + b * p.z_sb + l * p.z_sl + h * p.z_sh + c0;
-        const T *dp = db + b * p.dout_sb + l * p.dout_sl + h * p.dout_sh + c0;
-        const int64_t o = row * P + c0;
+        const T *zp, *dp;
+        int64_t o;
+        int c0;
+        if (packed) {
+            o = idx * VS;
+            c0 = 0;                               // (only its distance from the row's end matters below: a whole vector fits)
+            zp = zb + o;
+            dp = db + o;
+        } else {
+            const int64_t row = idx / pv;
+            c0 = (int)(idx - row * pv) * VS;
+            const int h = (int)(row % p.nheads);
+            const int64_t bl = row / p.nheads;
+            const int l = (int)(bl % p.seqlen), b = (int)(bl / p.seqlen);
+            zp = zb + b * p.z_sb + l * p.z_sl + h * p.z_sh + c0;
+            dp = db + b * p.dout_sb + l * p.dout_sl + h * p.dout_sh + c0;
+            o = row * P + c0;
+        }
         const bool vec = (c0 + VS <= P) && aligned16(zp, 0) && aligned16(dp, 0) && aligned16(ox + o, 0);
         float zv[VS], dv[VS], ov[VS];
         if (vec) {
