@@ -72,7 +72,14 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     // needs no float32 states at all
     const bool copies = bimamba2_state_copies(q) != 0;
     const bool saved_copies = is_bwd && q->fwd_saved && q->states16_f;
-    if (copies && !q->states_f && !q->states16_f) {
+    // a forward pass whose caller keeps no states (no pointer given for them) has one reader of the entering states, the scan
+    // kernel, and every 16-bit scan kernel reads the copies: the state passing then writes half the bytes, the scan reads half
+    // (under the conditions of the state-passing kernel that writes them)
+    auto al16 = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+    const bool fwd_only_copies = !is_bwd && !q->causal && (q->dtype == BIMAMBA2_BF16 || q->dtype == BIMAMBA2_F16) &&
+                                 (q->headdim * q->dstate) % 4 == 0 && al16(q->final_f) && al16(q->final_b) &&
+                                 al16(q->initial_f) && al16(q->initial_b) && !q->states_b && !q->states16_b;
+    if ((copies || fwd_only_copies) && !q->states_f && !q->states16_f) {
         q->states16_f = cv.take<char>(stn * 2);
         q->states16_b = cv.take<char>(stn * 2);
     }

@@ -257,8 +257,14 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                 __syncthreads();
                 load_arows(n0);
             }
-            tile_load_kcontig<T, float, PW, NW>(sF, stf + n0, N, P - p0, N - n0, Ident());
-            tile_load_kcontig<T, float, PW, NW>(sB, stb + n0, N, P - p0, N - n0, Ident());
+            if (sizeof(T) == 2 && !BWD && p.states16_f) {
+                // the 16-bit copies of the entering states (a forward pass whose caller keeps no states: half the bytes)
+                tile_load_kcontig<T, T, PW, NW>(sF, reinterpret_cast<const T *>(p.states16_f) + so + n0, N, P - p0, N - n0, Ident());
+                tile_load_kcontig<T, T, PW, NW>(sB, reinterpret_cast<const T *>(p.states16_b) + so + n0, N, P - p0, N - n0, Ident());
+            } else {
+                tile_load_kcontig<T, float, PW, NW>(sF, stf + n0, N, P - p0, N - n0, Ident());
+                tile_load_kcontig<T, float, PW, NW>(sB, stb + n0, N, P - p0, N - n0, Ident());
+            }
             __syncthreads();
 #pragma unroll
             for (int s = 0; s < NW / KSTEP; ++s) {
@@ -721,7 +727,8 @@ static int launch_scan_t(const bimamba2_params *p) {
             return check_launch();
         }
     }
-    if (p->causal || c16f) return BIMAMBA2_EUNSUPPORTED;
+    // (the kernels below read the forward pass's 16-bit copies of the entering states too, but not the mirror's)
+    if (p->causal || (c16f && (BWD || sizeof(T) != 2))) return BIMAMBA2_EUNSUPPORTED;
     if ((BWD ? p->CBT : p->CB) == nullptr) return BIMAMBA2_EINVAL;
     if (pw == 16) { if (qt == 1) BM2_SCAN(1, 1); else BM2_SCAN(2, 1); }
     else if (pw == 32) { if (qt == 1) BM2_SCAN(1, 2); else BM2_SCAN(2, 2); }

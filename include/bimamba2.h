@@ -127,10 +127,14 @@ typedef struct bimamba2_params {
        from there.  dstates16_f / dstates16_b likewise: written by bimamba2_state_passing_bwd (dstates_f / dstates_b keep
        the per-chunk gradients), read by bimamba2_chunk_scan_bwd_dx and bimamba2_chunk_state_bwd_db.  Only the kernels for
        16-bit dtype, dstate 64, headdim % 64 == 0, chunk_size % 64 == 0 and 16-byte aligned operands know them
-       (bimamba2_state_copies() == 1); the others return BIMAMBA2_EUNSUPPORTED when they are set.
+       (bimamba2_state_copies() == 1); the others return BIMAMBA2_EUNSUPPORTED when they are set - except the two
+       forward stages: bimamba2_state_passing_fwd writes, and bimamba2_chunk_scan_fwd reads, states16_* for every 16-bit
+       problem with headdim * dstate % 4 == 0 and 16-byte aligned state tensors.
        bimamba2_fwd / bimamba2_bwd use such copies on their own, from the workspace, where the caller leaves states_f
        resp. dstates_f NULL (does not ask for the float32 entering states); a caller that keeps the forward's intermediates
        for the backward pass (fwd_saved) then passes states16_f / states16_b to both instead of states_f / states_b.
+       bimamba2_fwd does so for every 16-bit problem (a forward pass without kept states has the scan stage as the only
+       reader), bimamba2_bwd where bimamba2_state_copies() == 1.
        The reference keeps its entering states in the input dtype as well (out_dtype=C.dtype, src/ssd/bi/ssd_combined.py:324-327). */
     void *states16_f, *states16_b;
     void *dstates16_f, *dstates16_b;
