@@ -1799,12 +1799,20 @@ int launch_bwd_dcb(const bimamba2_params *p) {
 // of a thread (its dCB row pieces, the slices it adds, the K operand) is requested before the first one is used.
 
 
-template <typename T, int QP, bool FAST>
+// SLIM (with FAST): dCB / dCBT hold 16-bit elements (in16) and there are at most two slices to add: a quarter of the
+// registers, and the staging tile of the result shares the LDS of the K operand, so that three workgroups fit a CU where
+// the general variant fits two (with few heads per group the launch has thousands of workgroups: 83 -> 76 us at 8 groups
+// of 4 heads, batch 4 x 4096, where the launch moves 250 MB).
+template <typename T, int QP, bool FAST, bool SLIM = false>
 __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int nc, int nslices, BlockId bid, bool in16 = false) {
     typedef Mma<T> M;
     constexpr int KPL = M::KPL, KSTEP = M::KSTEP;
     constexpr int LDX = QP + 16 / (int)sizeof(T);
-    __shared__ __attribute__((aligned(16))) T kT[64 * LDX];
+    constexpr int SLD = 64 + 4;
+    constexpr int KT_BYTES = 64 * LDX * (int)sizeof(T), STG_BYTES = 64 * SLD * 4;
+    __shared__ __attribute__((aligned(16))) unsigned char bmm_lds[SLIM ? (KT_BYTES > STG_BYTES ? KT_BYTES : STG_BYTES) : KT_BYTES + STG_BYTES];
+    T *kT = reinterpret_cast<T *>(bmm_lds);
+    float *stg = reinterpret_cast<float *>(bmm_lds + (SLIM ? 0 : KT_BYTES));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lr = lane & 15, lg = lane >> 4;
     const int nt = bid.x, rt = bid.y;
@@ -1821,18 +1829,17 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
     const float *res = which == 0 ? p.dBs : p.dCs;
     T *out = reinterpret_cast<T *>(which == 0 ? p.dB : p.dC);
     const int64_t slice = (int64_t)p.batch * p.seqlen * p.ngroups * N;
-    constexpr int VS = 16 / (int)sizeof(T), SLD = 64 + 4;
-    __shared__ __attribute__((aligned(16))) float stg[64 * SLD];
+    constexpr int VS = 16 / (int)sizeof(T);
     if constexpr (FAST) {
-        constexpr int NS = QP / KSTEP, NIT = 64 * (64 / VS) / NTHREADS, MAXSL = 8;
+        constexpr int NS = QP / KSTEP, NIT = 64 * (64 / VS) / NTHREADS, MAXSL = SLIM ? 2 : 8;
         // in16: dCB / dCBT hold elements of type T (written that way by the dCB kernel inside bimamba2_bwd): a row piece is
         // the MFMA operand as it lies in memory
-        float4 raw[NS][2];
-        if (in16) {
+        float4 raw[NS][SLIM ? 1 : 2];
+        if (SLIM || in16) {
             const T *arow16 = reinterpret_cast<const T *>(which == 0 ? p.dCBT : p.dCB) + (int64_t)bcg * Q * Q + (int64_t)min(r0 + wave * 16 + lr, Q - 1) * Q;
 #pragma unroll
             for (int s = 0; s < NS; ++s) raw[s][0] = *reinterpret_cast<const float4 *>(arow16 + s * KSTEP + lg * KPL);
-        } else {
+        } else if constexpr (!SLIM) {
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 raw[s][0] = *reinterpret_cast<const float4 *>(arow + s * KSTEP + lg * KPL);
@@ -1863,10 +1870,15 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             if (s * KSTEP < limit) {
-                float v[KPL] = {raw[s][0].x, raw[s][0].y, raw[s][0].z, raw[s][0].w, raw[s][1].x, raw[s][1].y, raw[s][1].z, raw[s][1].w};
                 typename M::Frag af;
-                if constexpr (sizeof(typename M::Frag) == 16) af = in16 ? __builtin_bit_cast(typename M::Frag, raw[s][0]) : M::pack(v);
-                else af = M::pack(v);
+                if constexpr (SLIM) {
+                    static_assert(!SLIM || sizeof(typename M::Frag) == 16, "16-bit operands");
+                    af = __builtin_bit_cast(typename M::Frag, raw[s][0]);
+                } else {
+                    float v[KPL] = {raw[s][0].x, raw[s][0].y, raw[s][0].z, raw[s][0].w, raw[s][1].x, raw[s][1].y, raw[s][1].z, raw[s][1].w};
+                    if constexpr (sizeof(typename M::Frag) == 16) af = in16 ? __builtin_bit_cast(typename M::Frag, raw[s][0]) : M::pack(v);
+                    else af = M::pack(v);
+                }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[j] = M::mma(af, M::load(kT + xt_index<T, LDX>(j * 16 + lr, s * KSTEP + lg * KPL)), acc[j]);
             }
@@ -1880,6 +1892,7 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
                 sw[it][sl][0] = *reinterpret_cast<const float4 *>(q);
                 sw[it][sl][1] = *reinterpret_cast<const float4 *>(q + 4);
             }
+        if constexpr (SLIM) __syncthreads();       // every wave is done with the K operand, whose LDS the staging tile shares
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -2166,13 +2179,13 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_bwd_kernel(const bimamb
 // The last two kernels of the backward pass in one launch: the first `nbmm` workgroups do the work of
 // bmm_chunk_bwd_kernel (16-bit path, chunk_size 256), the others that of chunk_cumsum_bwd_kernel.  Neither depends on the
 // other, both are short and latency-bound, and together they fit the machine in one wave of workgroups.
-template <typename T, typename DT>
+template <typename T, typename DT, bool SLIM = false>
 __global__ __launch_bounds__(NTHREADS) void bwd_tail_kernel(const bimamba2_params p, int nc, int nslices, int nqt, int nsplit, int nbmm,
                                                             int bmm_gy, int cs_gx, bool in16) {
     const int id = blockIdx.x;
     if (id < nbmm) {
         // bmm grid (1, bmm_gy, z)
-        bmm_chunk_bwd_body<T, 256, true>(p, nc, nslices, BlockId{0, id % bmm_gy, id / bmm_gy}, in16);
+        bmm_chunk_bwd_body<T, 256, true, SLIM>(p, nc, nslices, BlockId{0, id % bmm_gy, id / bmm_gy}, in16);
     } else {
         const int k = id - nbmm;                  // cumsum grid (cs_gx, nc, batch)
         chunk_cumsum_bwd_body<DT>(p, nc, nqt, nsplit, BlockId{k % cs_gx, (k / cs_gx) % nc, k / (cs_gx * nc)});
@@ -2197,6 +2210,15 @@ static int launch_bwd_tail_t(const bimamba2_params *p, int nc, int nqt, int nspl
     const int cs_gx = (p->nheads + 3) / 4, ncs = cs_gx * nc * p->batch;
     dim3 grid(nbmm + ncs);
     const int nsl = dbdc_slices(p);
+    if (in16 && nsl <= 2) {
+        switch (p->dt_dtype) {
+            case BIMAMBA2_F32: hipLaunchKernelGGL((bwd_tail_kernel<T, float, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx, in16); break;
+            case BIMAMBA2_BF16: hipLaunchKernelGGL((bwd_tail_kernel<T, bf16_t, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx, in16); break;
+            case BIMAMBA2_F16: hipLaunchKernelGGL((bwd_tail_kernel<T, f16_t, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx, in16); break;
+            default: return BIMAMBA2_EUNSUPPORTED;
+        }
+        return check_launch();
+    }
     switch (p->dt_dtype) {
         case BIMAMBA2_F32: hipLaunchKernelGGL((bwd_tail_kernel<T, float>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx, in16); break;
         case BIMAMBA2_BF16: hipLaunchKernelGGL((bwd_tail_kernel<T, bf16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsl, nqt, nsplit, nbmm, bmm_gy, cs_gx, in16); break;
