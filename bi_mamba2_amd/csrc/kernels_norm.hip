@@ -376,6 +376,7 @@ static int launch_norm_t(const bimamba2_norm_params *p, bool bwd) {
     const int nch = (p->group_size + 511) / 512;
     if (nch <= 1) return launch_norm_nch<T, 1>(p, bwd);
     if (nch <= 2) return launch_norm_nch<T, 2>(p, bwd);
+    if (nch == 3) return launch_norm_nch<T, 3>(p, bwd);    // 1536 columns: expand 2 x d_model 768, the benchmark layer's width
     if (nch <= 4) return launch_norm_nch<T, 4>(p, bwd);
     if (nch <= 8) return launch_norm_nch<T, 8>(p, bwd);
     if (nch <= 16) return launch_norm_nch<T, 16>(p, bwd);

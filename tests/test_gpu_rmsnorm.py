@@ -17,6 +17,7 @@ CASES = [
     ((4, 100), None, True, False, True, torch.float32),          # width not a multiple of 8: scalar accesses
     ((2, 64, 2048), None, True, False, True, torch.bfloat16),    # the benchmark layer's width
     ((2, 64, 2048), 512, True, True, False, torch.bfloat16),
+    ((5, 37, 1536), None, True, False, True, torch.bfloat16),    # 3 x 512 columns: the baseline layer's width (d_model 768)
     ((8, 4096), None, True, False, True, torch.float16),
     ((3, 8192), None, False, False, True, torch.bfloat16),       # the widest supported group
     ((600, 2, 128), None, True, True, True, torch.float32),      # more rows than partial-sum slots
