@@ -72,7 +72,7 @@ class ConvParams(ctypes.Structure):
         [("batch", _i64), ("seqlen", _i64), ("channels", _i32), ("width", _i32), ("dtype", _i32), ("has_bias", _i32)]
         + [(n, _i64) for n in ("x_sb", "x_sl", "dout_sb", "dout_sl")]
         + [(n, _vp) for n in ("x", "weight", "bias", "out", "dout", "dx", "dweight", "dbias", "workspace")]
-        + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
+        + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp), ("dx_sb", _i64), ("dx_sl", _i64)]
     )
 
 

@@ -60,12 +60,17 @@ def _conv1d_silu_fwd(x, weight, bias):
     return out
 
 
-def _conv1d_silu_bwd(dout, x, weight, bias):
-    """-> dx (batch, seqlen, channels), dweight (channels, width) float32, dbias (channels) float32 or None."""
+def _conv1d_silu_bwd(dout, x, weight, bias, dx_out=None):
+    """-> dx (batch, seqlen, channels), dweight (channels, width) float32, dbias (channels) float32 or None.
+    dx_out: where dx is to be written (same shape and dtype as x, unit stride along channels: e.g. a slice of a wider
+    buffer); a new tensor when None."""
     x, dout = _view3(x, "x"), _view3(dout, "dout")
     assert dout.shape == x.shape
     p, keep = _params(x, weight, bias)
-    dx = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+    if dx_out is not None and (dx_out.shape != x.shape or dx_out.dtype != x.dtype or dx_out.stride(-1) != 1 or dx_out.device != x.device):
+        dx_out = None
+    dx = dx_out if dx_out is not None else torch.empty(x.shape, device=x.device, dtype=x.dtype)
+    p.dx_sb, p.dx_sl = dx.stride(0), dx.stride(1)
     dw = torch.empty((p.channels, p.width), device=x.device, dtype=torch.float32)
     db = torch.empty((p.channels,), device=x.device, dtype=torch.float32) if bias is not None else None
     p.dout, p.dout_sb, p.dout_sl = dout.data_ptr(), dout.stride(0), dout.stride(1)
@@ -81,18 +86,22 @@ def _conv1d_silu_bwd(dout, x, weight, bias):
 
 class Conv1dSiluFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias=None):
+    def forward(ctx, x, weight, bias=None, dx_place=None):
         ctx.save_for_backward(x, weight, bias)
+        ctx.dx_place = dx_place
         return _conv1d_silu_fwd(x, weight, bias)
 
     @staticmethod
     def backward(ctx, dout):
         x, weight, bias = ctx.saved_tensors
-        dx, dw, db = _conv1d_silu_bwd(dout, x, weight, bias)
-        return dx, dw.reshape(weight.shape).to(weight.dtype), (db.to(bias.dtype) if bias is not None else None)
+        dx, dw, db = _conv1d_silu_bwd(dout, x, weight, bias, dx_out=ctx.dx_place() if ctx.dx_place is not None else None)
+        return dx, dw.reshape(weight.shape).to(weight.dtype), (db.to(bias.dtype) if bias is not None else None), None
 
 
-def conv1d_silu_fn(x, weight, bias=None):
+def conv1d_silu_fn(x, weight, bias=None, dx_place=None):
     """x: (batch, seqlen, channels), channels contiguous (a strided view is fine); weight: (channels, 1, width) as
-    nn.Conv1d keeps it, or (channels, width); bias: (channels,) or None.  width odd, at most 9."""
-    return Conv1dSiluFn.apply(x, weight, bias)
+    nn.Conv1d keeps it, or (channels, width); bias: (channels,) or None.  width odd, at most 9.
+    dx_place: optional callable, asked in the backward pass for the tensor the gradient of x is to be written into (shaped
+    like x, unit stride along channels) - the layer hands out slices of one buffer for the gradients of the pieces of its
+    projection output, which saves concatenating them."""
+    return Conv1dSiluFn.apply(x, weight, bias, dx_place)

@@ -113,7 +113,8 @@ __global__ __launch_bounds__(NTHREADS) void conv1d_silu_bwd_kernel(const bimamba
     }
     const T *xin = reinterpret_cast<const T *>(p.x) + b * p.x_sb + c0;
     const T *din = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + c0;
-    T *dx = reinterpret_cast<T *>(p.dx) + (b * p.seqlen) * p.channels + c0;
+    const int64_t dx_sl = p.dx_sl ? p.dx_sl : p.channels, dx_sb = p.dx_sl ? p.dx_sb : p.seqlen * p.channels;
+    T *dx = reinterpret_cast<T *>(p.dx) + b * dx_sb + c0;
     auto ldx = [&](int l) { return conv_load<T, VS>(xin + (int64_t)min(max(l, 0), L - 1) * p.x_sl); };
     auto ldd = [&](int l) { return conv_load<T, VS>(din + (int64_t)min(max(l, 0), L - 1) * p.dout_sl); };
     float xw[W][VS], gw[W][VS], dw[W][VS], db[VS];
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(NTHREADS) void conv1d_silu_bwd_kernel(const bimamba
                         for (int k = 0; k < W; ++k) a = __builtin_fmaf(w[k][i], gw[(u - k + W) % W][i], a);
                         o.v[i] = from_f<T>(a);
                     }
-                    *reinterpret_cast<ConvVec<T, VS> *>(dx + (int64_t)j * p.channels) = o;
+                    *reinterpret_cast<ConvVec<T, VS> *>(dx + (int64_t)j * dx_sl) = o;
                 }
             }
         }
@@ -237,7 +238,7 @@ static int launch_conv_vs(const bimamba2_conv_params *p, bool bwd) {
     auto al = [](const void *q, size_t a) { return (reinterpret_cast<uintptr_t>(q) % a) == 0; };
     const size_t va = sizeof(T) * VS;
     bool vec = p->channels % VS == 0 && al(p->x, va) && p->x_sb % VS == 0 && p->x_sl % VS == 0;
-    if (bwd) vec = vec && al(p->dout, va) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && al(p->dx, va);
+    if (bwd) vec = vec && al(p->dout, va) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && al(p->dx, va) && p->dx_sb % VS == 0 && p->dx_sl % VS == 0;
     else vec = vec && al(p->out, va);
 #define BM2_CONV(WV)                                                      \
     case WV: return vec ? launch_conv_w<T, WV, VS>(p, bwd) : launch_conv_w<T, WV, 1>(p, bwd)

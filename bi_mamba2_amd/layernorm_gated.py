@@ -74,14 +74,18 @@ def _layer_norm_fwd(x, weight, bias, eps, z=None, group_size=None, norm_before_g
     return (out, rstd) if is_rms_norm else (out, mean, rstd)
 
 
-def _layer_norm_bwd(dy, x, weight, bias, eps, rstd, z=None, group_size=None, norm_before_gate=True, mean=None):
+def _layer_norm_bwd(dy, x, weight, bias, eps, rstd, z=None, group_size=None, norm_before_gate=True, mean=None, dz_out=None):
     """-> dx, dweight (float32), dbias (float32 or None), dz (or None).  mean: the forward's group means (LayerNorm), None
-    for the RMS norm."""
+    for the RMS norm.  dz_out: where dz is to be written (rows like x, unit stride along the columns), a new tensor when
+    None."""
     p = _params(x, z, weight, bias, eps, group_size, norm_before_gate, mean is None)
     if mean is not None:
         p.mean = mean.data_ptr()
     dx = torch.empty_like(x, memory_format=torch.contiguous_format)
-    dz = torch.empty_like(x, memory_format=torch.contiguous_format) if z is not None else None
+    if dz_out is not None and (z is None or dz_out.shape != x.shape or dz_out.dtype != x.dtype or dz_out.stride(-1) != 1
+                               or dz_out.device != x.device):
+        dz_out = None
+    dz = dz_out if dz_out is not None else (torch.empty_like(x, memory_format=torch.contiguous_format) if z is not None else None)
     dw = torch.empty((x.shape[1],), device=x.device, dtype=torch.float32)
     db = torch.empty_like(dw) if bias is not None else None
     p.dout, p.dout_rs, p.rstd = dy.data_ptr(), dy.stride(0), rstd.data_ptr()
@@ -101,7 +105,11 @@ class LayerNormFn(torch.autograd.Function):
     """The reference's function of the same name: gated RMS norm (is_rms_norm=True) or gated LayerNorm."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True, is_rms_norm=False):
+    def forward(ctx, x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True, is_rms_norm=False,
+                dz_place=None):
+        # dz_place: optional callable, asked in the backward pass for the tensor the gradient of z is to be written into
+        # (shaped like z, unit stride along the last dimension, rows at one stride: e.g. a slice of a wider buffer)
+        ctx.dz_place = dz_place
         shape = x.shape
         x2 = _rows(x, "x")
         z2 = _rows(z, "z") if z is not None else None
@@ -128,10 +136,22 @@ class LayerNormFn(torch.autograd.Function):
         dy2 = _rows(dy, "dy")
         if dy2.dtype != x2.dtype:
             dy2 = dy2.to(x2.dtype)
+        place, dz_rows = None, None
+        if ctx.dz_place is not None and z2 is not None and ctx.zdtype == x2.dtype:
+            place = ctx.dz_place()
+            if place is not None and tuple(place.shape) == tuple(ctx.shape) and place.stride(-1) == 1:
+                try:
+                    dz_rows = place.view(-1, ctx.shape[-1])          # rows at one stride, or no view exists
+                except RuntimeError:
+                    place = None
+            else:
+                place = None
         dx, dw, db, dz = _layer_norm_bwd(dy2, x2, w32, b32, ctx.eps, rstd, z=z2, group_size=ctx.group_size,
-                                         norm_before_gate=ctx.norm_before_gate, mean=mean)
+                                         norm_before_gate=ctx.norm_before_gate, mean=mean, dz_out=dz_rows)
+        if dz is not None:
+            dz = place if (place is not None and dz is dz_rows) else dz.reshape(ctx.shape).to(ctx.zdtype)
         return (dx.reshape(ctx.shape), dw.to(ctx.wdtype), db.to(ctx.bdtype) if db is not None else None,
-                dz.reshape(ctx.shape).to(ctx.zdtype) if dz is not None else None, None, None, None, None)
+                dz, None, None, None, None, None)
 
 
 MAX_GROUP = 8192      # columns per normalisation group (bimamba2_rmsnorm_gated_fwd / _bwd refuse more)
@@ -141,8 +161,8 @@ def layernorm_fn(x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before
     return LayerNormFn.apply(x, weight, bias, z, eps, group_size, norm_before_gate, is_rms_norm)
 
 
-def rmsnorm_fn(x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True):
-    return LayerNormFn.apply(x, weight, bias, z, eps, group_size, norm_before_gate, True)
+def rmsnorm_fn(x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True, dz_place=None):
+    return LayerNormFn.apply(x, weight, bias, z, eps, group_size, norm_before_gate, True, dz_place)
 
 
 class LayerNorm(torch.nn.Module):
@@ -188,7 +208,8 @@ class RMSNorm(torch.nn.Module):
     def reset_parameters(self):
         torch.nn.init.ones_(self.weight)
 
-    def forward(self, x, z=None):
-        """norm(x) * silu(z) if norm_before_gate, else norm(x * silu(z)); plain norm without z."""
+    def forward(self, x, z=None, dz_place=None):
+        """norm(x) * silu(z) if norm_before_gate, else norm(x * silu(z)); plain norm without z.  dz_place (not in the
+        reference): see LayerNormFn.forward."""
         return rmsnorm_fn(x, self.weight, self.bias, z=z, eps=self.eps, group_size=self.group_size,
-                          norm_before_gate=self.norm_before_gate)
+                          norm_before_gate=self.norm_before_gate, dz_place=dz_place)

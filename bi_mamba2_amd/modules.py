@@ -21,6 +21,60 @@ from .ops import bimamba_chunk_scan_combined
 RMSNormGated = RMSNorm
 
 
+class _GradPieces:
+    """One buffer for the gradients of the pieces a tensor is split into along its last dimension.  torch.split's backward
+    concatenates the pieces' gradients, a copy of the whole projection output's gradient (100 MB at the benchmark layer);
+    here the kernels that produce the large pieces write them into slices of the buffer (piece(i), asked for in the
+    backward pass) and the split's backward hands the buffer on as it is."""
+
+    last_copied = None
+
+    def __init__(self, like, sizes):
+        self.shape, self.dtype, self.device = tuple(like.shape), like.dtype, like.device
+        self.bounds = [0]
+        for n in sizes:
+            self.bounds.append(self.bounds[-1] + n)
+        assert self.bounds[-1] == self.shape[-1]
+        self.buf = None
+
+    def piece(self, i):
+        if self.buf is None:
+            self.buf = torch.empty(self.shape, dtype=self.dtype, device=self.device)
+        return self.buf[..., self.bounds[i]:self.bounds[i + 1]]
+
+    def place(self, i):
+        return lambda: self.piece(i)
+
+    def take(self):
+        buf, self.buf = self.buf, None
+        return buf
+
+
+class _SplitInto(torch.autograd.Function):
+    """torch.split(t, sizes, dim=-1) whose backward fills a _GradPieces buffer: a gradient that already is the buffer's
+    slice stays where it is, any other one is copied in (a missing one counts as zero)."""
+
+    @staticmethod
+    def forward(ctx, t, pieces):
+        ctx.pieces = pieces
+        b = pieces.bounds
+        return tuple(t[..., b[i]:b[i + 1]] for i in range(len(b) - 1))
+
+    @staticmethod
+    def backward(ctx, *grads):
+        pieces = ctx.pieces
+        copied = []
+        for i, g in enumerate(grads):
+            dst = pieces.piece(i)
+            if g is None:
+                dst.zero_()
+            elif not (g.data_ptr() == dst.data_ptr() and g.shape == dst.shape and g.stride() == dst.stride() and g.dtype == dst.dtype):
+                dst.copy_(g)
+                copied.append(i)
+        _GradPieces.last_copied = tuple(copied)       # (for the tests: which pieces did not arrive in place)
+        return pieces.take(), None
+
+
 class BiMamba2(nn.Module):
     """Bidirectional Mamba-2 mixer layer; ``forward(u)`` maps (batch, seqlen, d_model) to the same shape."""
 
@@ -75,10 +129,19 @@ class BiMamba2(nn.Module):
         bc = self.ngroups * self.d_state
         zxbcdt = self.in_proj(u)
         A = -torch.exp(self.A_log.float())
-        z, xBC, dt = torch.split(zxbcdt, [self.d_inner, self.d_inner + 2 * bc, self.nheads], dim=-1)
+        sizes = [self.d_inner, self.d_inner + 2 * bc, self.nheads]
+        if torch.is_grad_enabled() and zxbcdt.requires_grad:
+            # the gradients of z (from the norm) and of xBC (from the convolution) are written straight into their places
+            # in the gradient of the projection output
+            grads = _GradPieces(zxbcdt, sizes)
+            z, xBC, dt = _SplitInto.apply(zxbcdt, grads)
+            dz_place, dxbc_place = grads.place(0), grads.place(1)
+        else:
+            z, xBC, dt = torch.split(zxbcdt, sizes, dim=-1)
+            dz_place = dxbc_place = None
         # conv1d + SiLU on the channels-last view, one HIP kernel (the reference transposes, calls nn.Conv1d, transposes
         # back and applies the activation, modules.py:162-164 there); self.conv1d only holds the parameters
-        xBC = conv1d_silu_fn(xBC, self.conv1d.weight, self.conv1d.bias)
+        xBC = conv1d_silu_fn(xBC, self.conv1d.weight, self.conv1d.bias, dx_place=dxbc_place)
         x, B, C = torch.split(xBC, [self.d_inner, bc, bc], dim=-1)
         kw = {} if tuple(self.dt_limit) == (0.0, float("inf")) else {"dt_limit": tuple(self.dt_limit)}
         # softplus(dt + dt_bias) (modules.py:158 there) happens inside the operator's first kernel
@@ -86,5 +149,5 @@ class BiMamba2(nn.Module):
             x.unflatten(-1, (self.nheads, self.headdim)), dt, A,
             B.unflatten(-1, (self.ngroups, self.d_state)), C.unflatten(-1, (self.ngroups, self.d_state)),
             chunk_size=self.chunk_size, D=self.D, z=None, dt_bias=self.dt_bias, dt_softplus=True, **kw)
-        y = self.norm(y.flatten(-2), z)
+        y = self.norm(y.flatten(-2), z, dz_place=dz_place)
         return self.out_proj(y)

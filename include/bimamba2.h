@@ -304,6 +304,8 @@ typedef struct bimamba2_conv_params {
     void *workspace;
     size_t workspace_bytes;
     void *stream;               /* hipStream_t */
+    int64_t dx_sb, dx_sl;       /* element strides of dx: batch, position; both 0 = contiguous (seqlen * channels, channels).
+                                   Lets the gradient land in a slice of a wider buffer (the layer's projection gradient). */
 } bimamba2_conv_params;
 
 size_t bimamba2_conv_params_size(void);

@@ -53,6 +53,26 @@ def test_conv1d_silu_forward_and_backward(case):
         assert_close(bd.grad, b64.grad, dtype, "dbias")
 
 
+@pytest.mark.parametrize("dtype,C", [(torch.bfloat16, 64), (torch.float32, 5)])
+def test_conv1d_silu_gradient_into_a_slice(dtype, C):
+    """dx_place: the gradient of x lands in a slice of a wider buffer (the layer's use), bit for bit what the plain call
+    returns, and the rest of the buffer stays as it was."""
+    from bi_mamba2_amd.conv1d import conv1d_silu_fn
+    g = torch.Generator().manual_seed(2)
+    b, L, W = 2, 50, 7
+    x = torch.randn(b, L, C, generator=g).to(dtype).cuda()
+    w = (0.3 * torch.randn(C, 1, W, generator=g)).cuda()
+    bias = (0.1 * torch.randn(C, generator=g)).cuda()
+    dout = torch.randn(b, L, C, generator=g).to(dtype).cuda()
+    xa = x.clone().requires_grad_(True)
+    conv1d_silu_fn(xa, w, bias).backward(dout)
+    wide = torch.full((b, L, C + 24), 7.0, dtype=dtype, device="cuda")
+    xb = x.clone().requires_grad_(True)
+    conv1d_silu_fn(xb, w, bias, dx_place=lambda: wide[..., 8:8 + C]).backward(dout)
+    assert torch.equal(xb.grad, xa.grad) and torch.equal(wide[..., 8:8 + C], xa.grad)
+    assert (wide[..., :8] == 7.0).all() and (wide[..., 8 + C:] == 7.0).all()
+
+
 def test_conv1d_silu_errors():
     from bi_mamba2_amd.conv1d import conv1d_silu_fn
     x = torch.randn(1, 8, 4)

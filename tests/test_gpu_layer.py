@@ -63,6 +63,34 @@ def test_bimamba2_layer_forward_backward():
         assert p.grad is not None, name
         assert_close(p.grad, dp_ref[name], torch.float32, "layer d" + name)
     assert set(dp_ref) | set(UNUSED) == set(m.state_dict())
+    # the gradients of z (norm) and xBC (convolution) were written in place into the projection output's gradient; only the
+    # small dt piece was copied there
+    from bi_mamba2_amd.modules import _GradPieces
+    assert _GradPieces.last_copied == (2,)
+
+
+def test_bimamba2_layer_without_input_gradient_and_twice():
+    """Frozen input (only the parameters take gradients) and two backward passes through two forwards that share the
+    layer: the buffer of the split's gradients belongs to one forward call."""
+    from bi_mamba2_amd.modules import BiMamba2
+    torch.manual_seed(0)
+    m = BiMamba2(d_model=64, d_state=16, headdim=16, ngroups=1, chunk_size=64).cuda()
+    u1 = torch.randn(2, 100, 64, device="cuda")
+    u2 = torch.randn(2, 100, 64, device="cuda", requires_grad=True)
+    o1, o2 = m(u1), m(u2)
+    (o1.sum() + 2 * o2.sum()).backward()
+    g_both = {n: p.grad.clone() for n, p in m.named_parameters() if p.grad is not None}
+    du2 = u2.grad.clone()
+    m.zero_grad()
+    u2.grad = None
+    m(u1).sum().backward()
+    g1 = {n: p.grad.clone() for n, p in m.named_parameters() if p.grad is not None}
+    m.zero_grad()
+    (2 * m(u2).sum()).backward()
+    for n, p in m.named_parameters():
+        if p.grad is not None:
+            assert_close(g_both[n], (g1[n] + p.grad).double(), torch.float32, "sum of two passes, d" + n, scaled=True)
+    assert torch.equal(du2, u2.grad)
 
 
 def test_bimamba2_layer_bf16_runs():

@@ -67,6 +67,24 @@ def test_rmsnorm_strided_rows_and_module():
     assert_close(out, ref, torch.float32, "out (strided)")
 
 
+def test_rmsnorm_gate_gradient_into_a_slice():
+    """dz_place: the gradient of z lands in a slice of a wider buffer (the layer's use), bit for bit what the plain call
+    returns."""
+    from bi_mamba2_amd.layernorm_gated import rmsnorm_fn
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(3, 21, 128, generator=g).to(torch.bfloat16).cuda()
+    z = torch.randn(3, 21, 128, generator=g).to(torch.bfloat16).cuda()
+    w = (1.0 + 0.1 * torch.randn(128, generator=g)).cuda()
+    dy = torch.randn(3, 21, 128, generator=g).to(torch.bfloat16).cuda()
+    za = z.clone().requires_grad_(True)
+    rmsnorm_fn(x, w, None, z=za, eps=1e-5).backward(dy)
+    wide = torch.full((3, 21, 128 + 40), 3.0, dtype=torch.bfloat16, device="cuda")
+    zb = z.clone().requires_grad_(True)
+    rmsnorm_fn(x, w, None, z=zb, eps=1e-5, dz_place=lambda: wide[..., 16:16 + 128]).backward(dy)
+    assert torch.equal(zb.grad, za.grad) and torch.equal(wide[..., 16:16 + 128], za.grad)
+    assert (wide[..., :16] == 3.0).all() and (wide[..., 16 + 128:] == 3.0).all()
+
+
 def test_layernorm_module():
     """The LayerNorm module (weight and bias parameters), gated, against the oracle."""
     from bi_mamba2_amd.layernorm_gated import LayerNorm
