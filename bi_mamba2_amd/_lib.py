@@ -50,7 +50,8 @@ CONV_ENTRY_POINTS = ("bimamba2_conv1d_silu_fwd", "bimamba2_conv1d_silu_bwd")
 ALL_SYMBOLS = ENTRY_POINTS + ("bimamba2_strerror", "bimamba2_version", "bimamba2_params_size",
                               "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb", "bimamba2_state_copies", "bimamba2_norm_params_size",
                               "bimamba2_rmsnorm_gated_workspace_bytes", "bimamba2_conv_params_size",
-                              "bimamba2_conv1d_silu_workspace_bytes") + NORM_ENTRY_POINTS + CONV_ENTRY_POINTS
+                              "bimamba2_conv1d_silu_workspace_bytes", "bimamba2_cast_params_size",
+                              "bimamba2_cast_many") + NORM_ENTRY_POINTS + CONV_ENTRY_POINTS
 
 _lib = None
 
@@ -74,6 +75,20 @@ class ConvParams(ctypes.Structure):
         + [(n, _vp) for n in ("x", "weight", "bias", "out", "dout", "dx", "dweight", "dbias", "workspace")]
         + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp), ("dx_sb", _i64), ("dx_sl", _i64)]
     )
+
+
+CAST_MAX = 8
+CAST_COPY, CAST_NEG_EXP, CAST_MUL = 0, 1, 2
+
+
+class CastItem(ctypes.Structure):
+    _fields_ = [("src", _vp), ("dst", _vp), ("aux", _vp), ("n", _i64), ("src_dtype", _i32), ("dst_dtype", _i32), ("op", _i32),
+                ("reserved", _i32)]
+
+
+class CastParams(ctypes.Structure):
+    """Mirror of ``struct bimamba2_cast_params`` (several small conversions in one launch)."""
+    _fields_ = [("count", _i32), ("reserved", _i32), ("item", CastItem * CAST_MAX), ("stream", _vp)]
 
 
 def load():
@@ -120,6 +135,11 @@ def load():
         raise RuntimeError("bimamba2_conv_params layout mismatch between the library and its Python mirror")
     lib.bimamba2_conv1d_silu_workspace_bytes.argtypes = [ctypes.POINTER(ConvParams)]
     lib.bimamba2_conv1d_silu_workspace_bytes.restype = ctypes.c_size_t
+    lib.bimamba2_cast_params_size.restype = ctypes.c_size_t
+    if lib.bimamba2_cast_params_size() != ctypes.sizeof(CastParams):
+        raise RuntimeError("bimamba2_cast_params layout mismatch between the library and its Python mirror")
+    lib.bimamba2_cast_many.argtypes = [ctypes.POINTER(CastParams)]
+    lib.bimamba2_cast_many.restype = ctypes.c_int
     _lib = lib
     return lib
 

@@ -451,6 +451,21 @@ int bimamba2_rmsnorm_gated_bwd(const bimamba2_norm_params *p) {
 
 size_t bimamba2_conv_params_size(void) { return sizeof(bimamba2_conv_params); }
 
+size_t bimamba2_cast_params_size(void) { return sizeof(bimamba2_cast_params); }
+
+int bimamba2_cast_many(const bimamba2_cast_params *p) {
+    if (!p || p->count < 0 || p->count > BIMAMBA2_CAST_MAX) return BIMAMBA2_EINVAL;
+    auto known = [](int d) { return d == BIMAMBA2_F32 || d == BIMAMBA2_BF16 || d == BIMAMBA2_F16; };
+    for (int k = 0; k < p->count; ++k) {
+        const bimamba2_cast_item &it = p->item[k];
+        if (it.n < 0 || (it.n > 0 && (!it.src || !it.dst))) return BIMAMBA2_EINVAL;
+        if (!known(it.src_dtype) || !known(it.dst_dtype)) return BIMAMBA2_EUNSUPPORTED;
+        if (it.op < BIMAMBA2_CAST_COPY || it.op > BIMAMBA2_CAST_MUL) return BIMAMBA2_EINVAL;
+        if (it.op == BIMAMBA2_CAST_MUL && it.n > 0 && !it.aux) return BIMAMBA2_EINVAL;
+    }
+    return launch_cast_many(p);
+}
+
 static int check_conv(const bimamba2_conv_params *p) {
     if (!p) return BIMAMBA2_EINVAL;
     if (p->batch < 0 || p->seqlen < 0 || p->channels <= 0) return BIMAMBA2_EINVAL;

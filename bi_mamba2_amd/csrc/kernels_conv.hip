@@ -260,6 +260,47 @@ static int launch_conv_t(const bimamba2_conv_params *p, bool bwd) {
     return launch_conv_vs<T, 2>(p, bwd);
 }
 
+// ---- several small element-wise conversions in one launch (bimamba2_cast_many) -------------------------------------
+namespace {
+__device__ __forceinline__ float cast_load(const void *src, int dtype, int64_t i) {
+    if (dtype == BIMAMBA2_F32) return reinterpret_cast<const float *>(src)[i];
+    if (dtype == BIMAMBA2_BF16) return to_f(reinterpret_cast<const bf16_t *>(src)[i]);
+    return to_f(reinterpret_cast<const f16_t *>(src)[i]);
+}
+__device__ __forceinline__ void cast_store(void *dst, int dtype, int64_t i, float v) {
+    if (dtype == BIMAMBA2_F32) reinterpret_cast<float *>(dst)[i] = v;
+    else if (dtype == BIMAMBA2_BF16) reinterpret_cast<bf16_t *>(dst)[i] = from_f<bf16_t>(v);
+    else reinterpret_cast<f16_t *>(dst)[i] = from_f<f16_t>(v);
+}
+}  // namespace
+
+// blocks are dealt to the items in order: item k owns ceil(n_k / 256) of them
+__global__ __launch_bounds__(NTHREADS) void cast_many_kernel(const bimamba2_cast_params p) {
+    int blk = blockIdx.x, k = 0;
+    for (; k < p.count; ++k) {
+        const int nb = (int)((p.item[k].n + NTHREADS - 1) / NTHREADS);
+        if (blk < nb) break;
+        blk -= nb;
+    }
+    if (k >= p.count) return;
+    const bimamba2_cast_item &it = p.item[k];
+    const int64_t i = (int64_t)blk * NTHREADS + threadIdx.x;
+    if (i >= it.n) return;
+    float v = cast_load(it.src, it.src_dtype, i);
+    if (it.op == BIMAMBA2_CAST_NEG_EXP) v = -expf(v);
+    else if (it.op == BIMAMBA2_CAST_MUL) v *= it.aux[i];
+    cast_store(it.dst, it.dst_dtype, i, v);
+}
+
+int launch_cast_many(const bimamba2_cast_params *p) {
+    int64_t blocks = 0;
+    for (int k = 0; k < p->count; ++k) blocks += (p->item[k].n + NTHREADS - 1) / NTHREADS;
+    if (blocks == 0) return BIMAMBA2_OK;
+    if (blocks > 0x7fffffff) return BIMAMBA2_EUNSUPPORTED;
+    hipLaunchKernelGGL(cast_many_kernel, dim3((unsigned)blocks), dim3(NTHREADS), 0, reinterpret_cast<hipStream_t>(p->stream), *p);
+    return check_launch();
+}
+
 int launch_conv1d_silu(const bimamba2_conv_params *p, bool bwd) {
     switch (p->dtype) {
         case BIMAMBA2_F32: return launch_conv_t<float>(p, bwd);

@@ -54,5 +54,7 @@ int launch_colsum(const float *in, float *out, int ni, int nj, hipStream_t strea
 // depthwise conv1d + SiLU (kernels_conv.hip)
 int launch_conv1d_silu(const bimamba2_conv_params *p, bool bwd);
 size_t conv_workspace_bytes(const bimamba2_conv_params *p);
+// several small element-wise conversions in one launch (kernels_conv.hip)
+int launch_cast_many(const bimamba2_cast_params *p);
 
 }  // namespace bm2

@@ -6,15 +6,17 @@ non-causal depthwise conv1d + SiLU -> split x, B, C -> bidirectional SSD with D 
 out_proj.  Parameters are created in the reference's order, so a seeded construction draws the same values.
 The projections and the convolution are ordinary torch ops; the SSD and the gated RMS norm are the HIP operators.
 """
+import ctypes
 import math
 
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import _lib
 from .conv1d import conv1d_silu_fn
-from .layernorm_gated import RMSNorm
-from .ops import bimamba_chunk_scan_combined
+from .layernorm_gated import RMSNorm, rmsnorm_fn
+from .ops import _DT, bimamba_chunk_scan_combined
 
 
 # the gated RMS norm of the layer runs on the HIP kernels (bi_mamba2_amd/layernorm_gated.py)
@@ -48,6 +50,67 @@ class _GradPieces:
     def take(self):
         buf, self.buf = self.buf, None
         return buf
+
+
+def _cast_many(items, device):
+    """items: (src, dst, op, aux) tensors (contiguous, same number of elements each pair) -> one launch."""
+    p = _lib.CastParams()
+    assert len(items) <= _lib.CAST_MAX
+    p.count = len(items)
+    for k, (src, dst, op, aux) in enumerate(items):
+        it = p.item[k]
+        it.src, it.dst, it.n = src.data_ptr(), dst.data_ptr(), src.numel()
+        it.src_dtype, it.dst_dtype, it.op = _DT[src.dtype], _DT[dst.dtype], op
+        it.aux = aux.data_ptr() if aux is not None else None
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        p.stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.bimamba2_cast_many(ctypes.byref(p))
+    if rc != 0:
+        raise RuntimeError(f"bimamba2_cast_many: {lib.bimamba2_strerror(rc).decode()} (code {rc})")
+
+
+class _ParamsAsFloat32(torch.autograd.Function):
+    """(A_log, D, dt_bias, conv weight, conv bias or None, norm weight) -> (A = -exp(A_log), and the others) as float32, in
+    one launch, and their gradients back into the parameters' types in one launch.  The kernels of the layer compute with
+    float32 parameters; when the module holds them in a 16-bit type (model.to(torch.bfloat16)) each of these maps is
+    otherwise a torch op of its own, forward and backward: about twenty launches of 4 us per step."""
+
+    @staticmethod
+    def forward(ctx, *params):
+        live = [t for t in params if t is not None]
+        buf = torch.empty(sum(t.numel() for t in live), dtype=torch.float32, device=live[0].device)
+        outs, items, at = [], [], 0
+        for i, t in enumerate(params):
+            if t is None:
+                outs.append(None)
+                continue
+            o = buf[at:at + t.numel()].view(t.shape)
+            at += t.numel()
+            items.append((t.detach().contiguous(), o, _lib.CAST_NEG_EXP if i == 0 else _lib.CAST_COPY, None))
+            outs.append(o)
+        _cast_many(items, buf.device)
+        ctx.meta = [(t.dtype, t.shape) if t is not None else None for t in params]
+        ctx.save_for_backward(outs[0])
+        ctx.mark_non_differentiable(*[o for o, need in zip(outs, ctx.needs_input_grad) if o is not None and not need])
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        (A,) = ctx.saved_tensors
+        res, items = [], []
+        for i, (g, meta) in enumerate(zip(grads, ctx.meta)):
+            if g is None or meta is None or not ctx.needs_input_grad[i]:
+                res.append(None)
+                continue
+            dtype, shape = meta
+            g = g.float().contiguous()
+            o = torch.empty(shape, dtype=dtype, device=g.device)
+            items.append((g, o, _lib.CAST_MUL if i == 0 else _lib.CAST_COPY, A if i == 0 else None))   # dA_log = dA * A
+            res.append(o)
+        if items:
+            _cast_many(items, A.device)
+        return tuple(res)
 
 
 class _SplitInto(torch.autograd.Function):
@@ -128,7 +191,13 @@ class BiMamba2(nn.Module):
     def forward(self, u):
         bc = self.ngroups * self.d_state
         zxbcdt = self.in_proj(u)
-        A = -torch.exp(self.A_log.float())
+        prm = (self.A_log, self.D, self.dt_bias, self.conv1d.weight, self.conv1d.bias, self.norm.weight)
+        if u.is_cuda and any(t is not None and t.dtype != torch.float32 for t in prm) and all(t is None or t.dtype in _DT for t in prm):
+            # 16-bit parameters: all maps to float32 (and A = -exp(A_log)) in one launch, their gradients likewise
+            A, D, dt_bias, conv_w, conv_b, norm_w = _ParamsAsFloat32.apply(*prm)
+        else:
+            A = -torch.exp(self.A_log.float())
+            D, dt_bias, conv_w, conv_b, norm_w = prm[1:]
         sizes = [self.d_inner, self.d_inner + 2 * bc, self.nheads]
         if torch.is_grad_enabled() and zxbcdt.requires_grad:
             # the gradients of z (from the norm) and of xBC (from the convolution) are written straight into their places
@@ -141,13 +210,15 @@ class BiMamba2(nn.Module):
             dz_place = dxbc_place = None
         # conv1d + SiLU on the channels-last view, one HIP kernel (the reference transposes, calls nn.Conv1d, transposes
         # back and applies the activation, modules.py:162-164 there); self.conv1d only holds the parameters
-        xBC = conv1d_silu_fn(xBC, self.conv1d.weight, self.conv1d.bias, dx_place=dxbc_place)
+        xBC = conv1d_silu_fn(xBC, conv_w, conv_b, dx_place=dxbc_place)
         x, B, C = torch.split(xBC, [self.d_inner, bc, bc], dim=-1)
         kw = {} if tuple(self.dt_limit) == (0.0, float("inf")) else {"dt_limit": tuple(self.dt_limit)}
         # softplus(dt + dt_bias) (modules.py:158 there) happens inside the operator's first kernel
         y = bimamba_chunk_scan_combined(
             x.unflatten(-1, (self.nheads, self.headdim)), dt, A,
             B.unflatten(-1, (self.ngroups, self.d_state)), C.unflatten(-1, (self.ngroups, self.d_state)),
-            chunk_size=self.chunk_size, D=self.D, z=None, dt_bias=self.dt_bias, dt_softplus=True, **kw)
-        y = self.norm(y.flatten(-2), z, dz_place=dz_place)
+            chunk_size=self.chunk_size, D=D, z=None, dt_bias=dt_bias, dt_softplus=True, **kw)
+        # (self.norm's forward, with the weight as prepared above)
+        y = rmsnorm_fn(y.flatten(-2), norm_w, None, z=z, eps=self.norm.eps, group_size=self.norm.group_size,
+                       norm_before_gate=self.norm.norm_before_gate, dz_place=dz_place)
         return self.out_proj(y)

@@ -315,6 +315,32 @@ int bimamba2_conv1d_silu_fwd(const bimamba2_conv_params *p);
 /* x weight [bias] dout -> dx dweight [dbias] */
 int bimamba2_conv1d_silu_bwd(const bimamba2_conv_params *p);
 
+/* ---------------------------------------------------------------------------------------------------------
+ * Several small element-wise conversions in ONE launch: the parameter maps in front of and behind the layer's kernels
+ * (A = -exp(A_log), and dt_bias, D, the convolution's filter and bias and the norm's weight as float32 when the module
+ * holds them in a 16-bit type; on the way back the float32 gradients into the parameters' types, dA_log = dA * A).  The
+ * reference does them as separate torch ops (src/ssd/modules.py:156, the .float() calls in its kernels' wrappers);
+ * captured in a graph each of those is a launch of a few microseconds.
+ * ------------------------------------------------------------------------------------------------------- */
+#define BIMAMBA2_CAST_MAX 8
+enum { BIMAMBA2_CAST_COPY = 0,      /* dst = src */
+       BIMAMBA2_CAST_NEG_EXP = 1,   /* dst = -exp(src) */
+       BIMAMBA2_CAST_MUL = 2 };     /* dst = src * aux (aux: float32, same length) */
+typedef struct bimamba2_cast_item {
+    const void *src;
+    void *dst;
+    const float *aux;
+    int64_t n;                  /* elements (contiguous) */
+    int32_t src_dtype, dst_dtype, op, reserved;
+} bimamba2_cast_item;
+typedef struct bimamba2_cast_params {
+    int32_t count, reserved;    /* items in use, at most BIMAMBA2_CAST_MAX */
+    bimamba2_cast_item item[BIMAMBA2_CAST_MAX];
+    void *stream;               /* hipStream_t */
+} bimamba2_cast_params;
+size_t bimamba2_cast_params_size(void);
+int bimamba2_cast_many(const bimamba2_cast_params *p);
+
 #ifdef __cplusplus
 }
 #endif

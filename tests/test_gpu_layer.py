@@ -93,6 +93,37 @@ def test_bimamba2_layer_without_input_gradient_and_twice():
     assert torch.equal(du2, u2.grad)
 
 
+def test_parameter_maps_in_one_launch():
+    """_ParamsAsFloat32 (bimamba2_cast_many behind it): A = -exp(A_log) and float32 copies of 16-bit parameters, and their
+    gradients back in the parameters' types, against the torch ops they replace; a missing bias and a parameter without
+    gradient included."""
+    from bi_mamba2_amd.modules import _ParamsAsFloat32
+    g = torch.Generator().manual_seed(4)
+    mk = lambda *shape, dt: torch.randn(*shape, generator=g).to(dt).cuda().requires_grad_(True)
+    A_log, D, dtb = mk(24, dt=torch.bfloat16), mk(24, dt=torch.float32), mk(24, dt=torch.float16)
+    cw, nw = mk(300, 1, 7, dt=torch.bfloat16), mk(1536, dt=torch.bfloat16)
+    nw.requires_grad_(False)
+    outs = _ParamsAsFloat32.apply(A_log, D, dtb, cw, None, nw)
+    assert outs[4] is None and all(o.dtype == torch.float32 for o in outs if o is not None)
+    refs = (-torch.exp(A_log.float()), D.float(), dtb.float(), cw.float(), None, nw.float())
+    for o, r in zip(outs, refs):
+        if o is not None:
+            assert o.shape == r.shape
+            # exp of a 16-bit value in float32: the library's and torch's exp may differ in the last bit
+            assert torch.allclose(o, r.detach(), rtol=1e-6, atol=0)
+    assert not outs[5].requires_grad
+    gs = [torch.randn(o.shape, generator=g).cuda() for o in outs[:4]]
+    loss = sum((o * w).sum() for o, w in zip(outs[:4], gs))
+    loss.backward()
+    want = {"A_log": (gs[0] * refs[0].detach()).to(torch.bfloat16), "D": gs[1], "dt_bias": gs[2].to(torch.float16),
+            "conv": gs[3].to(torch.bfloat16)}
+    got = {"A_log": A_log.grad, "D": D.grad, "dt_bias": dtb.grad, "conv": cw.grad}
+    for k in want:
+        assert got[k].dtype == want[k].dtype and got[k].shape == want[k].shape, k
+        assert torch.allclose(got[k].float(), want[k].float(), rtol=1e-2 if k == "A_log" else 0, atol=0), k
+    assert nw.grad is None
+
+
 def test_bimamba2_layer_bf16_runs():
     from bi_mamba2_amd.modules import BiMamba2
     torch.manual_seed(0)
