@@ -34,6 +34,7 @@ class Params(ctypes.Structure):
                               "initial_f", "initial_b", "dfinal_f", "dfinal_b", "dinitial_f", "dinitial_b", "seq_idx",
                               "states16_f", "states16_b", "dstates16_f", "dstates16_b", "workspace")]
         + [("workspace_bytes", ctypes.c_size_t), ("stream", _vp)]
+        + [(n, _i64) for n in ("dx_sb", "dx_sl", "dB_sb", "dB_sl", "dC_sb", "dC_sl")]
     )
 
 

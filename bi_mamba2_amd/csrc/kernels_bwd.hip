@@ -1828,6 +1828,9 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
     const float *arow = (which == 0 ? p.dCBT : p.dCB) + (int64_t)bcg * Q * Q + (int64_t)min(r0 + wave * 16 + lr, Q - 1) * Q;
     const float *res = which == 0 ? p.dBs : p.dCs;
     T *out = reinterpret_cast<T *>(which == 0 ? p.dB : p.dC);
+    // (dB / dC may be slices of a wider buffer: their own position and batch strides; 0 = contiguous)
+    const int64_t o_sl = (which == 0 ? p.dB_sl : p.dC_sl) ? (which == 0 ? p.dB_sl : p.dC_sl) : (int64_t)p.ngroups * p.dstate;
+    const int64_t o_sb = (which == 0 ? p.dB_sl : p.dC_sl) ? (which == 0 ? p.dB_sb : p.dC_sb) : p.seqlen * o_sl;
     const int64_t slice = (int64_t)p.batch * p.seqlen * p.ngroups * N;
     constexpr int VS = 16 / (int)sizeof(T);
     if constexpr (FAST) {
@@ -1917,7 +1920,7 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
                 Vec16<T> ov;
 #pragma unroll
                 for (int i = 0; i < VS; ++i) ov.v[i] = from_f<T>(v[i]);
-                *reinterpret_cast<Vec16<T> *>(out + oa[it]) = ov;
+                *reinterpret_cast<Vec16<T> *>(out + (b * o_sb + ((int64_t)c * Q + r0 + rl) * o_sl + (int64_t)g * N + nt * 64 + cc)) = ov;
             }
         }
         return;
@@ -1954,12 +1957,13 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
 #pragma unroll
         for (int i = 0; i < 4; ++i) stg[(wave * 16 + lg * 4 + i) * SLD + j * 16 + lr] = acc[j][i];
     __syncthreads();
-    const bool ovec = N % VS == 0;
+    const bool ovec = N % VS == 0 && o_sl % VS == 0 && o_sb % VS == 0;
     for (int id = threadIdx.x; id < 64 * (64 / VS); id += NTHREADS) {
         const int rl = id / (64 / VS), cc = (id % (64 / VS)) * VS;
         const int r = r0 + rl, n = nt * 64 + cc;
         if (r >= limit || n >= N) continue;
         const int64_t a = (((int64_t)b * p.seqlen + (int64_t)c * Q + r) * p.ngroups + g) * N + n;
+        const int64_t ao = b * o_sb + ((int64_t)c * Q + r) * o_sl + (int64_t)g * N + n;
         float v[VS];
 #pragma unroll
         for (int i = 0; i < VS; ++i) v[i] = stg[rl * SLD + cc + i];
@@ -1973,14 +1977,14 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
             Vec16<T> ov;
 #pragma unroll
             for (int i = 0; i < VS; ++i) ov.v[i] = from_f<T>(v[i]);
-            *reinterpret_cast<Vec16<T> *>(out + a) = ov;
+            *reinterpret_cast<Vec16<T> *>(out + ao) = ov;
         } else {
 #pragma unroll
             for (int i = 0; i < VS; ++i)
                 if (n + i < N) {
                     float u = v[i];
                     for (int sl = 0; sl < nslices; ++sl) u += res[a + sl * slice + i];
-                    out[a + i] = from_f<T>(u);
+                    out[ao + i] = from_f<T>(u);
                 }
         }
     }
@@ -1999,7 +2003,7 @@ static int launch_bmm_bwd_t(const bimamba2_params *p) {
     auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
     const bool fast = sizeof(T) == 2 && (Q == 64 || Q == 128 || Q == 256) && p->dstate % 64 == 0 && nsl <= 8 && al(p->Bm) && al(p->Cm)
                       && mult(p->B_sb, p->B_sl, p->B_sg) && mult(p->C_sb, p->C_sl, p->C_sg) && al(p->dCB) && al(p->dCBT) && al(p->dBs)
-                      && al(p->dCs) && al(p->dB) && al(p->dC);
+                      && al(p->dCs) && al(p->dB) && al(p->dC) && mult(p->dB_sb, p->dB_sl, p->dC_sb) && p->dC_sl % 8 == 0;
 #define BM2_BMMB(QPV)                                                                                                              \
     do {                                                                                                                       \
         if constexpr (sizeof(T) == 2) {                                                                                        \
@@ -2198,7 +2202,7 @@ static bool bmm_bwd_fast(const bimamba2_params *p) {
     const int Q = p->chunk_size;
     return p->dtype != BIMAMBA2_F32 && (Q == 64 || Q == 128 || Q == 256) && p->dstate % 64 == 0 && dbdc_slices(p) <= 8 && al(p->Bm) &&
            al(p->Cm) && mult(p->B_sb, p->B_sl, p->B_sg) && mult(p->C_sb, p->C_sl, p->C_sg) && al(p->dCB) && al(p->dCBT) && al(p->dBs) &&
-           al(p->dCs) && al(p->dB) && al(p->dC);
+           al(p->dCs) && al(p->dB) && al(p->dC) && mult(p->dB_sb, p->dB_sl, p->dC_sb) && p->dC_sl % 8 == 0;
 }
 
 // whether launch_bwd_tail() exists for this problem

@@ -615,7 +615,9 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
                             dsum[i] += to_f(e2[B_][ps].v[i]) * to_f(ex[B_][ps].v[i]);
                         }
                     }
-                    store_vec(reinterpret_cast<T *>(p.dx) + orow, ovec, ncol, dxv, true);
+                    // (dx may be a slice of a wider buffer: its own position and batch strides)
+                    const int64_t dxo = p.dx_sl ? b * p.dx_sb + ((int64_t)c * Q + r) * p.dx_sl + (int64_t)h * P + col : orow;
+                    store_vec(reinterpret_cast<T *>(p.dx) + dxo, ovec && (p.dx_sl % VS == 0) && (p.dx_sb % VS == 0), ncol, dxv, true);
                 }
             }
             if (BWD) {
@@ -671,7 +673,7 @@ static bool scan_fast(const bimamba2_params *p, bool bwd, int pw, int vs) {
     auto mult = [vs](int64_t a, int64_t b, int64_t c) { return a % vs == 0 && b % vs == 0 && c % vs == 0; };
     bool fast = p->chunk_size % 32 == 0 && p->headdim % pw == 0 && p->dstate % 64 == 0 && al16(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
     if (bwd) {
-        fast = fast && al16(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al16(p->dx);
+        fast = fast && al16(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al16(p->dx) && mult(p->dx_sb, p->dx_sl, 0);
         fast = fast && (p->has_z ? al16(p->dout_x) : (al16(p->dout) && mult(p->dout_sb, p->dout_sl, p->dout_sh)));
     } else {
         fast = fast && al16(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg) && al16(p->out);

@@ -570,8 +570,11 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             // output rows: uniform base of the (chunk, head) + this lane's row and column group
             int hh = h;
             asm volatile("" : "+s"(hh));            // (addresses are built here, not kept from the top of the loop)
-            const int64_t obase = (((int64_t)b * p.seqlen + (int64_t)c * Q) * H + hh) * P + p0;
-            const unsigned orow = (unsigned)min(r_lane, limit - 1) * (unsigned)(H * P) + cq;
+            // (dx may be a slice of a wider buffer: its own position and batch strides)
+            const bool own = BWD && p.dx_sl != 0;
+            const unsigned osl = own ? (unsigned)p.dx_sl : (unsigned)(H * P);
+            const int64_t obase = (own ? b * p.dx_sb + (int64_t)c * Q * p.dx_sl : ((int64_t)b * p.seqlen + (int64_t)c * Q) * (H * P)) + (int64_t)hh * P + p0;
+            const unsigned orow = (unsigned)min(r_lane, limit - 1) * osl + cq;
             if (live) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {

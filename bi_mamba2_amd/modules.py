@@ -30,6 +30,7 @@ class _GradPieces:
     backward pass) and the split's backward hands the buffer on as it is."""
 
     last_copied = None
+    copies_log = []             # (for the tests: last_copied of the most recent backward passes)
 
     def __init__(self, like, sizes):
         self.shape, self.dtype, self.device = tuple(like.shape), like.dtype, like.device
@@ -135,6 +136,7 @@ class _SplitInto(torch.autograd.Function):
                 dst.copy_(g)
                 copied.append(i)
         _GradPieces.last_copied = tuple(copied)       # (for the tests: which pieces did not arrive in place)
+        _GradPieces.copies_log = _GradPieces.copies_log[-7:] + [tuple(copied)]
         return pieces.take(), None
 
 
@@ -211,8 +213,16 @@ class BiMamba2(nn.Module):
         # conv1d + SiLU on the channels-last view, one HIP kernel (the reference transposes, calls nn.Conv1d, transposes
         # back and applies the activation, modules.py:162-164 there); self.conv1d only holds the parameters
         xBC = conv1d_silu_fn(xBC, conv_w, conv_b, dx_place=dxbc_place)
-        x, B, C = torch.split(xBC, [self.d_inner, bc, bc], dim=-1)
         kw = {} if tuple(self.dt_limit) == (0.0, float("inf")) else {"dt_limit": tuple(self.dt_limit)}
+        if torch.is_grad_enabled() and xBC.requires_grad and self.headdim <= 128:
+            # likewise the operator's dx, dB, dC: slices of the gradient of the convolution's output
+            g2 = _GradPieces(xBC, [self.d_inner, bc, bc])
+            x, B, C = _SplitInto.apply(xBC, g2)
+            kw["grad_places"] = {"dx": lambda: g2.piece(0).unflatten(-1, (self.nheads, self.headdim)),
+                                 "dB": lambda: g2.piece(1).unflatten(-1, (self.ngroups, self.d_state)),
+                                 "dC": lambda: g2.piece(2).unflatten(-1, (self.ngroups, self.d_state))}
+        else:
+            x, B, C = torch.split(xBC, [self.d_inner, bc, bc], dim=-1)
         # softplus(dt + dt_bias) (modules.py:158 there) happens inside the operator's first kernel
         y = bimamba_chunk_scan_combined(
             x.unflatten(-1, (self.nheads, self.headdim)), dt, A,

@@ -78,6 +78,21 @@ class _Call:
         t = torch.empty(shape, device=self.device, dtype=dtype)
         return self.put(field, t)
 
+    def put_grad(self, field, t, shape, dtype):
+        """dx, dB or dC given by the caller: (batch, seqlen, heads or groups, width) with the two inner dimensions
+        contiguous; batch and position strides are passed on (a slice of a wider buffer)."""
+        _require_gpu(t, field)
+        if tuple(t.shape) != tuple(shape) or t.dtype != dtype:
+            raise ValueError(f"{field}: expected {tuple(shape)} {dtype}, got {tuple(t.shape)} {t.dtype}")
+        if t.stride(3) != 1 or t.stride(2) != shape[3]:
+            raise ValueError(f"{field}: the two inner dimensions must be contiguous")
+        self.keep.append(t)
+        setattr(self.p, field, t.data_ptr())
+        contiguous = t.is_contiguous()
+        setattr(self.p, field + "_sb", 0 if contiguous else t.stride(0))
+        setattr(self.p, field + "_sl", 0 if contiguous else t.stride(1))
+        return t
+
     # ---- strided inputs -----------------------------------------------------------------------------
     def _strided(self, field, prefix, t, dtype):
         _require_gpu(t, field)
@@ -636,10 +651,11 @@ def _mamba_chunk_scan_combined_bwd(dout, x, dt, A, B, C, out, chunk_size, D=None
         assert out.shape == x.shape
         c.put("out_x", out.contiguous() if out.dtype == x.dtype else out.to(x.dtype).contiguous())
         dz = c.put("dz", dz) if dz is not None else c.new("dz", x.shape, x.dtype)
-    dx = c.put("dx", dx) if dx is not None else c.new("dx", x.shape, x.dtype)
+    c.p.dx_sb = c.p.dx_sl = c.p.dB_sb = c.p.dB_sl = c.p.dC_sb = c.p.dC_sl = 0
+    dx = c.put_grad("dx", dx, x.shape, x.dtype) if dx is not None else c.new("dx", x.shape, x.dtype)
     ddt = c.put("ddt", ddt) if ddt is not None else c.new("ddt", dt.shape, dt.dtype)
-    dB = c.put("dB", dB) if dB is not None else c.new("dB", B.shape, x.dtype)
-    dC = c.put("dC", dC) if dC is not None else c.new("dC", C.shape, x.dtype)
+    dB = c.put_grad("dB", dB, B.shape, x.dtype) if dB is not None else c.new("dB", B.shape, x.dtype)
+    dC = c.put_grad("dC", dC, C.shape, x.dtype) if dC is not None else c.new("dC", C.shape, x.dtype)
     dA = c.new("dA", (nheads,))
     dD = c.new("dD", tuple(D.shape)) if D is not None else None
     ddt_bias = c.new("ddt_bias", (nheads,)) if dt_bias is not None else None
@@ -663,9 +679,11 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
                 dt_limit=(0.0, _INF), return_final_states=False, *extra):
-        # extra: nothing (as in the reference), or (initial_states_f, initial_states_b[, seq_idx]) - extensions
-        assert len(extra) in (0, 2, 3)
-        initial_states, seq_idx = tuple(extra[:2]), (extra[2] if len(extra) == 3 else None)
+        # extra: nothing (as in the reference), or (initial_states_f, initial_states_b[, seq_idx[, grad_places]]) -
+        # extensions
+        assert len(extra) in (0, 2, 3, 4)
+        initial_states, seq_idx = tuple(extra[:2]), (extra[2] if len(extra) >= 3 else None)
+        ctx.grad_places = extra[3] if len(extra) == 4 else None
         ctx.seq_idx = seq_idx
         ctx.n_extra = len(extra)
         ctx.dt_dtype = dt.dtype
@@ -701,21 +719,30 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
             dout = torch.zeros_like(x)
         init = (init_f, init_b) if (init_f is not None or init_b is not None) else None
         dfin = tuple(dfinal) if any(t is not None for t in dfinal) else None
+        given = {}
+        if ctx.grad_places:
+            # destinations for dx / dB / dC handed out by the caller (e.g. slices of one buffer); one that does not fit the
+            # kernels' layout is not used
+            for name, like in (("dx", x), ("dB", B), ("dC", C)):
+                t = ctx.grad_places[name]() if ctx.grad_places.get(name) else None
+                if (t is not None and tuple(t.shape) == tuple(like.shape) and t.dtype == x.dtype and like.dtype == x.dtype
+                        and t.stride(3) == 1 and t.stride(2) == like.shape[3] and t.device == x.device):
+                    given[name] = t
         res = _mamba_chunk_scan_combined_bwd(
             dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
-            dt_limit=ctx.dt_limit, saved=saved, dfinal_states=dfin, initial_states=init, seq_idx=ctx.seq_idx)
+            dt_limit=ctx.dt_limit, saved=saved, dfinal_states=dfin, initial_states=init, seq_idx=ctx.seq_idx, **given)
         dx, ddt, dA, dB, dC, dD, dz, ddt_bias = res[:8]
         grads = (dx, ddt, dA, dB, dC, None, dD, dz, ddt_bias, None, None, None)
         if ctx.n_init:
             grads += tuple(res[8]) if init is not None else (None, None)
-        if ctx.n_extra == 3:
-            grads += (None,)
+        if ctx.n_extra >= 3:
+            grads += (None,) * (ctx.n_extra - 2)
         return grads
 
 
 def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_bias=None, dt_softplus=False,
                                 dt_limit=(0.0, _INF), return_final_states=False, initial_states_f=None,
-                                initial_states_b=None, seq_idx=None):
+                                initial_states_b=None, seq_idx=None, grad_places=None):
     """Bidirectional SSD:  y = SS(x) + flip(SS(flip(x))) + D*x, gated by silu(z) when z is given.
 
     Argument:
@@ -738,6 +765,9 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
         seq_idx: (batch, seqlen) integers, optional - not in the bidirectional reference (its causal sibling has it):
             constant over each of several sequences packed one behind the other; positions with different seq_idx do
             not interact in either direction.
+        grad_places: {"dx": f, "dB": f, "dC": f}, optional - not in the reference: callables asked in the backward pass for
+            the tensors these gradients are to be written into (shaped like x / B / C, the two inner dimensions contiguous;
+            e.g. slices of one buffer, which saves concatenating them when x, B, C are pieces of one tensor).
     Return:
         out: (batch, seqlen, nheads, headdim), or (out, final_states_f, final_states_b) with
         return_final_states=True (final states are (batch, nheads, headdim, dstate) float32)
@@ -764,6 +794,9 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
         if not return_final_states:
             return res.reshape(x.shape)
         return (res[0].reshape(x.shape),) + tuple(t.reshape(batch, nheads, headdim, -1) for t in res[1:])
+    if grad_places is not None:
+        return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
+                                              return_final_states, initial_states_f, initial_states_b, seq_idx, grad_places)
     if initial_states_f is None and initial_states_b is None and seq_idx is None:
         return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
                                               return_final_states)

@@ -141,6 +141,12 @@ typedef struct bimamba2_params {
     void *workspace;
     size_t workspace_bytes;
     void *stream;                   /* hipStream_t */
+    /* Element strides (batch, position) of the gradients dx (batch, seqlen, nheads, headdim), dB and dC (batch, seqlen,
+       ngroups, dstate); the inner dimensions are always contiguous.  A position stride of 0 (the default) means the
+       contiguous tensor.  With strides the three can be slices of one (batch, seqlen, channels) buffer, as x, B and C are
+       slices of the convolution's output in the BiMamba2 layer: no concatenation of the gradients afterwards.  Multiples of
+       8 elements (16 bytes) where the vector kernels are to run. */
+    int64_t dx_sb, dx_sl, dB_sb, dB_sl, dC_sb, dC_sl;
 } bimamba2_params;
 
 /* text of an error code */

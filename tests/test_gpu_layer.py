@@ -67,6 +67,9 @@ def test_bimamba2_layer_forward_backward():
     # small dt piece was copied there
     from bi_mamba2_amd.modules import _GradPieces
     assert _GradPieces.last_copied == (2,)
+    # (the same class serves the split of the convolution's output into x, B, C, whose backward runs first: its three
+    # gradients - the operator's dx, dB, dC - arrive in place as well)
+    assert _GradPieces.copies_log[-2:] == [(), (2,)]
 
 
 def test_bimamba2_layer_without_input_gradient_and_twice():
