@@ -92,6 +92,67 @@ __global__ __launch_bounds__(NTHREADS) void conv1d_silu_fwd_kernel(const bimamba
     }
 }
 
+// Tiled forward for 16-bit activations, channels a multiple of 64 and 16-byte aligned rows: a workgroup brings a tile of
+// 64 positions (plus the filter's reach on both sides) x 64 channels into LDS with 16-byte loads, every thread walks
+// 8 positions of one channel pair through a register window fed from there, and the results leave through LDS as 16-byte
+// vectors.  Four times fewer memory instructions than the register kernel above, whose lanes move 4 bytes each.
+constexpr int CONV_TP = 64, CONV_TC = 64;
+template <typename T, int W>
+__global__ __launch_bounds__(NTHREADS) void conv1d_silu_fwd_tiled_kernel(const bimamba2_conv_params p) {
+    static_assert(sizeof(T) == 2, "16-bit activations");
+    constexpr int H = W / 2, ROWS = CONV_TP + W - 1, SEG = CONV_TP / 8;
+    __shared__ __attribute__((aligned(16))) T xs[ROWS * CONV_TC];
+    __shared__ __attribute__((aligned(16))) T os[CONV_TP * CONV_TC];
+    const int c0 = blockIdx.x * CONV_TC, l0 = blockIdx.y * CONV_TP;
+    const int64_t b = blockIdx.z;
+    const int L = (int)p.seqlen;
+    const T *xin = reinterpret_cast<const T *>(p.x) + b * p.x_sb + c0;
+    // this thread's channel pair and run of positions
+    const int cp = threadIdx.x % 32, seg = threadIdx.x / 32;
+    float w[W][2], bias[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        bias[i] = p.has_bias ? p.bias[c0 + 2 * cp + i] : 0.f;
+#pragma unroll
+        for (int k = 0; k < W; ++k) w[k][i] = p.weight[(int64_t)(c0 + 2 * cp + i) * W + k];
+    }
+    for (int u = threadIdx.x; u < ROWS * (CONV_TC / 8); u += NTHREADS) {
+        const int r = u / (CONV_TC / 8), ch = (u % (CONV_TC / 8)) * 8, l = l0 - H + r;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (l >= 0 && l < L) v = *reinterpret_cast<const f32x4 *>(xin + (int64_t)l * p.x_sl + ch);
+        *reinterpret_cast<f32x4 *>(xs + r * CONV_TC + ch) = v;
+    }
+    __syncthreads();
+    typedef T Pair __attribute__((ext_vector_type(2)));
+    const T *col = xs + (seg * SEG) * CONV_TC + 2 * cp;     // row q of the segment: positions l0 + seg*SEG + q - H .. + H
+    float win[W][2];
+#pragma unroll
+    for (int j = 0; j < W - 1; ++j) {
+        const Pair v = *reinterpret_cast<const Pair *>(col + j * CONV_TC);
+        win[j][0] = to_f(v[0]); win[j][1] = to_f(v[1]);
+    }
+#pragma unroll
+    for (int q = 0; q < SEG; ++q) {
+        const Pair v = *reinterpret_cast<const Pair *>(col + (q + W - 1) * CONV_TC);
+        win[(q + W - 1) % W][0] = to_f(v[0]); win[(q + W - 1) % W][1] = to_f(v[1]);
+        Pair o;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            float a = bias[i];
+#pragma unroll
+            for (int k = 0; k < W; ++k) a = __builtin_fmaf(w[k][i], win[(q + k) % W][i], a);
+            o[i] = from_f<T>(a * sigmoid_f(a));
+        }
+        *reinterpret_cast<Pair *>(os + (seg * SEG + q) * CONV_TC + 2 * cp) = o;
+    }
+    __syncthreads();
+    T *out = reinterpret_cast<T *>(p.out) + (b * p.seqlen) * p.channels + c0;
+    for (int u = threadIdx.x; u < CONV_TP * (CONV_TC / 8); u += NTHREADS) {
+        const int r = u / (CONV_TC / 8), ch = (u % (CONV_TC / 8)) * 8, l = l0 + r;
+        if (l < L) *reinterpret_cast<f32x4 *>(out + (int64_t)l * p.channels + ch) = *reinterpret_cast<const f32x4 *>(os + r * CONV_TC + ch);
+    }
+}
+
 // Steps t = 0 .. TL + 2H - 1 visit positions l = l0 - H + t: g[l] is formed (needs x[l - H .. l + H]) and dx[l - H] leaves.
 template <typename T, int W, int VS>
 __global__ __launch_bounds__(NTHREADS) void conv1d_silu_bwd_kernel(const bimamba2_conv_params p, int ntl, int TL, float *part) {
@@ -216,6 +277,14 @@ static int launch_conv_w(const bimamba2_conv_params *p, bool bwd) {
     if (blocks <= 0 || blocks > 0x7fffffff) return BIMAMBA2_EUNSUPPORTED;
     hipStream_t s = reinterpret_cast<hipStream_t>(p->stream);
     if (!bwd) {
+        if constexpr (sizeof(T) == 2 && VS > 1) {
+            auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+            if (p->channels % CONV_TC == 0 && al16(p->x) && al16(p->out) && p->x_sb % 8 == 0 && p->x_sl % 8 == 0 && p->batch <= 65535) {
+                const dim3 grid(p->channels / CONV_TC, (unsigned)((p->seqlen + CONV_TP - 1) / CONV_TP), (unsigned)p->batch);
+                hipLaunchKernelGGL((conv1d_silu_fwd_tiled_kernel<T, W>), grid, dim3(NTHREADS), 0, s, *p);
+                return check_launch();
+            }
+        }
         hipLaunchKernelGGL((conv1d_silu_fwd_kernel<T, W, VS>), dim3((unsigned)blocks), dim3(NTHREADS), 0, s, *p, ntl, tl);
         return check_launch();
     }
