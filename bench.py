@@ -236,6 +236,8 @@ def cpu_baseline(w, budget_s=15.0):
 
 
 # The other benchmark configurations (the headline stays WORKLOAD): name -> (shape, z gate, backward too)
+SPIN_UP_S = 0.5     # seconds of untimed work on the device before the first timed leg
+
 OTHER_CONFIGS = {
     "config1_fwd": (dict(batch=4, seqlen=2048, nheads=32, headdim=64, ngroups=1, dstate=64, chunk_size=256), True, False),
     "config2_fwd": (dict(batch=2, seqlen=16384, nheads=48, headdim=64, ngroups=1, dstate=128, chunk_size=256), False, False),
@@ -257,6 +259,17 @@ def graphed(fn):
     with torch.cuda.graph(graph):
         fn()
     return graph.replay
+
+
+def spin_up(fn, seconds):
+    """Keeps the device busy with fn for `seconds` (untimed)."""
+    import torch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
 
 
 def timed(fn, n):
@@ -389,6 +402,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.config != "target":
+        spin_up(lambda: torch.empty(1 << 26, device=dev).fill_(1.0), SPIN_UP_S)
         line = layer_line(dev, args.steps, args.warmup) if args.config == "layer_config4" else config_line(args.config, dev, args.steps, args.warmup)
         print(json.dumps({args.config: line}))
         return
@@ -427,7 +441,11 @@ def main():
     # configurations, and only then the forward-only pass, the comparator and the step that `value` reports, each as
     # --warmup untimed and exactly --steps timed replays, with the per-kernel stage loops right behind them.  A training run
     # keeps the GPU busy for hours; timed right after start-up, with 25 steps behind it, the same step reads about 3 % slower
-    # than after a few hundred milliseconds of work (measured: 0.272 against 0.263 ms).
+    # than after a few hundred milliseconds of work (measured: 0.272 against 0.263 ms); the run therefore starts with
+    # SPIN_UP_S seconds of untimed steps as well, which covers the legs in front.
+    # the device is kept busy for SPIN_UP_S seconds before anything is timed (every leg below then sees the clocks of a
+    # GPU that is in use, whatever its place in the order)
+    spin_up(step, SPIN_UP_S)
     for _ in range(args.warmup):
         step()
     t_eager = timed(step, args.steps)
@@ -451,8 +469,8 @@ def main():
     if not args.no_extras:
         extras["gated_rmsnorm"] = rmsnorm_line(w, dtype, dev, max(10, args.steps))
         extras["conv1d_silu"] = conv_line(w, dtype, dev, max(10, args.steps))
-        extras["configs"] = {name: config_line(name, dev, max(10, args.steps // 2), 3) for name in OTHER_CONFIGS}
-        extras["layer_config4"] = layer_line(dev, max(10, args.steps // 2), 3)
+        extras["configs"] = {name: config_line(name, dev, max(30, args.steps), 10) for name in OTHER_CONFIGS}
+        extras["layer_config4"] = layer_line(dev, max(30, args.steps), 10)
     # ---- the operator's own legs, the reported step last
     for _ in range(args.warmup):
         fwd_fn()
@@ -574,6 +592,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "device_spin_up_s": SPIN_UP_S,
         "ms_per_step": t_step * 1e3,
         "launch": "eager (autograd, one Python call per pass)" if t_graph is None else "HIP graph replay of the captured forward + backward step",
         "eager": {"ms_per_step": t_eager * 1e3, "Mtokens_s": tokens / t_eager / 1e6},
