@@ -272,9 +272,11 @@ __device__ __forceinline__ void state_passing_bwd_vec_body(const bimamba2_params
             const int sj = min(s0 + j, nc - 1);            // past the last chunk: a valid chunk again, never used
             const int c = dir == 0 ? nc - 1 - sj : sj;
             dec[j] = cs[(int64_t)c * Q];
-            dp[j] = *reinterpret_cast<const f32x4 *>(ds + c * cstride);
+            // (both are read for the last time in the pass: past the caches)
+            dp[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(ds + c * cstride));
             if constexpr (PREV16) {
-                const V4 t = *reinterpret_cast<const V4 *>(prev16 + c * cstride);
+                typedef float f32x2 __attribute__((ext_vector_type(2)));
+                const V4 t = __builtin_bit_cast(V4, __builtin_nontemporal_load(reinterpret_cast<const f32x2 *>(prev16 + c * cstride)));
 #pragma unroll
                 for (int k = 0; k < 4; ++k) pv[j][k] = to_f(t.v[k]);
             } else {

@@ -617,7 +617,8 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const b
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int si = min(s0 + i, nc - 1), c = dir == 0 ? si : nc - 1 - si;
-            v[i] = *reinterpret_cast<const f32x4 *>(st + c * cstride);
+            // (with the 16-bit copies the per-chunk states are read for the last time here: past the caches)
+            v[i] = COPY ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(st + c * cstride)) : *reinterpret_cast<const f32x4 *>(st + c * cstride);
             d[i] = cs[(int64_t)c * Q];
         }
 #pragma unroll
