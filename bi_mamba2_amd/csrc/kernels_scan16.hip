@@ -87,9 +87,12 @@ template <int I, int N, class F> __device__ __forceinline__ void static_for(F &&
 // load16_to_lds(base + off) with the address in the scalar-base form: `base` wave-uniform, `off` this lane's 32-bit byte
 // offset.  The offset passes through an empty asm right in front of the load, which keeps the 64-bit add next to the load
 // (hoisted into another block it could not be folded into the instruction and would cost two registers per address).
+// NT: the lines are not kept in the caches (data that no later kernel of the pass reads).
+template <bool NT = false>
 __device__ __forceinline__ void load16_to_lds_at(const char *base, unsigned off, void *lds_wave_base) {
     asm volatile("" : "+v"(off));
-    load16_to_lds(base + off, lds_wave_base);
+    if constexpr (NT) __builtin_amdgcn_global_load_lds((gbl_ptr_t)(base + off), (lds_ptr_t)lds_wave_base, 16, 0, 2);
+    else load16_to_lds(base + off, lds_wave_base);
 }
 
 // A wave-uniform pointer, made visibly so (through 64-bit address arithmetic the compiler loses sight of it and would build
@@ -157,7 +160,8 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             else kp = reinterpret_cast<const char *>(reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * p.dout_sl + h * p.dout_sh + p0);
             kp = uniform_ptr(kp);
             // (rows behind the last K step are never read; their requests go to the clamped, valid row all the same)
-            load16_to_lds_at(kp, tile_off(ln, part, ks_bytes), smem + S16_XR + buf * 32768 + wave * 2048 + part * 1024);
+            // (the mirror is the last kernel of the pass that reads dout_x and the gradients of the entering states)
+            load16_to_lds_at<BWD>(kp, tile_off(ln, part, ks_bytes), smem + S16_XR + buf * 32768 + wave * 2048 + part * 1024);
         } else if (part == 2) {
             const int dir = wave >> 3;
             if (!(UNI && dir)) {
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 // thread t of a half brings row t/8, chunk position t%8 <- chunk (t%8) ^ (row%8)
                 const int row = (wave & 7) * 8 + (ln >> 3);
                 const unsigned soff = (unsigned)((row * 64 + (((ln & 7) ^ (row & 7)) << 3)) * sizeof(T));
-                load16_to_lds_at(uniform_ptr(src + so), soff, smem + S16_ST + (buf * 2 + dir) * 8192 + (wave & 7) * 1024);
+                load16_to_lds_at<BWD>(uniform_ptr(src + so), soff, smem + S16_ST + (buf * 2 + dir) * 8192 + (wave & 7) * 1024);
             }
         } else if (wave < 3) {
             // cs_f, cs_b, dt (waves 0, 1, 2): 256 floats each (entries past chunk_size are never used: clamped to stay inside)
