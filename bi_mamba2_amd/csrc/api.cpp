@@ -422,7 +422,7 @@ static int check_norm(const bimamba2_norm_params *p) {
     if (!p) return BIMAMBA2_EINVAL;
     if (p->rows < 0 || p->cols <= 0 || p->group_size <= 0 || p->cols % p->group_size) return BIMAMBA2_EINVAL;
     if (p->dtype != BIMAMBA2_F32 && p->dtype != BIMAMBA2_BF16 && p->dtype != BIMAMBA2_F16) return BIMAMBA2_EUNSUPPORTED;
-    if (p->group_size > 8192) return BIMAMBA2_EUNSUPPORTED;
+    if (p->group_size > 32768) return BIMAMBA2_EUNSUPPORTED;
     if (!p->x || !p->weight || (p->has_z && !p->z) || (p->has_bias && !p->bias)) return BIMAMBA2_EINVAL;
     return BIMAMBA2_OK;
 }

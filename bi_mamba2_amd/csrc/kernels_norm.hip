@@ -289,10 +289,200 @@ __global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_kernel(const bimam
     }
 }
 
+// ---- groups wider than 8192 columns (up to 32768: the reference's kernel takes 64 KB of a 16-bit row) ---------------
+// One WORKGROUP per (row, group): wave w owns the columns [w, w + 1) * NCH * 512 of the group, the row sums cross the
+// waves through LDS.  Otherwise the math of the kernels above (no registers held between the passes: the row is read again
+// from cache).
+__device__ __forceinline__ float block4_sum(float v, float *red, int wave, int lane) {
+    v = wave_sum(v);
+    __syncthreads();                               // (red may still be read from the sum before this one)
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
+template <typename T, int NCH>
+__global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_fwd_wide_kernel(const bimamba2_norm_params p, bool vec, bool wvec) {
+    __shared__ float red[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ngroups = p.cols / p.group_size, gs = p.group_size;
+    const int64_t item = blockIdx.x;
+    const int g = (int)(item % ngroups);
+    const int64_t row = item / ngroups;
+    const T *x = reinterpret_cast<const T *>(p.x) + row * p.x_rs + g * gs;
+    const T *z = p.has_z ? reinterpret_cast<const T *>(p.z) + row * p.z_rs + g * gs : nullptr;
+    T *out = reinterpret_cast<T *>(p.out) + row * p.out_rs + g * gs;
+    const float *w = p.weight + g * gs, *bias = p.has_bias ? p.bias + g * gs : nullptr;
+    const bool gate_first = p.has_z && !p.norm_before_gate;
+    float xv[NCH][8];
+    T zk[NCH][8];
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int c = ((wave * NCH + k) * 64 + lane) * 8;
+        load8(x + c, vec, gs - c, xv[k]);
+        if (p.has_z) {
+            float zv[8];
+            load8(z + c, vec, gs - c, zv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (gate_first) xv[k][i] *= silu_f(zv[i]);
+                else zk[k][i] = from_f<T>(zv[i]);
+            }
+        }
+    }
+    if (p.layer_norm) {
+        float sm = 0.f;
+#pragma unroll
+        for (int k = 0; k < NCH; ++k)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sm += xv[k][i];
+        const float mean = block4_sum(sm, red, wave, lane) / gs;
+        if (threadIdx.x == 0 && p.mean) p.mean[item] = mean;
+#pragma unroll
+        for (int k = 0; k < NCH; ++k)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (((wave * NCH + k) * 64 + lane) * 8 + i < gs) xv[k][i] -= mean;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += xv[k][i] * xv[k][i];
+    ss = block4_sum(ss, red, wave, lane);
+    const float rstd = 1.f / sqrtf(ss / gs + p.eps);
+    if (threadIdx.x == 0 && p.rstd) p.rstd[item] = rstd;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int c = ((wave * NCH + k) * 64 + lane) * 8;
+        if (c >= gs) continue;
+        float wv[8], yv[8];
+        load8(w + c, wvec, gs - c, wv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) yv[i] = xv[k][i] * rstd * wv[i];
+        if (bias) {
+            float bv[8];
+            load8(bias + c, wvec, gs - c, bv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) yv[i] += bv[i];
+        }
+        if (p.has_z && p.norm_before_gate) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) yv[i] *= silu_f(to_f(zk[k][i]));
+        }
+        store8(out + c, vec, gs - c, yv);
+    }
+}
+
+// grid (row blocks, groups): workgroup bx handles rows bx, bx + gridDim.x, ... and leaves ONE partial row of dweight / dbias
+// (each wave the columns it owns)
+template <typename T, int NCH, bool HAS_BIAS>
+__global__ __launch_bounds__(NTHREADS) void rmsnorm_gated_bwd_wide_kernel(const bimamba2_norm_params p, bool vec, bool wvec, float *part_w,
+                                                                          float *part_b) {
+    __shared__ float red[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ngroups = p.cols / p.group_size, gs = p.group_size;
+    const int g = blockIdx.y;
+    const float *w = p.weight + g * gs, *bias = HAS_BIAS ? p.bias + g * gs : nullptr;
+    const bool gate_first = p.has_z && !p.norm_before_gate, gate_last = p.has_z && p.norm_before_gate;
+    float dw[NCH][8], db[HAS_BIAS ? NCH : 1][8];
+#pragma unroll
+    for (int k = 0; k < NCH; ++k)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            dw[k][i] = 0.f;
+            if (HAS_BIAS) db[k][i] = 0.f;
+        }
+    for (int64_t row = blockIdx.x; row < p.rows; row += gridDim.x) {
+        const T *x = reinterpret_cast<const T *>(p.x) + row * p.x_rs + g * gs;
+        const T *z = p.has_z ? reinterpret_cast<const T *>(p.z) + row * p.z_rs + g * gs : nullptr;
+        const T *dout = reinterpret_cast<const T *>(p.dout) + row * p.dout_rs + g * gs;
+        T *dx = reinterpret_cast<T *>(p.dx) + row * p.dx_rs + g * gs;
+        T *dz = p.has_z ? reinterpret_cast<T *>(p.dz) + row * p.dz_rs + g * gs : nullptr;
+        const float rstd = p.rstd[row * ngroups + g];
+        const float mean = p.layer_norm ? p.mean[row * ngroups + g] : 0.f;
+        // (the same per-element terms as in rmsnorm_gated_bwd_kernel)
+        auto element = [&](int k, int c, bool first, float (&xhat)[8], float (&wdy)[8], float (&slv)[8], float (&g2v)[8]) {
+            float xv[8], dy[8], zv[8], wv[8], bv[8], dzv[8];
+            load8(x + c, vec, gs - c, xv);
+            load8(dout + c, vec, gs - c, dy);
+            load8(w + c, wvec, gs - c, wv);
+            if (HAS_BIAS && first) load8(bias + c, wvec, gs - c, bv);
+            if (p.has_z) load8(z + c, vec, gs - c, zv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float sg = 0.f, si = 1.f, ds = 0.f;
+                if (p.has_z) {
+                    sg = sigmoid_f(zv[i]);
+                    si = zv[i] * sg;
+                    ds = sg * (1.f + zv[i] * (1.f - sg));
+                }
+                slv[i] = si;
+                g2v[i] = xv[i] * ds;
+                xhat[i] = ((gate_first ? xv[i] * si : xv[i]) - mean) * rstd;
+                if (c + i >= gs) xhat[i] = 0.f;
+                if (gate_last) {
+                    dzv[i] = dy[i] * (xhat[i] * wv[i] + (HAS_BIAS && first ? bv[i] : 0.f)) * ds;
+                    dy[i] *= si;
+                }
+                wdy[i] = wv[i] * dy[i];
+                if (first) {
+                    dw[k][i] += dy[i] * xhat[i];
+                    if (HAS_BIAS) db[k][i] += dy[i];
+                }
+            }
+            if (gate_last && first) store8(dz + c, vec, gs - c, dzv);
+        };
+        float c1 = 0.f, c2 = 0.f;
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) {
+            const int c = ((wave * NCH + k) * 64 + lane) * 8;
+            if (c >= gs) continue;
+            float xhat[8], wdy[8], slv[8], g2v[8];
+            element(k, c, true, xhat, wdy, slv, g2v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                c1 += xhat[i] * wdy[i];
+                c2 += wdy[i];
+            }
+        }
+        c1 = block4_sum(c1, red, wave, lane) / gs;
+        c2 = p.layer_norm ? block4_sum(c2, red, wave, lane) / gs : 0.f;
+#pragma unroll
+        for (int k = 0; k < NCH; ++k) {
+            const int c = ((wave * NCH + k) * 64 + lane) * 8;
+            if (c >= gs) continue;
+            float xhat[8], wdy[8], slv[8], g2v[8], dxv[8], dzv[8];
+            element(k, c, false, xhat, wdy, slv, g2v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float dxg = (wdy[i] - xhat[i] * c1 - c2) * rstd;
+                dxv[i] = gate_first ? dxg * slv[i] : dxg;
+                dzv[i] = dxg * g2v[i];
+            }
+            store8(dx + c, vec, gs - c, dxv);
+            if (gate_first) store8(dz + c, vec, gs - c, dzv);
+        }
+    }
+    const int64_t prow = (int64_t)blockIdx.x * p.cols + g * gs;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int c = ((wave * NCH + k) * 64 + lane) * 8;
+        if (c >= gs) continue;
+        store8(part_w + prow + c, false, gs - c, dw[k]);
+        if (HAS_BIAS) store8(part_b + prow + c, false, gs - c, db[k]);
+    }
+}
+
 // workgroups along the rows, and partial rows of dweight / dbias they leave (one per workgroup up to groups of 4096
-// columns, one per wave above)
-static int norm_row_blocks(const bimamba2_norm_params *p) { return (int)std::min<int64_t>((p->rows + 3) / 4, p->group_size <= 4096 ? 1024 : 256); }
-static int norm_partial_rows(const bimamba2_norm_params *p) { return norm_row_blocks(p) * (p->group_size <= 4096 ? 1 : 4); }
+// columns, one per wave above; one per workgroup again for the wide kernels, beyond 8192 columns)
+static int norm_row_blocks(const bimamba2_norm_params *p) {
+    if (p->group_size > 8192) return (int)std::min<int64_t>(p->rows, 512);
+    return (int)std::min<int64_t>((p->rows + 3) / 4, p->group_size <= 4096 ? 1024 : 256);
+}
+static int norm_partial_rows(const bimamba2_norm_params *p) {
+    return norm_row_blocks(p) * ((p->group_size <= 4096 || p->group_size > 8192) ? 1 : 4);
+}
 
 size_t norm_workspace_bytes(const bimamba2_norm_params *p) {
     return (size_t)norm_partial_rows(p) * p->cols * sizeof(float) * (p->has_bias ? 2 : 1);
@@ -371,9 +561,41 @@ static int launch_norm_nch(const bimamba2_norm_params *p, bool bwd) {
     return check_launch();
 }
 
+// groups of more than 8192 columns: NCH chunks of 512 per wave, four waves per (row, group)
+template <typename T, int NCH>
+static int launch_norm_wide(const bimamba2_norm_params *p, bool bwd) {
+    const bool vec = norm_vec_ok(p, bwd, (int)sizeof(T));
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    const bool wvec = p->group_size % 4 == 0 && al(p->weight) && (!p->has_bias || al(p->bias));
+    const int ngroups = p->cols / p->group_size;
+    if (!bwd) {
+        const int64_t items = (int64_t)p->rows * ngroups;
+        if (items <= 0) return BIMAMBA2_OK;
+        if (items > 0x7fffffff) return BIMAMBA2_EUNSUPPORTED;
+        hipLaunchKernelGGL((rmsnorm_gated_fwd_wide_kernel<T, NCH>), dim3((unsigned)items), dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec);
+        return check_launch();
+    }
+    const int nb = norm_row_blocks(p), npr = norm_partial_rows(p);
+    float *part_w = reinterpret_cast<float *>(p->workspace);
+    float *part_b = p->has_bias ? part_w + (size_t)npr * p->cols : nullptr;
+    const dim3 grid(std::max(nb, 1), ngroups);
+    if (p->has_bias) hipLaunchKernelGGL((rmsnorm_gated_bwd_wide_kernel<T, NCH, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+    else hipLaunchKernelGGL((rmsnorm_gated_bwd_wide_kernel<T, NCH, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, vec, wvec, part_w, part_b);
+    int rc = check_launch();
+    if (rc) return rc;
+    hipLaunchKernelGGL(colsum_kernel, dim3((p->cols + 15) / 16, p->has_bias ? 2 : 1), dim3(NTHREADS), 0, stream_of(p), part_w, p->dweight,
+                       part_b, p->dbias, npr, p->cols);
+    return check_launch();
+}
+
 template <typename T>
 static int launch_norm_t(const bimamba2_norm_params *p, bool bwd) {
     const int nch = (p->group_size + 511) / 512;
+    if (nch > 16) {
+        if (nch <= 32) return launch_norm_wide<T, 8>(p, bwd);
+        if (nch <= 64) return launch_norm_wide<T, 16>(p, bwd);
+        return BIMAMBA2_EUNSUPPORTED;
+    }
     if (nch <= 1) return launch_norm_nch<T, 1>(p, bwd);
     if (nch <= 2) return launch_norm_nch<T, 2>(p, bwd);
     if (nch == 3) return launch_norm_nch<T, 3>(p, bwd);    // 1536 columns: expand 2 x d_model 768, the benchmark layer's width

@@ -154,7 +154,7 @@ class LayerNormFn(torch.autograd.Function):
                 dz, None, None, None, None, None)
 
 
-MAX_GROUP = 8192      # columns per normalisation group (bimamba2_rmsnorm_gated_fwd / _bwd refuse more)
+MAX_GROUP = 32768     # columns per normalisation group (bimamba2_rmsnorm_gated_fwd / _bwd refuse more)
 
 
 def layernorm_fn(x, weight, bias, z=None, eps=1e-6, group_size=None, norm_before_gate=True, is_rms_norm=False):

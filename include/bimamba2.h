@@ -248,7 +248,8 @@ int bimamba2_chunk_cumsum_bwd(const bimamba2_params *p);
  *   xg = x (norm_before_gate) or x * silu(z);  y = xg * rstd * weight (+ bias), rstd = 1/sqrt(mean_group(xg^2) + eps);
  *   out = y * silu(z) (norm_before_gate) or y.
  * Rows of `cols` elements (last dim contiguous, row strides in elements), groups of `group_size` consecutive columns
- * (group_size divides cols, <= 8192).  Replaces rmsnorm_fn / RMSNorm of the reference, i.e. _layer_norm_fwd
+ * (group_size divides cols, <= 32768: 64 KB of a 16-bit row, the reference kernel's limit; beyond 8192 columns a workgroup
+ * instead of a wave works on a (row, group)).  Replaces rmsnorm_fn / RMSNorm of the reference, i.e. _layer_norm_fwd
  * (src/ssd/bi/layernorm_gated.py:108-152, kernel :45-105) and _layer_norm_bwd (:271-330, kernel :155-268) with
  * is_rms_norm = True; math of rms_norm_ref (:18-39). */
 typedef struct bimamba2_norm_params {

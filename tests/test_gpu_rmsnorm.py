@@ -19,8 +19,12 @@ CASES = [
     ((2, 64, 2048), 512, True, True, False, torch.bfloat16),
     ((5, 37, 1536), None, True, False, True, torch.bfloat16),    # 3 x 512 columns: the baseline layer's width (d_model 768)
     ((8, 4096), None, True, False, True, torch.float16),
-    ((3, 8192), None, False, False, True, torch.bfloat16),       # the widest supported group
+    ((3, 8192), None, False, False, True, torch.bfloat16),       # the widest group one wave holds
     ((600, 2, 128), None, True, True, True, torch.float32),      # more rows than partial-sum slots
+    ((5, 16384), None, True, False, True, torch.bfloat16),       # beyond 8192 columns: one workgroup per (row, group)
+    ((3, 2, 24576), 12288, True, True, False, torch.float16),    # two wide groups, bias, gate first
+    ((4, 9000), None, False, True, True, torch.float32),         # wide, no gate, width not a multiple of 512
+    ((2, 32768), None, True, False, True, torch.bfloat16),       # the widest group (64 KB of a 16-bit row, as the reference)
 ]
 
 
