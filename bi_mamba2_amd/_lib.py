@@ -42,7 +42,7 @@ ENTRY_POINTS = (
     "bimamba2_fwd", "bimamba2_bwd", "bimamba2_fwd_static",
     "bimamba2_chunk_cumsum_fwd", "bimamba2_bmm_chunk_fwd", "bimamba2_chunk_state_fwd",
     "bimamba2_state_passing_fwd", "bimamba2_chunk_scan_fwd",
-    "bimamba2_chunk_scan_bwd_dz", "bimamba2_chunk_scan_bwd_dstates", "bimamba2_state_passing_bwd",
+    "bimamba2_chunk_scan_bwd_dz", "bimamba2_chunk_scan_bwd_dstates", "bimamba2_chunk_scan_bwd_dz_dstates", "bimamba2_state_passing_bwd",
     "bimamba2_chunk_scan_bwd_dx", "bimamba2_chunk_state_bwd_db", "bimamba2_chunk_scan_bwd_dc",
     "bimamba2_chunk_scan_bwd_dcb", "bimamba2_bmm_chunk_bwd", "bimamba2_chunk_cumsum_bwd",
 )

@@ -237,6 +237,14 @@ int bimamba2_chunk_scan_bwd_dstates(const bimamba2_params *p) {
     return launch_chunk_state(p, true);
 }
 
+int bimamba2_chunk_scan_bwd_dz_dstates(const bimamba2_params *p) {
+    TRY(check_problem(p));
+    if (!p->has_z) return BIMAMBA2_EINVAL;
+    REQUIRE(p->z); REQUIRE(p->dout); REQUIRE(p->out_x); REQUIRE(p->dz); REQUIRE(p->dout_x);
+    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->dstates_f); REQUIRE(p->dstates_b);
+    return launch_bwd_dz_dstates(p);       // BIMAMBA2_EUNSUPPORTED where only the two separate kernels exist
+}
+
 int bimamba2_state_passing_bwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->cs_f); REQUIRE(p->cs_b);
@@ -365,20 +373,23 @@ int bimamba2_bwd(const bimamba2_params *p) {
     const bool need_cbt = !scan_recomputes_cb(&q, true), need_cb = need_cbt || !dcb_recomputes_cb(&q);
     if (need_cb) TRY(bimamba2_bmm_chunk_fwd(&q));  // CB for the dCB kernel, CB^T for the dx kernel, unless they rebuild it
     else q.CB = nullptr;
-    if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
+    // dz and dstates as one launch where the kernel for it exists (dout_x goes from the first to the second inside the workgroup)
+    const bool dz_dstates = q.has_z && bwd_dz_dstates_fused(&q);
+    if (dz_dstates) TRY(bimamba2_chunk_scan_bwd_dz_dstates(&q));
+    else if (q.has_z) TRY(bimamba2_chunk_scan_bwd_dz(&q));
     // the dCB kernel is bound by instruction issue and moves little data: right behind dz it runs while the memory system
     // still writes back dz's output, which the memory-bound kernels after it would otherwise wait behind
     if (bwd_dcb_sp_merged(&q)) {
         // the backward state passing (streams, few instructions) rides along with the dCB kernel in one launch
         TRY(bimamba2_chunk_scan_bwd_dc(&q));
-        TRY(bimamba2_chunk_scan_bwd_dstates(&q));
+        if (!dz_dstates) TRY(bimamba2_chunk_scan_bwd_dstates(&q));
         REQUIRE(q.x); REQUIRE(q.dt_out); REQUIRE(q.cs_f); REQUIRE(q.cs_b); REQUIRE(q.dCB); REQUIRE(q.dCBT); REQUIRE(q.da_intra);
         REQUIRE(q.dstates_f); REQUIRE(q.ddA_chunk_f); REQUIRE(q.ddA_chunk_b);
         if (q.has_z) REQUIRE(q.dout_x); else REQUIRE(q.dout);
         TRY(launch_bwd_dcb_sp(&q, dcb16));
     } else {
         TRY(bimamba2_chunk_scan_bwd_dcb(&q));
-        TRY(bimamba2_chunk_scan_bwd_dstates(&q));
+        if (!dz_dstates) TRY(bimamba2_chunk_scan_bwd_dstates(&q));
         TRY(bimamba2_chunk_scan_bwd_dc(&q));           // (between the two memory-bound state kernels: measured best)
         TRY(bimamba2_state_passing_bwd(&q));
     }

@@ -44,10 +44,11 @@ __device__ __forceinline__ float raw_global_load_f32(const float *p) {
     asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
     return v;
 }
-template <typename V> __device__ __forceinline__ V raw_global_load_b128(const void *p) {
+template <typename V, bool NT = false> __device__ __forceinline__ V raw_global_load_b128(const void *p) {   // NT: non-temporal
     static_assert(sizeof(V) == 16, "16-byte value");
     V v;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    if constexpr (NT) asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(v) : "v"(p) : "memory");
+    else asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
     return v;
 }
 __device__ __forceinline__ unsigned raw_global_load_u16(const void *p) {      // zero-extended 16 bits

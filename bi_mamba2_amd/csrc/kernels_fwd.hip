@@ -438,6 +438,158 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// dz and dstates in one pass (16-bit types, z gate, dstate 64, headdim % 64 == 0, chunk_size % 32 == 0): the workgroup of
+// (b, c, h, 64 channels) takes dout, z and the ungated forward output through registers, 32 positions at a time and two
+// steps ahead, writes dz and dout_x = dout silu(z) for the later kernels and puts dout_x into LDS where the other kernel
+// requests it from memory: dstates is then the chunk-state product of dout_x with C as above.  dout_x is not read back
+// by this kernel and the launch of the dz kernel goes away.
+// Order of a wave's vector memory operations: two loads for the weight tables, then per step dout, z, out_x (registers)
+// and its 8 rows of the C tile (direct to LDS); the stores of a step follow its loads by two steps.  Loads complete in
+// order among themselves, stores do not keep that order, so a wait counts the younger loads only.
+// ---------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void bwd_dz_dstates_kernel(const bimamba2_params p, int nc) {
+    typedef Mma<T> M;
+    typedef typename M::Frag Frag;
+    static_assert(sizeof(T) == 2, "16-bit operands");
+    constexpr int KX = 2, KB = 3;                          // slots of the dout_x ring (written here) and of the C ring (requests 2 steps ahead)
+    __shared__ __attribute__((aligned(16))) T xt[KX * 32 * 64];
+    __shared__ __attribute__((aligned(16))) T bt[KB * 32 * 64];
+    __shared__ __attribute__((aligned(16))) float wf[BIMAMBA2_MAX_CHUNK], wb[BIMAMBA2_MAX_CHUNK];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lr = lane & 15, lg = lane >> 4;
+    const int pt = blockIdx.y;
+    const int h = blockIdx.z % p.nheads, bc = blockIdx.z / p.nheads, c = bc % nc, b = bc / nc;
+    const int g = h / (p.nheads / p.ngroups);
+    const int Q = p.chunk_size, N = p.dstate, P = p.headdim;
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int nsteps = ((limit + 31) & ~31) / 32;
+    const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
+    // this lane's 16 bytes of a step: row 8 wave + lane / 8 of the step's 32, the column chunk that the swizzled tile holds
+    // at lane % 8 (the swizzle of a row does not depend on the step)
+    const int row0 = 8 * wave + (lane >> 3);
+    const int col = pt * 64 + (((lane & 7) ^ tile64_swz(row0)) << 3);
+    const T *zp = reinterpret_cast<const T *>(p.z) + b * p.z_sb + (int64_t)c * Q * p.z_sl + h * p.z_sh + col;
+    const T *dp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * p.dout_sl + h * p.dout_sh + col;
+    const int64_t os = (int64_t)p.nheads * P;               // row stride of out_x, dz, dout_x
+    const int64_t ob = ((int64_t)b * p.seqlen + (int64_t)c * Q) * os + (int64_t)h * P + col;
+    const T *oxp = reinterpret_cast<const T *>(p.out_x) + ob;
+    T *dzp = reinterpret_cast<T *>(p.dz) + ob;
+    T *doxp = reinterpret_cast<T *>(p.dout_x) + ob;
+    const int64_t bs = p.C_sl;
+    const T *bp = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * bs + g * p.C_sg + (((lane & 7) ^ tile64_swz(row0)) << 3);
+    float r_cf, r_cb;
+    {
+        const int q = min((int)threadIdx.x, limit - 1);
+        r_cf = raw_global_load_f32(p.cs_f + o + q);
+        r_cb = raw_global_load_f32(p.cs_b + o + q);
+    }
+    f32x4 rd[2], rz[2], ro[2];                               // two steps in flight
+    auto issue = [&](auto S) {
+        constexpr int s = decltype(S)::value;
+        const int row = min(32 * s + row0, limit - 1);
+        rd[s % 2] = raw_global_load_b128<f32x4>(dp + (int64_t)row * p.dout_sl);
+        rz[s % 2] = raw_global_load_b128<f32x4>(zp + (int64_t)row * p.z_sl);
+        ro[s % 2] = raw_global_load_b128<f32x4>(oxp + (int64_t)row * os);
+        load16_to_lds(bp + (int64_t)row * bs, bt + ((s % KB) * 4 + wave) * 512);
+    };
+    issue(std::integral_constant<int, 0>());
+    if (nsteps > 1) issue(std::integral_constant<int, 1>());
+    const unsigned wf_a = lds_addr(wf), wb_a = lds_addr(wb);
+    if (nsteps > 1) wait_vmcnt<8>(); else wait_vmcnt<4>();
+    raw_lds_use(r_cf); raw_lds_use(r_cb);
+    {
+        const int q = threadIdx.x;
+        raw_lds_write_at<0>(wf_a + q * 4, q < limit ? __expf(r_cf) : 0.f);
+        raw_lds_write_at<0>(wb_a + q * 4, q < limit ? __expf(r_cb) : 0.f);
+        raw_lds_wait();
+    }
+    const int kk = 8 * lg + (lr >> 2), nn = 4 * (lr & 3);
+    const unsigned xa_lo = lds_addr(xt) + tile64_tr_offset(kk, wave * 16 + nn), xa_hi = lds_addr(xt) + tile64_tr_offset(kk + 4, wave * 16 + nn);
+    unsigned ba_lo[4], ba_hi[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        ba_lo[j] = lds_addr(bt) + tile64_tr_offset(kk, j * 16 + nn);
+        ba_hi[j] = lds_addr(bt) + tile64_tr_offset(kk + 4, j * 16 + nn);
+    }
+    const unsigned xw = lds_addr(xt) + wave * 1024 + lane * 16;     // where this lane's 16 bytes of dout_x go (slot 0)
+    const unsigned wfl = wf_a + 32 * lg, wbl = wb_a + 32 * lg;
+    f32x4 accf[4] = {}, accb[4] = {};
+    auto kstep = [&](auto S) {
+        constexpr int s = decltype(S)::value;
+        constexpr int XO = (s % KX) * 32 * 128, BO = (s % KB) * 32 * 128, WO = s * 32 * 4;
+        if (s + 1 < nsteps) wait_vmcnt<4>(); else wait_vmcnt<0>();      // this wave's loads of step s have landed
+        raw_lds_use(rd[s % 2]); raw_lds_use(rz[s % 2]); raw_lds_use(ro[s % 2]);
+        {
+            const Vec16<T> a = __builtin_bit_cast(Vec16<T>, rz[s % 2]), d = __builtin_bit_cast(Vec16<T>, rd[s % 2]),
+                           e = __builtin_bit_cast(Vec16<T>, ro[s % 2]);
+            Vec16<T> r1, r2;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float zv = to_f(a.v[i]), dv = to_f(d.v[i]), ov = to_f(e.v[i]);
+                const float sg = sigmoid_f(zv);
+                r1.v[i] = from_f<T>(dv * ov * sg * (1.f + zv * (1.f - sg)));
+                r2.v[i] = from_f<T>(dv * zv * sg);
+            }
+            raw_lds_write128_at<XO>(xw, __builtin_bit_cast(f32x4, r2));
+            const int row = 32 * s + row0;
+            if (row < limit) {
+                __builtin_nontemporal_store(__builtin_bit_cast(f32x4, r1), reinterpret_cast<f32x4 *>(dzp + (int64_t)row * os));
+                *reinterpret_cast<f32x4 *>(doxp + (int64_t)row * os) = __builtin_bit_cast(f32x4, r2);
+            }
+        }
+        raw_lds_wait();
+        raw_lds_barrier();          // dout_x and everybody's C rows of step s are in LDS; the slots of step s - 1 are free again
+        if constexpr (s + 2 < 8) {
+            if (s + 2 < nsteps) issue(std::integral_constant<int, s + 2>());
+        }
+        i16x4 alo = raw_lds_tr16_read_at<XO>(xa_lo), ahi = raw_lds_tr16_read_at<XO>(xa_hi);
+        f32x4 f0 = raw_lds_read_at<f32x4, WO>(wfl), f1 = raw_lds_read_at<f32x4, WO + 16>(wfl);
+        f32x4 r0 = raw_lds_read_at<f32x4, WO>(wbl), r1 = raw_lds_read_at<f32x4, WO + 16>(wbl);
+        i16x4 blo[4], bhi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { blo[j] = raw_lds_tr16_read_at<BO>(ba_lo[j]); bhi[j] = raw_lds_tr16_read_at<BO>(ba_hi[j]); }
+        raw_lds_wait();
+        raw_lds_use(alo); raw_lds_use(ahi); raw_lds_use(f0); raw_lds_use(f1); raw_lds_use(r0); raw_lds_use(r1);
+        const Frag a = __builtin_bit_cast(Frag, __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7));
+        float vf[8], vb[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float v = to_f(a[i]);
+            vf[i] = v * (i < 4 ? f0[i & 3] : f1[i & 3]);
+            vb[i] = v * (i < 4 ? r0[i & 3] : r1[i & 3]);
+        }
+        const Frag af = M::pack(vf), ab = M::pack(vb);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            raw_lds_use(blo[j]); raw_lds_use(bhi[j]);
+            const Frag bfr = __builtin_bit_cast(Frag, __builtin_shufflevector(blo[j], bhi[j], 0, 1, 2, 3, 4, 5, 6, 7));
+            accf[j] = M::mma(af, bfr, accf[j]);
+            accb[j] = M::mma(ab, bfr, accb[j]);
+        }
+    };
+    static_assert(BIMAMBA2_MAX_CHUNK == 256, "eight K steps of 32 positions");
+    kstep(std::integral_constant<int, 0>());
+    if (nsteps > 1) kstep(std::integral_constant<int, 1>());
+    if (nsteps > 2) kstep(std::integral_constant<int, 2>());
+    if (nsteps > 3) kstep(std::integral_constant<int, 3>());
+    if (nsteps > 4) kstep(std::integral_constant<int, 4>());
+    if (nsteps > 5) kstep(std::integral_constant<int, 5>());
+    if (nsteps > 6) kstep(std::integral_constant<int, 6>());
+    if (nsteps > 7) kstep(std::integral_constant<int, 7>());
+    float *of = p.dstates_f + (int64_t)blockIdx.z * P * N;
+    float *obk = p.dstates_b + (int64_t)blockIdx.z * P * N;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int pp = pt * 64 + wave * 16 + lg * 4 + i, n = j * 16 + lr;
+            of[(int64_t)pp * N + n] = accf[j][i];
+            obk[(int64_t)pp * N + n] = accb[j][i];
+        }
+}
+
 // =========================================================================================================
 // inter-chunk recurrences, both directions, in place:
 //   forward : prev_f[0] = 0, prev_f[c+1] = e^{tot_c} prev_f[c] + S_f[c]   (final_f = value after the last chunk)
@@ -587,6 +739,24 @@ bool chunk_state_does_cumsum(const bimamba2_params *p) {
     if (p->seq_idx) return false;                 // packed sequences: the stand-alone cumsum kernel applies the cuts
     return p->dtype != BIMAMBA2_F32 && p->headdim % 64 == 0 && p->dstate % 64 == 0 && p->chunk_size % 32 == 0 && al(p->Bm) &&
            mult(p->B_sb, p->B_sl, p->B_sg) && al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
+}
+
+// whether launch_bwd_dz_dstates(p) exists for this problem
+bool bwd_dz_dstates_fused(const bimamba2_params *p) {
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
+    return p->has_z && !p->causal && p->dtype != BIMAMBA2_F32 && p->headdim % 64 == 0 && p->dstate == 64 && p->chunk_size % 32 == 0 &&
+           al(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg) && al(p->z) && mult(p->z_sb, p->z_sl, p->z_sh) && al(p->dout) &&
+           mult(p->dout_sb, p->dout_sl, p->dout_sh) && al(p->out_x) && al(p->dz) && al(p->dout_x);
+}
+
+int launch_bwd_dz_dstates(const bimamba2_params *p) {
+    if (!bwd_dz_dstates_fused(p)) return BIMAMBA2_EUNSUPPORTED;
+    const int nc = nchunks(p);
+    dim3 grid(1, p->headdim / 64, p->batch * nc * p->nheads);
+    if (p->dtype == BIMAMBA2_BF16) hipLaunchKernelGGL(bwd_dz_dstates_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    else hipLaunchKernelGGL(bwd_dz_dstates_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    return check_launch();
 }
 
 // The same with 16-byte accesses and one direction per workgroup (blockIdx.z = 2 b + dir); the loads of 8 chunks go out

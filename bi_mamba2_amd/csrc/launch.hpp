@@ -22,6 +22,8 @@ bool scan_recomputes_cb(const bimamba2_params *p, bool bwd);
 bool dcb_recomputes_cb(const bimamba2_params *p);
 
 int launch_bwd_dz(const bimamba2_params *p);
+bool bwd_dz_dstates_fused(const bimamba2_params *p);   // dz and dstates as one launch
+int launch_bwd_dz_dstates(const bimamba2_params *p);
 int launch_state_passing_bwd(const bimamba2_params *p);
 int launch_bwd_dbdc(const bimamba2_params *p, bool is_db);
 int launch_bwd_dcb(const bimamba2_params *p);

@@ -336,6 +336,24 @@ def _chunk_scan_bwd_dstates(C, dA_cumsum_f, dA_cumsum_b, dout, headdim=None):
     return df, db
 
 
+def _chunk_scan_bwd_dz_dstates(z, out_x, dout, C, dA_cumsum_f, dA_cumsum_b):
+    """_chunk_scan_bwd_dz and _chunk_scan_bwd_dstates as one launch -> dz, dout_x, dstates_f, dstates_b.  Raises for
+    problems that only the two separate kernels cover (see include/bimamba2.h)."""
+    batch, seqlen, nheads, hd = dout.shape
+    _, _, nchunks, chunk_size = dA_cumsum_f.shape
+    _, _, ngroups, dstate = C.shape
+    assert z.shape == dout.shape and out_x.shape == dout.shape
+    c = _Call(batch, seqlen, nheads, hd, ngroups, dstate, chunk_size, dout.dtype, dout.device)
+    c.set_z(z); c.set_dout(dout); c.set_C(C)
+    c.put("out_x", out_x.contiguous(), dout.dtype)
+    c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
+    dz = c.new("dz", dout.shape, dout.dtype); dout_x = c.new("dout_x", dout.shape, dout.dtype)
+    shape = (batch, nchunks, nheads, hd, dstate)
+    df = c.new("dstates_f", shape); db = c.new("dstates_b", shape)
+    c.run("bimamba2_chunk_scan_bwd_dz_dstates")
+    return dz, dout_x, df, db
+
+
 def _state_passing_bwd(states_f, states_b, dA_cumsum_f, dA_cumsum_b, dstates_f, dstates_b):
     """states_*: states entering each chunk; dstates_*: gradient w.r.t. them.
     -> gradient w.r.t. each chunk's own state (both directions) and ddA_chunk_f/b (batch, nheads, nchunks)."""

@@ -221,6 +221,12 @@ int bimamba2_chunk_scan_bwd_dz(const bimamba2_params *p);
 /* dout (dout_x when has_z), Cm, cs_f, cs_b -> dstates_f/b.  Replaces _chunk_scan_bwd_dstates
  * (src/ssd/bi/ssd_chunk_scan.py:1801-1826). */
 int bimamba2_chunk_scan_bwd_dstates(const bimamba2_params *p);
+/* The two above as one launch: z, out_x, dout, Cm, cs_f, cs_b -> dz, dout_x, dstates_f/b, with the same results.  A
+ * workgroup forms dout_x for its (batch, chunk, head) and multiplies it with C without reading it back.  Exists for
+ * 16-bit types with a z gate, dstate 64, headdim % 64 == 0, chunk_size % 32 == 0 and 16-byte aligned operands with
+ * strides that are multiples of 8 elements; BIMAMBA2_EUNSUPPORTED otherwise (bimamba2_bwd then runs the two).  Replaces
+ * _chunk_scan_bwd_dz and _chunk_scan_bwd_dstates (src/ssd/bi/ssd_combined.py:381-392). */
+int bimamba2_chunk_scan_bwd_dz_dstates(const bimamba2_params *p);
 /* states_f/b, dstates_f/b (in place), cs [dfinal_f/b] -> dstates_f/b (gradient of each chunk state), ddA_chunk_f/b
  * [dinitial_f/b].  Replaces the two _state_passing_bwd calls (src/ssd/bi/ssd_state_passing.py:210-248). */
 int bimamba2_state_passing_bwd(const bimamba2_params *p);

@@ -77,6 +77,12 @@ def test_backward_stages(ops, shape, dtype):
     assert_close(dpf, prf.grad, dtype, "dprev_f", scaled=big)
     assert_close(dpb, prb.grad, dtype, "dprev_b", scaled=big)
 
+    # ---- the two stages above as one launch, where that kernel exists: the same bits
+    if dtype != torch.float32 and N == 64 and P % 64 == 0 and Q % 32 == 0:
+        dz1, dox1, dpf1, dpb1 = ops._chunk_scan_bwd_dz_dstates(d["z"], out_x, dout.cuda(), d["C"], csf, csb)
+        assert torch.equal(dz1, dz) and torch.equal(dox1, dout_x), "dz / dout_x of the merged launch"
+        assert torch.equal(dpf1, dpf) and torch.equal(dpb1, dpb), "dstates of the merged launch"
+
     # ---- adjoint of the two inter-chunk recurrences + gradient of the chunk totals   (a10)
     dSf, dSb, ddAcf, ddAcb = ops._state_passing_bwd(pf, pb, csf, csb, dpf, dpb)
     Sf, Sb, cf, cb_ = _leaf(sf), _leaf(sb), _leaf(csf), _leaf(csb)
@@ -143,3 +149,42 @@ def test_backward_stages(ops, shape, dtype):
     assert_close(ddt, dt_l.grad, dtype, "ddt", scaled=big)
     assert_close(dA, A_l.grad, dtype, "dA", scaled=big)
     assert_close(ddt_bias, bias_l.grad, dtype, "ddt_bias", scaled=big)
+
+
+# batch, seqlen, H, P, G, N, chunk, dtype: one K step, a last chunk of one position, two channel tiles, grouped heads, fp16
+MERGED = [
+    (2, 64, 2, 64, 1, 64, 32, torch.bfloat16),
+    (1, 257, 4, 64, 2, 64, 256, torch.bfloat16),
+    (1, 200, 2, 128, 2, 64, 96, torch.bfloat16),
+    (2, 300, 4, 64, 4, 64, 128, torch.float16),
+]
+
+
+@pytest.mark.parametrize("case", MERGED)
+def test_dz_and_dstates_in_one_launch(ops, case):
+    """bimamba2_chunk_scan_bwd_dz_dstates against the two separate entry points (themselves held to the oracle above), on
+    strided z / dout views as the layer passes them, and its refusal of what it does not cover."""
+    b, L, H, P, G, N, Q, dtype = case
+    gen = torch.Generator().manual_seed(5)
+    wide = torch.randn(b, L, 2 * H * P + 8, generator=gen).to(dtype).cuda()
+    z = wide[..., :H * P].view(b, L, H, P)                      # row stride 2 H P + 8: a slice of a wider projection
+    dout = wide[..., H * P + 8:].view(b, L, H, P)
+    out_x = torch.randn(b, L, H, P, generator=gen).to(dtype).cuda()
+    C = torch.randn(b, L, G, N, generator=gen).to(dtype).cuda()
+    dt = torch.rand(b, L, H, generator=gen).cuda() * 0.1
+    A = -torch.rand(H, generator=gen).cuda() - 0.5
+    csf, csb, _ = ops._chunk_cumsum_fwd(dt, A, Q)
+    dz, dox = ops._chunk_scan_bwd_dz(out_x, z, out_x, dout, Q)
+    dz1, dox1, dpf1, dpb1 = ops._chunk_scan_bwd_dz_dstates(z, out_x, dout, C, csf, csb)
+    if dtype == torch.bfloat16:
+        assert torch.equal(dz1, dz) and torch.equal(dox1, dox)
+    else:
+        # float16: the compiler rounds the products to 16 bits in one step in one kernel and in two in the other, which
+        # moves one value in 10 000 by one unit in the last place
+        for got, want in ((dz1, dz), (dox1, dox)):
+            torch.testing.assert_close(got.float(), want.float(), rtol=2.0 ** -10, atol=2.0 ** -24)
+            assert int((got != want).sum()) <= got.numel() // 2000
+    dpf, dpb = ops._chunk_scan_bwd_dstates(C, csf, csb, dox1)    # from the merged launch's own dout_x: the same bits
+    assert torch.equal(dpf1, dpf) and torch.equal(dpb1, dpb)
+    with pytest.raises(ValueError):                             # float32: the two separate kernels only (unsupported)
+        ops._chunk_scan_bwd_dz_dstates(z.float(), out_x.float(), dout.float(), C.float(), csf, csb)
