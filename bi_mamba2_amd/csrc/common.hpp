@@ -100,6 +100,9 @@ __device__ __forceinline__ void tile64_request(T *tile, const T *src, int64_t ro
 // ALL outstanding vector memory operations, which defeats prefetching through LDS.  These accessors hide the DS
 // instruction from it.  Protocol: raw_lds_read / raw_lds_write any number of times, then raw_lds_wait(), then
 // raw_lds_use(v) on every value read before its first use (the empty asm ties the value to the wait, in program order).
+// A value read this way must reach its raw_lds_use() under ONE name: a copy (`r = f`) made before the wait is the same
+// value to the compiler, the second raw_lds_use() then needs a register copy, and that copy may be placed in front of the
+// wait, where the register still holds what was there before the read.
 // With RAW = false they are ordinary accesses and the other two are no-ops.
 __device__ __forceinline__ unsigned lds_addr(const void *p) {
     return (unsigned)(size_t)(const __attribute__((address_space(3))) void *)p;

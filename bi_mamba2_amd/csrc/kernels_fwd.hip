@@ -447,8 +447,9 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
 // Order of a wave's vector memory operations: two loads for the weight tables, then per step dout, z, out_x (registers)
 // and its 8 rows of the C tile (direct to LDS); the stores of a step follow its loads by two steps.  Loads complete in
 // order among themselves, stores do not keep that order, so a wait counts the younger loads only.
+// UNI: forward direction only (single-direction comparator).
 // ---------------------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, bool UNI = false>
 __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void bwd_dz_dstates_kernel(const bimamba2_params p, int nc) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
@@ -483,7 +484,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
     {
         const int q = min((int)threadIdx.x, limit - 1);
         r_cf = raw_global_load_f32(p.cs_f + o + q);
-        r_cb = raw_global_load_f32(p.cs_b + o + q);
+        r_cb = raw_global_load_f32((UNI ? p.cs_f : p.cs_b) + o + q);     // (UNI: a second load all the same, the waits below count two)
     }
     f32x4 rd[2], rz[2], ro[2];                               // two steps in flight
     auto issue = [&](auto S) {
@@ -502,7 +503,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
     {
         const int q = threadIdx.x;
         raw_lds_write_at<0>(wf_a + q * 4, q < limit ? __expf(r_cf) : 0.f);
-        raw_lds_write_at<0>(wb_a + q * 4, q < limit ? __expf(r_cb) : 0.f);
+        if (!UNI) raw_lds_write_at<0>(wb_a + q * 4, q < limit ? __expf(r_cb) : 0.f);
         raw_lds_wait();
     }
     const int kk = 8 * lg + (lr >> 2), nn = 4 * (lr & 3);
@@ -546,12 +547,14 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
         }
         i16x4 alo = raw_lds_tr16_read_at<XO>(xa_lo), ahi = raw_lds_tr16_read_at<XO>(xa_hi);
         f32x4 f0 = raw_lds_read_at<f32x4, WO>(wfl), f1 = raw_lds_read_at<f32x4, WO + 16>(wfl);
-        f32x4 r0 = raw_lds_read_at<f32x4, WO>(wbl), r1 = raw_lds_read_at<f32x4, WO + 16>(wbl);
+        f32x4 r0 = {0.f, 0.f, 0.f, 0.f}, r1 = {0.f, 0.f, 0.f, 0.f};
+        if (!UNI) { r0 = raw_lds_read_at<f32x4, WO>(wbl); r1 = raw_lds_read_at<f32x4, WO + 16>(wbl); }
         i16x4 blo[4], bhi[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) { blo[j] = raw_lds_tr16_read_at<BO>(ba_lo[j]); bhi[j] = raw_lds_tr16_read_at<BO>(ba_hi[j]); }
         raw_lds_wait();
-        raw_lds_use(alo); raw_lds_use(ahi); raw_lds_use(f0); raw_lds_use(f1); raw_lds_use(r0); raw_lds_use(r1);
+        raw_lds_use(alo); raw_lds_use(ahi); raw_lds_use(f0); raw_lds_use(f1);
+        if (!UNI) { raw_lds_use(r0); raw_lds_use(r1); }
         const Frag a = __builtin_bit_cast(Frag, __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7));
         float vf[8], vb[8];
 #pragma unroll
@@ -566,7 +569,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
             raw_lds_use(blo[j]); raw_lds_use(bhi[j]);
             const Frag bfr = __builtin_bit_cast(Frag, __builtin_shufflevector(blo[j], bhi[j], 0, 1, 2, 3, 4, 5, 6, 7));
             accf[j] = M::mma(af, bfr, accf[j]);
-            accb[j] = M::mma(ab, bfr, accb[j]);
+            if (!UNI) accb[j] = M::mma(ab, bfr, accb[j]);
         }
     };
     static_assert(BIMAMBA2_MAX_CHUNK == 256, "eight K steps of 32 positions");
@@ -579,14 +582,14 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
     if (nsteps > 6) kstep(std::integral_constant<int, 6>());
     if (nsteps > 7) kstep(std::integral_constant<int, 7>());
     float *of = p.dstates_f + (int64_t)blockIdx.z * P * N;
-    float *obk = p.dstates_b + (int64_t)blockIdx.z * P * N;
+    float *obk = (UNI ? p.dstates_f : p.dstates_b) + (int64_t)blockIdx.z * P * N;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int pp = pt * 64 + wave * 16 + lg * 4 + i, n = j * 16 + lr;
             of[(int64_t)pp * N + n] = accf[j][i];
-            obk[(int64_t)pp * N + n] = accb[j][i];
+            if (!UNI) obk[(int64_t)pp * N + n] = accb[j][i];
         }
 }
 
@@ -745,7 +748,7 @@ bool chunk_state_does_cumsum(const bimamba2_params *p) {
 bool bwd_dz_dstates_fused(const bimamba2_params *p) {
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
-    return p->has_z && !p->causal && p->dtype != BIMAMBA2_F32 && p->headdim % 64 == 0 && p->dstate == 64 && p->chunk_size % 32 == 0 &&
+    return p->has_z && p->dtype != BIMAMBA2_F32 && p->headdim % 64 == 0 && p->dstate == 64 && p->chunk_size % 32 == 0 &&
            al(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg) && al(p->z) && mult(p->z_sb, p->z_sl, p->z_sh) && al(p->dout) &&
            mult(p->dout_sb, p->dout_sl, p->dout_sh) && al(p->out_x) && al(p->dz) && al(p->dout_x);
 }
@@ -754,8 +757,13 @@ int launch_bwd_dz_dstates(const bimamba2_params *p) {
     if (!bwd_dz_dstates_fused(p)) return BIMAMBA2_EUNSUPPORTED;
     const int nc = nchunks(p);
     dim3 grid(1, p->headdim / 64, p->batch * nc * p->nheads);
-    if (p->dtype == BIMAMBA2_BF16) hipLaunchKernelGGL(bwd_dz_dstates_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
-    else hipLaunchKernelGGL(bwd_dz_dstates_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    if (p->causal) {
+        if (p->dtype == BIMAMBA2_BF16) hipLaunchKernelGGL((bwd_dz_dstates_kernel<bf16_t, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+        else hipLaunchKernelGGL((bwd_dz_dstates_kernel<f16_t, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    } else {
+        if (p->dtype == BIMAMBA2_BF16) hipLaunchKernelGGL((bwd_dz_dstates_kernel<bf16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+        else hipLaunchKernelGGL((bwd_dz_dstates_kernel<f16_t>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+    }
     return check_launch();
 }
 
