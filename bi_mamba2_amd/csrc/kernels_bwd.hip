@@ -1888,15 +1888,17 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
                 for (int j = 0; j < 4; ++j) acc[j] = M::mma(af, M::load(kT + xt_index<T, LDX>(j * 16 + lr, s * KSTEP + lg * KPL)), acc[j]);
             }
         }
-        float4 sw[NIT][HSL][2];
+        float4 sw[NIT][HSL][2] = {};
+        if (nslices > HSL) {                        // (with one half's worth of slices there is nothing more to wait for)
 #pragma unroll
-        for (int it = 0; it < NIT; ++it)
+            for (int it = 0; it < NIT; ++it)
 #pragma unroll
-            for (int sl = 0; sl < HSL; ++sl) {
-                const float *q = res + oa[it] + (int64_t)min(HSL + sl, nslices - 1) * slice;
-                sw[it][sl][0] = *reinterpret_cast<const float4 *>(q);
-                sw[it][sl][1] = *reinterpret_cast<const float4 *>(q + 4);
-            }
+                for (int sl = 0; sl < HSL; ++sl) {
+                    const float *q = res + oa[it] + (int64_t)min(HSL + sl, nslices - 1) * slice;
+                    sw[it][sl][0] = *reinterpret_cast<const float4 *>(q);
+                    sw[it][sl][1] = *reinterpret_cast<const float4 *>(q + 4);
+                }
+        }
         if constexpr (SLIM) __syncthreads();       // every wave is done with the K operand, whose LDS the staging tile shares
 #pragma unroll
         for (int j = 0; j < 4; ++j)
