@@ -108,7 +108,8 @@ __device__ __forceinline__ const char *uniform_ptr(const void *ptr) {
 // UNI: the single-direction (causal) operator: the reverse direction's state product, the K steps on the far side of the
 // diagonal and the far half of the diagonal step are left out.
 // hpw: heads per workgroup (divides nheads / ngroups, <= S16_MAX_HEADS); blockIdx.x = ((pt * nslices + slice) * nbc + bc).
-template <typename T, bool BWD, bool UNI>
+// DCOLS (mirror): dD per (head, headdim column); else one value per head.
+template <typename T, bool BWD, bool UNI, bool DCOLS = false>
 __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba2_params p, int nc, int npt, int hpw) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
@@ -506,7 +507,8 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         else wait_vmcnt<4>();
         // ---- epilogue.  acc[2t][i], acc[2t+1][i] = row wr0 + lr, headdim columns p0 + 32 t + 8 lg + i, + 4 + i ----
         f32x4 res_a[2], res_b[2];                  // packed results of the two column halves: out / dx, and out_x
-        float rsum = 0.f;
+        float rsum = 0.f, dsum = 0.f;
+        constexpr bool d_cols = DCOLS;             // mirror: dD per (head, column), else one value per head
         const bool live = r_own < limit;
         if (active) {
             const bool need_d = p.has_D;
@@ -560,8 +562,10 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                         float dxv = a[e] * dtr;
                         if (need_d) dxv = __builtin_fmaf(dcol[e], yv, dxv);
                         ov.v[e] = from_f<T>(dxv);
-                        // dD: kept in the accumulator's place (it is dead from here on); rows behind the end count nothing
-                        acc[2 * t + (e >> 2)][e & 3] = live ? yv * xv : 0.f;
+                        // dD: per headdim column kept in the accumulator's place (it is dead from here on; rows behind the end
+                        // count nothing); one value per head: a running sum
+                        if (d_cols) acc[2 * t + (e >> 2)][e & 3] = live ? yv * xv : 0.f;
+                        else dsum = __builtin_fmaf(yv, xv, dsum);
                     }
                     res_a[t] = __builtin_bit_cast(f32x4, ov);
                 }
@@ -602,15 +606,25 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             }
         }
         if (BWD && p.has_D) {
-            // dD partial of this (b, c, h): column sums of dy * x over the rows; a lane holds columns s16_col(j, 4 lg + i) of
-            // row lr: add the 16 lanes of a row group, then the waves
-            const unsigned red_a = sb + S16_RED + (wave * 64 + 8 * lg) * 4;
-            static_for<0, 16>([&](auto JI) __attribute__((always_inline)) {
-                constexpr int j = decltype(JI)::value >> 2, i = decltype(JI)::value & 3;
-                const float v = row16_sum(active ? acc[j][i] : 0.f);
-                if (lr == 0) raw_lds_write_at<s16_col(j, i) * 4>(red_a, v);   // s16_col(j, 4 lg + i) = s16_col(j, i) + 8 lg
-                return true;
-            });
+            if (d_cols) {
+                // dD partial of this (b, c, h): column sums of dy * x over the rows; a lane holds columns s16_col(j, 4 lg + i) of
+                // row lr: add the 16 lanes of a row group, then the waves
+                const unsigned red_a = sb + S16_RED + (wave * 64 + 8 * lg) * 4;
+                static_for<0, 16>([&](auto JI) __attribute__((always_inline)) {
+                    constexpr int j = decltype(JI)::value >> 2, i = decltype(JI)::value & 3;
+                    const float v = row16_sum(active ? acc[j][i] : 0.f);
+                    if (lr == 0) raw_lds_write_at<s16_col(j, i) * 4>(red_a, v);   // s16_col(j, 4 lg + i) = s16_col(j, i) + 8 lg
+                    return true;
+                });
+            } else {
+                // one value per head: the wave's sum of dy * x over its live rows
+                int ln = lane;
+                asm volatile("" : "+v"(ln));
+                float v = row16_sum((active && live) ? dsum : 0.f);
+                v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((ln ^ 16) << 2, __builtin_bit_cast(int, v)));
+                v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((ln ^ 32) << 2, __builtin_bit_cast(int, v)));
+                if (ln == 0) raw_lds_write_at<0>(sb + S16_RED + wave * 4, v);
+            }
         }
         // #2: everybody is done with this head's tiles, tables and z rows (a bare barrier: the stores just issued need not
         // have completed)
@@ -618,15 +632,25 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         raw_lds_barrier();
         if (BWD && p.has_D && threadIdx.x < 64) {
             float pv[S16_WAVES];
-            const unsigned red_a = sb + S16_RED + threadIdx.x * 4;
-            static_for<0, S16_WAVES>([&](auto WV) __attribute__((always_inline)) {
-                pv[decltype(WV)::value] = raw_lds_read_at<float, decltype(WV)::value * 256>(red_a);
-                return true;
-            });
+            // per column: the waves' sums of this thread's column; per head: the waves' sums, kept by thread 0 (the partial sums
+            // have the same layout either way, [(b, c)][h][P]: the other columns of the head then hold zeros)
+            const unsigned red_a = sb + S16_RED + (d_cols ? threadIdx.x * 4 : 0u);
+            if (d_cols) {
+                static_for<0, S16_WAVES>([&](auto WV) __attribute__((always_inline)) {
+                    pv[decltype(WV)::value] = raw_lds_read_at<float, decltype(WV)::value * 256>(red_a);
+                    return true;
+                });
+            } else {
+                static_for<0, S16_WAVES>([&](auto WV) __attribute__((always_inline)) {
+                    pv[decltype(WV)::value] = raw_lds_read_at<float, decltype(WV)::value * 4>(red_a);
+                    return true;
+                });
+            }
             raw_lds_wait();
             float v = 0.f;
 #pragma unroll
             for (int wv = 0; wv < S16_WAVES; ++wv) { raw_lds_use(pv[wv]); v += pv[wv]; }
+            if (!d_cols && threadIdx.x != 0) v = 0.f;
             p.red[((int64_t)(b * nc + c) * H + h) * P + p0 + threadIdx.x] = v;   // partials [(b, c)][h][P]
         }
         // the fragment addresses move on to the other buffer
@@ -673,8 +697,13 @@ static int launch_scan16_t(const bimamba2_params *p, int nc) {
     const int npt = p->headdim / 64, hpw = scan16_heads_per_block(p, nc);
     dim3 grid(p->batch * nc * (p->nheads / hpw) * npt);
     hipStream_t s = reinterpret_cast<hipStream_t>(p->stream);
-    if (p->causal) hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, true>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
-    else hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, false>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
+    if (BWD && p->has_D && p->D_has_hdim) {
+        if (p->causal) hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, true, BWD>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
+        else hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, false, BWD>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
+    } else {
+        if (p->causal) hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, true>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
+        else hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, false>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
+    }
     return check_launch();
 }
 
