@@ -22,6 +22,7 @@ from ._lib import Params
 _DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
 _INF = float("inf")
 MAX_CHUNK_SIZE, MAX_HEADDIM = 256, 128     # BIMAMBA2_MAX_CHUNK, BIMAMBA2_MAX_HEADDIM of include/bimamba2.h
+MAX_DSTATE = 256                           # BIMAMBA2_MAX_DSTATE
 
 
 def _require_gpu(t, name):
@@ -768,7 +769,7 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
         dt: (batch, seqlen, nheads)
         A: (nheads)
         B: (batch, seqlen, ngroups, dstate)
-        C: (batch, seqlen, ngroups, dstate)
+        C: (batch, seqlen, ngroups, dstate)   (dstate above the kernels' 256: computed in pieces of the state dimension)
         chunk_size: int, at least 32 (above 256 the kernels use 256: the result does not depend on it)
         D: (nheads, headdim) or (nheads,)
         z: (batch, seqlen, nheads, headdim)
@@ -812,6 +813,35 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
         if not return_final_states:
             return res.reshape(x.shape)
         return (res[0].reshape(x.shape),) + tuple(t.reshape(batch, nheads, headdim, -1) for t in res[1:])
+    dstate = B.shape[-1]
+    if dstate > MAX_DSTATE:
+        # The state columns do not interact: SS(x) with (B, C) is the sum over pieces of the state dimension of SS(x) with
+        # that piece of B and of C.  Pieces of at most 256 columns (views: the kernels take strided B / C) go through the
+        # kernels without D and gate; the sum, the D term and the gate are differentiable torch glue in float32, and the
+        # final states of the pieces lie side by side.
+        # The pieces run in float32 whatever the inputs' type: their outputs are summed, and 16-bit pieces, each rounded on
+        # its own, would leave the sum several times the rounding error of the one pass the reference makes.
+        cuts = [(n0, min(n0 + MAX_DSTATE, dstate)) for n0 in range(0, dstate, MAX_DSTATE)]
+        piece = lambda t, n0, n1: t[..., n0:n1] if t is not None else None
+        x32, B32, C32 = x.float(), B.float(), C.float()
+        y, fins = None, []
+        for n0, n1 in cuts:
+            r = bimamba_chunk_scan_combined(
+                x32, dt, A, piece(B32, n0, n1), piece(C32, n0, n1), chunk_size, dt_bias=dt_bias, dt_softplus=dt_softplus,
+                dt_limit=dt_limit, return_final_states=return_final_states,
+                initial_states_f=piece(initial_states_f, n0, n1), initial_states_b=piece(initial_states_b, n0, n1), seq_idx=seq_idx)
+            if return_final_states:
+                fins.append(r[1:])
+                r = r[0]
+            y = r if y is None else y + r
+        if D is not None:
+            y = y + x32 * (D.float() if D.dim() == 2 else D.float()[:, None])
+        if z is not None:
+            y = y * torch.nn.functional.silu(z.float())
+        out = y.to(x.dtype)
+        if not return_final_states:
+            return out
+        return out, torch.cat([f[0] for f in fins], dim=-1), torch.cat([f[1] for f in fins], dim=-1)
     if grad_places is not None:
         return MambaChunkScanCombinedFn.apply(x, dt, A, B, C, chunk_size, D, z, dt_bias, dt_softplus, dt_limit,
                                               return_final_states, initial_states_f, initial_states_b, seq_idx, grad_places)

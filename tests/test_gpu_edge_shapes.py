@@ -45,14 +45,17 @@ WIDE = [
     (2, 100, 2, 256, 1, 16, 64, torch.float32, True, True, False),       # heads of 256 channels: two pieces of 128
     (1, 300, 4, 192, 2, 64, 128, torch.bfloat16, False, False, True),    # 192 channels: two pieces of 96; final states
     (1, 700, 2, 64, 1, 32, 512, torch.float32, True, False, False),      # chunk_size above the kernels' 256
+    (1, 200, 2, 32, 1, 320, 64, torch.float32, True, False, True),       # dstate above the kernels' 256: pieces of 256 + 64
+    (1, 300, 4, 64, 2, 384, 128, torch.bfloat16, True, True, False),     # the same in bf16: 256 + 128
 ]
 
 
 @pytest.mark.parametrize("case", WIDE)
 def test_heads_wider_and_chunks_longer_than_the_kernels(case):
-    """Shapes the reference accepts beyond the kernels' limits (headdim > 128, chunk_size > 256): the public function
-    splits wide heads into narrower ones that share dt, A, dt_bias (and D) and caps the chunk size (the result does not
-    depend on it); output, final states and every gradient against the oracle at the shape the caller gave."""
+    """Shapes the reference accepts beyond the kernels' limits (headdim > 128, chunk_size > 256, dstate > 256): the public
+    function splits wide heads into narrower ones that share dt, A, dt_bias (and D), caps the chunk size (the result does
+    not depend on it) and sums over pieces of a wide state dimension; output, final states and every gradient against the
+    oracle at the shape the caller gave."""
     from bi_mamba2_amd import ops
     b, L, H, P, G, N, Q, dtype, z, Dhp, fin = case
     inp = make_case(b, L, H, P, G, N, dtype, with_z=z, D_has_hdim=Dhp)
