@@ -214,7 +214,7 @@ class BiMamba2(nn.Module):
         # back and applies the activation, modules.py:162-164 there); self.conv1d only holds the parameters
         xBC = conv1d_silu_fn(xBC, conv_w, conv_b, dx_place=dxbc_place)
         kw = {} if tuple(self.dt_limit) == (0.0, float("inf")) else {"dt_limit": tuple(self.dt_limit)}
-        if torch.is_grad_enabled() and xBC.requires_grad and self.headdim <= 128:
+        if torch.is_grad_enabled() and xBC.requires_grad and self.headdim <= 128 and self.d_state <= 256:
             # likewise the operator's dx, dB, dC: slices of the gradient of the convolution's output
             g2 = _GradPieces(xBC, [self.d_inner, bc, bc])
             x, B, C = _SplitInto.apply(xBC, g2)

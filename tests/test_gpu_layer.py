@@ -72,6 +72,26 @@ def test_bimamba2_layer_forward_backward():
     assert _GradPieces.copies_log[-2:] == [(), (2,)]
 
 
+def test_bimamba2_layer_with_a_state_wider_than_the_kernels():
+    """d_state 320: the operator sums over pieces of the state dimension, and the layer lets autograd put the gradients
+    of x, B, C together (the in-place route is for what the kernels take in one piece)."""
+    from bi_mamba2_amd.modules import BiMamba2
+    torch.manual_seed(3)
+    m = BiMamba2(d_model=32, d_state=320, headdim=32, ngroups=1, chunk_size=64).cuda()
+    with torch.no_grad():
+        m.A_log.copy_(torch.log(torch.rand(m.nheads) * 4 + 0.5))
+    u = torch.randn(1, 150, 32, device="cuda", requires_grad=True)
+    dy = torch.randn(1, 150, 32, generator=torch.Generator().manual_seed(1)).cuda()
+    out = m(u)
+    out.backward(dy)
+    ref, du_ref, dp_ref = _reference_grads(m, u, dy, chunked=False)
+    assert_close(out, ref, torch.float32, "layer output")
+    assert_close(u.grad, du_ref, torch.float32, "layer du")
+    for name, p in m.named_parameters():
+        if name not in UNUSED:
+            assert_close(p.grad, dp_ref[name], torch.float32, "layer d" + name)
+
+
 def test_bimamba2_layer_without_input_gradient_and_twice():
     """Frozen input (only the parameters take gradients) and two backward passes through two forwards that share the
     layer: the buffer of the split's gradients belongs to one forward call."""
