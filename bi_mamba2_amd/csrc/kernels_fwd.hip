@@ -216,8 +216,23 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     __shared__ __attribute__((aligned(16))) float wf[BIMAMBA2_MAX_CHUNK], wb[BIMAMBA2_MAX_CHUNK];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lr = lane & 15, lg = lane >> 4;
-    const int nt = blockIdx.x, pt = blockIdx.y;
-    const int h = blockIdx.z % p.nheads, bc = blockIdx.z / p.nheads, c = bc % nc, b = bc / nc;
+    // Workgroups are dealt to the chip's eight dies in launch order, one after the other, and each die has its own L2.  With
+    // several tiles per (b, c, h) - which all read the same x rows - the launch order is remapped so that the tiles of one
+    // (b, c, h) are eight workgroups apart, i.e. on the same die: groups of eight (b, c, h), tile by tile.
+    int nt = blockIdx.x, pt = blockIdx.y, bch = blockIdx.z;
+    {
+        const int tiles = gridDim.x * gridDim.y, nbch = gridDim.z;
+        if (tiles > 1) {
+            const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+            const int full = nbch / 8, grp = lin / (8 * tiles);
+            int tile;
+            if (grp < full) { const int r = lin - grp * 8 * tiles; tile = r / 8; bch = grp * 8 + r % 8; }
+            else { const int m = nbch - full * 8, r = lin - full * 8 * tiles; tile = r / m; bch = full * 8 + r % m; }
+            nt = tile % (int)gridDim.x;
+            pt = tile / (int)gridDim.x;
+        }
+    }
+    const int h = bch % p.nheads, bc = bch / p.nheads, c = bc % nc, b = bc / nc;
     const int g = h / (p.nheads / p.ngroups);
     const int Q = p.chunk_size, N = p.dstate, P = p.headdim;
     const int limit = min(Q, p.seqlen - c * Q);
@@ -413,8 +428,8 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     if (nsteps > 5) kstep(std::integral_constant<int, 5>());
     if (nsteps > 6) kstep(std::integral_constant<int, 6>());
     if (nsteps > 7) kstep(std::integral_constant<int, 7>());
-    float *of = (DSTATES ? p.dstates_f : p.states_f) + (int64_t)blockIdx.z * P * N;
-    float *ob = (DSTATES ? p.dstates_b : p.states_b) + (int64_t)blockIdx.z * P * N;
+    float *of = (DSTATES ? p.dstates_f : p.states_f) + (int64_t)bch * P * N;
+    float *ob = (DSTATES ? p.dstates_b : p.states_b) + (int64_t)bch * P * N;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
