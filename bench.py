@@ -36,10 +36,12 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def stage_table(w, e, fused=(False, False, False), copies=False):
+def stage_table(w, e, fused=(False, False, False), copies=False, heads_per_wg=(1, 1)):
     """Algorithmic flops and bytes per launch of every stage kernel (e = bytes per element of x/B/C/z).
     fused[0] / [1] / [2]: the forward scan / the dx kernel / the dCB kernel rebuilds its CB tiles from C and B instead of
-    reading them.  copies: the states entering the chunks (and their gradients) are kept in e-byte copies."""
+    reading them.  copies: the states entering the chunks (and their gradients) are kept in e-byte copies.
+    heads_per_wg: heads of a group that one workgroup of the forward scan / the dx kernel works through with ONE rebuilt
+    C.B^T (the flops of the rebuild are counted once per workgroup, which is what the kernel executes)."""
     B, L, H, P, G, N, Q = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate", "chunk_size"))
     nc = (L + Q - 1) // Q
     u, ug = B * nc * H, B * nc * G                 # (b, c, h) and (b, c, g) units
@@ -47,7 +49,8 @@ def stage_table(w, e, fused=(False, False, False), copies=False):
     st = 4 * B * nc * H * P * N                     # one float32 state tensor
     se = (e if copies else 4) * B * nc * H * P * N  # one tensor of entering states as the kernels read it
     cb = 4 * ug * Q * Q
-    scan_cb = [(u * 2 * Q * Q * N, e * T2) if f else (0, cb) for f in fused]   # (extra flops, bytes) for the CB tiles
+    hw = tuple(heads_per_wg) + (1,)
+    scan_cb = [((u // hw[i]) * 2 * Q * Q * N, e * T2) if f else (0, cb) for i, f in enumerate(fused)]   # (extra flops, bytes) for the CB tiles
     return {
         # entry point: (flops, bytes)
         "bimamba2_chunk_cumsum_fwd": (0, 4 * B * L * H + 3 * 4 * T1),
@@ -157,10 +160,13 @@ def conv_line(w, dtype, dev, reps):
             "torch_conv1d_fwd_bwd_us": round(t_t, 2)}
 
 
-def whole_op_bytes(w, e, has_z):
+def whole_op_bytes(w, e, has_z, training=True):
+    """Algorithmic HBM bytes of the operator: inputs read once, outputs written once.  A forward pass that a backward
+    pass follows (training) also writes the pre-gate output when there is a z gate; a forward pass on its own
+    (torch.no_grad(): the scan kernel skips that store) does not."""
     B, L, H, P, G, N = (w[k] for k in ("batch", "seqlen", "nheads", "headdim", "ngroups", "dstate"))
     T4, T2, T1 = B * L * H * P, B * L * G * N, B * L * H
-    fwd = e * T4 * (2 + (2 if has_z else 0)) + 2 * e * T2 + 4 * T1
+    fwd = e * T4 * (2 + ((2 if training else 1) if has_z else 0)) + 2 * e * T2 + 4 * T1
     bwd = e * T4 * (3 + (3 if has_z else 0)) + 4 * e * T2 + 8 * T1
     return fwd, bwd
 
@@ -310,13 +316,54 @@ def config_line(name, dev, steps, warmup, spin=False):
     for _ in range(warmup):
         replay()
     t = timed(replay, steps)
-    fwd_b, bwd_b = whole_op_bytes(w, e, has_z)
+    fwd_b, bwd_b = whole_op_bytes(w, e, has_z, training=bwd)
     nbytes = fwd_b + (bwd_b if bwd else 0)
     tokens = w["batch"] * w["seqlen"]
     return {"workload": {**w, "has_z": has_z, "dtype": "bf16"}, "pass": "fwd+bwd" if bwd else "fwd",
             "ms": round(t * 1e3, 4), "Mtokens_s": round(tokens / t / 1e6, 2), "alg_MB": round(nbytes / 1e6, 1),
             "hbm_roofline_us": round(nbytes / (HBM_PEAK_GBS * 1e9) * 1e6, 1),
             "hbm_frac": round(nbytes / t / (HBM_PEAK_GBS * 1e9), 4)}
+
+
+def ref_shape_line(dev, steps, warmup):
+    """The one shape the reference publishes timings for (benchmark/benchmark_fwd_all.py:9-26 and benchmark_bwd_all.py:9-28
+    there): batch 2, 4 heads x headdim 16, 4 groups, dstate 16, chunk 128, float32, z gate, D (nheads, headdim), dt_bias +
+    softplus, seqlen 2048 and 8192.  Timed the way those scripts time it: the private forward and the private backward
+    function called directly (no autograd), eager launches, mean over `steps` calls; and the same calls replayed from a
+    HIP graph.  This leg runs the float32 generic kernels, which no other leg times.  A is drawn negative as in the
+    other legs (the scripts draw it from N(0, 1))."""
+    import torch
+    from bi_mamba2_amd import ops
+    res = {"workload": "batch 2 x 4 heads x headdim 16, 4 groups, dstate 16, chunk 128, float32, z gate, D (nheads, headdim), "
+                       "dt_bias + softplus; private forward / backward functions as the reference's benchmark scripts call them",
+           "published_ms_other_hardware": {"fwd_L2048": 0.20, "fwd_L8192": 0.82, "bwd_L4096": 0.97, "bwd_L8192": 2.2,
+                                           "source": "plots of the reference (RTX 4060 Ti), read off to about 5 %"}}
+    for L in (2048, 8192):
+        w = dict(batch=2, seqlen=L, nheads=4, headdim=16, ngroups=4, dstate=16, chunk_size=128)
+        inp = make_inputs(w["batch"], L, 4, 16, 4, 16, torch.float32, True)
+        t = {k: v.to(dev) for k, v in inp.items()}
+        D = torch.randn(4, 16, generator=torch.Generator().manual_seed(3)).to(dev)
+        dout = torch.rand(inp["x"].shape, generator=torch.Generator().manual_seed(1)).to(dev)
+        kw = dict(D=D, z=t["z"], dt_bias=t["dt_bias"], dt_softplus=True)
+
+        def fwd():
+            return ops._mamba_chunk_scan_combined_fwd(t["x"], t["dt"], t["A"], t["B"], t["C"], 128, return_intermediates=False,
+                                                      want_final=False, **kw)
+        out_x = fwd()[1]
+
+        def bwd():
+            ops._mamba_chunk_scan_combined_bwd(dout, t["x"], t["dt"], t["A"], t["B"], t["C"], out_x, 128, **kw)
+        line = {}
+        for name, fn in (("fwd", fwd), ("bwd", bwd)):
+            for _ in range(warmup):
+                fn()
+            line[name + "_eager_ms"] = round(timed(fn, steps) * 1e3, 4)
+            replay = graphed(fn)
+            for _ in range(warmup):
+                replay()
+            line[name + "_graph_ms"] = round(timed(replay, steps) * 1e3, 4)
+        res[f"L{L}"] = line
+    return res
 
 
 def layer_line(dev, steps, warmup, spin=False):
@@ -392,7 +439,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the causal comparator, the other configurations and the layer's legs (keeps a profile of the run to "
                          "the operator)")
-    ap.add_argument("--config", choices=["target"] + sorted(OTHER_CONFIGS) + ["layer_config4"], default="target",
+    ap.add_argument("--config", choices=["target"] + sorted(OTHER_CONFIGS) + ["layer_config4", "ref_published_shape"], default="target",
                     help="target (default): the headline workload with every leg; another name: only that configuration's leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -407,8 +454,12 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.config != "target":
-        line = (layer_line(dev, args.steps, args.warmup, spin=True) if args.config == "layer_config4"
-                else config_line(args.config, dev, args.steps, args.warmup, spin=True))
+        if args.config == "layer_config4":
+            line = layer_line(dev, args.steps, args.warmup, spin=True)
+        elif args.config == "ref_published_shape":
+            line = ref_shape_line(dev, args.steps, args.warmup)
+        else:
+            line = config_line(args.config, dev, args.steps, args.warmup, spin=True)
         print(json.dumps({args.config: line}))
         return
     w = WORKLOAD
@@ -469,6 +520,7 @@ def main():
         causal_fn = causal_step if args.eager else graphed(causal_step)
     tokens = w["batch"] * w["seqlen"]
     fwd_b, bwd_b = whole_op_bytes(w, e, has_z)
+    fwd_only_b = whole_op_bytes(w, e, has_z, training=False)[0]     # the forward-only leg runs under torch.no_grad()
 
     extras = {}
     if not args.no_extras:
@@ -476,6 +528,7 @@ def main():
         extras["conv1d_silu"] = conv_line(w, dtype, dev, max(10, args.steps))
         extras["configs"] = {name: config_line(name, dev, max(30, args.steps), 10) for name in OTHER_CONFIGS}
         extras["layer_config4"] = layer_line(dev, max(30, args.steps), 10)
+        extras["ref_published_shape"] = ref_shape_line(dev, max(30, args.steps), 10)
     # ---- the operator's own legs, the reported step last
     for _ in range(args.warmup):
         fwd_fn()
@@ -536,7 +589,8 @@ def main():
     if copies:
         for f in ("states16_f", "states16_b", "dstates16_f", "dstates16_b"):
             c.new(f, sts, dtype)
-    table = stage_table(w, e, fused=tuple(r == 0 for r in reads_cb), copies=copies)
+    hpw = tuple(int(_lib.load().bimamba2_chunk_scan_heads_per_workgroup(ctypes.byref(c.p), d)) for d in (0, 1))
+    table = stage_table(w, e, fused=tuple(r == 0 for r in reads_cb), copies=copies, heads_per_wg=hpw)
     if not any(reads_cb):
         del table["bimamba2_bmm_chunk_fwd"]     # not launched by the composites for this problem
     if _lib.load().bimamba2_chunk_scan_reads_cb(ctypes.byref(c.p), 3) == 0:
@@ -623,7 +677,8 @@ def main():
         "whole_op": {"fwd_ms": t_fwd * 1e3, "fwd_Mtokens_s": tokens / t_fwd / 1e6,
                      "fwd_bwd_alg_MB": (fwd_b + bwd_b) / 1e6,
                      "fwd_bwd_hbm_frac": (fwd_b + bwd_b) / t_step / (HBM_PEAK_GBS * 1e9),
-                     "fwd_hbm_frac": fwd_b / t_fwd / (HBM_PEAK_GBS * 1e9),
+                     "fwd_alg_MB": fwd_only_b / 1e6,
+                     "fwd_hbm_frac": fwd_only_b / t_fwd / (HBM_PEAK_GBS * 1e9),
                      "sum_kernel_us": round(sum(k["us"] for k in kernels.values()), 1),
                      "measured_copy_GBs": round(copy_gbs, 1)},
         "kernels": kernels,

@@ -49,7 +49,8 @@ ENTRY_POINTS = (
 NORM_ENTRY_POINTS = ("bimamba2_rmsnorm_gated_fwd", "bimamba2_rmsnorm_gated_bwd")
 CONV_ENTRY_POINTS = ("bimamba2_conv1d_silu_fwd", "bimamba2_conv1d_silu_bwd")
 ALL_SYMBOLS = ENTRY_POINTS + ("bimamba2_strerror", "bimamba2_version", "bimamba2_params_size",
-                              "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb", "bimamba2_state_copies", "bimamba2_norm_params_size",
+                              "bimamba2_workspace_bytes", "bimamba2_chunk_scan_reads_cb", "bimamba2_state_copies",
+                              "bimamba2_chunk_scan_heads_per_workgroup", "bimamba2_ddt_direct_planes", "bimamba2_norm_params_size",
                               "bimamba2_rmsnorm_gated_workspace_bytes", "bimamba2_conv_params_size",
                               "bimamba2_conv1d_silu_workspace_bytes", "bimamba2_cast_params_size",
                               "bimamba2_cast_many") + NORM_ENTRY_POINTS + CONV_ENTRY_POINTS
@@ -111,6 +112,10 @@ def load():
     lib.bimamba2_version.restype = ctypes.c_int
     lib.bimamba2_chunk_scan_reads_cb.argtypes = [ctypes.POINTER(Params), ctypes.c_int]
     lib.bimamba2_chunk_scan_reads_cb.restype = ctypes.c_int
+    lib.bimamba2_chunk_scan_heads_per_workgroup.argtypes = [ctypes.POINTER(Params), ctypes.c_int]
+    lib.bimamba2_chunk_scan_heads_per_workgroup.restype = ctypes.c_int
+    lib.bimamba2_ddt_direct_planes.argtypes = [ctypes.POINTER(Params)]
+    lib.bimamba2_ddt_direct_planes.restype = ctypes.c_int
     lib.bimamba2_state_copies.argtypes = [ctypes.POINTER(Params)]
     lib.bimamba2_state_copies.restype = ctypes.c_int
     lib.bimamba2_params_size.restype = ctypes.c_size_t

@@ -100,7 +100,7 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
         need_f(q->dstates_b, stn);
         if (q->has_z && !q->dout_x)
             q->dout_x = cv.take<char>((size_t)q->batch * q->seqlen * q->nheads * q->headdim * elem_size(q->dtype));
-        need_f(q->ddt_direct, bhcq);
+        need_f(q->ddt_direct, bhcq * ddt_direct_planes(*q));
         need_f(q->u_f, bhcq);
         need_f(q->u_b, bhcq);
         need_f(q->v_f, bhcq);
@@ -186,6 +186,16 @@ int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which) {
     return scan_recomputes_cb(p, which != 0) ? 0 : 1;
 }
 
+int bimamba2_chunk_scan_heads_per_workgroup(const bimamba2_params *p, int bwd) {
+    if (check_problem(p)) return 1;
+    return chunk_scan_uses_scan16(p, bwd != 0) ? chunk_scan16_heads_per_workgroup(p) : 1;
+}
+
+int bimamba2_ddt_direct_planes(const bimamba2_params *p) {
+    if (check_problem(p)) return 1;
+    return ddt_direct_planes(*p);
+}
+
 int bimamba2_chunk_cumsum_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->dt); REQUIRE(p->A); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
@@ -262,8 +272,6 @@ int bimamba2_chunk_scan_bwd_dx(const bimamba2_params *p) {
     if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
     if (p->has_D) { REQUIRE(p->D); REQUIRE(p->dD); REQUIRE(p->red); }
     const int nc = nchunks(p);
-    if (p->headdim > (p->dtype == BIMAMBA2_F32 ? 32 : 64))   // several headdim tiles add their row sums atomically
-        TRY(launch_fill(p->ddt_direct, (size_t)p->batch * p->nheads * nc * p->chunk_size, 0.f, stream_of(p)));
     TRY(launch_chunk_scan(p, true));
     if (p->has_D) {
         if (p->D_has_hdim) return launch_reduce(p->red, p->dD, p->batch * nc, p->nheads * p->headdim, 1, stream_of(p));
@@ -402,8 +410,6 @@ int bimamba2_bwd(const bimamba2_params *p) {
         REQUIRE(qx.dx); REQUIRE(qx.ddt_direct);
         if (qx.has_D) { REQUIRE(qx.D); REQUIRE(qx.dD); }
         const int nc = nchunks(&q);
-        if (q.headdim > (q.dtype == BIMAMBA2_F32 ? 32 : 64))
-            TRY(launch_fill(q.ddt_direct, (size_t)q.batch * q.nheads * nc * q.chunk_size, 0.f, stream_of(&q)));
         TRY(launch_chunk_scan(&qx, true));
         if (q.has_D) {
             if (q.D_has_hdim) jobs.job[jobs.n++] = ReduceJob{q.red, q.dD, q.batch * nc, q.nheads * q.headdim, 1};

@@ -1961,7 +1961,8 @@ __device__ __forceinline__ void bmm_chunk_bwd_body(const bimamba2_params &p, int
 #pragma unroll
         for (int i = 0; i < 4; ++i) stg[(wave * 16 + lg * 4 + i) * SLD + j * 16 + lr] = acc[j][i];
     __syncthreads();
-    const bool ovec = N % VS == 0 && o_sl % VS == 0 && o_sb % VS == 0;
+    // (16-byte stores: the strides and the base of the destination slice must both allow them)
+    const bool ovec = N % VS == 0 && o_sl % VS == 0 && o_sb % VS == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
     for (int id = threadIdx.x; id < 64 * (64 / VS); id += NTHREADS) {
         const int rl = id / (64 / VS), cc = (id % (64 / VS)) * VS;
         const int r = r0 + rl, n = nt * 64 + cc;
@@ -2049,6 +2050,8 @@ __device__ __forceinline__ void chunk_cumsum_bwd_body(const bimamba2_params &p, 
     // Every load of the kernel goes out here, unconditionally and from clamped (valid) addresses, before anything is
     // used: a load that is waited for costs microseconds, and conditional loads get serialised by the compiler.
     float vf[4], vb[4], uf[4], ub[4], di[4], dtr[4], ddr[4];
+    const int nplanes = ddt_direct_planes(p);
+    const int64_t plane = (int64_t)p.batch * H * nc * Q;
     const DT *dt = reinterpret_cast<const DT *>(p.dt) + b * p.dt_sb + (int64_t)c * Q * p.dt_sl + h * p.dt_sh;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -2058,6 +2061,7 @@ __device__ __forceinline__ void chunk_cumsum_bwd_body(const bimamba2_params &p, 
         uf[e] = p.u_f[o + qc];
         ub[e] = p.u_b[o + qc];
         ddr[e] = p.ddt_direct[o + qc];
+        for (int pl = 1; pl < nplanes; ++pl) ddr[e] += p.ddt_direct[pl * plane + o + qc];    // one plane per headdim tile of the dx kernel
         dtr[e] = to_f(dt[(int64_t)qc * p.dt_sl]);
     }
     if (p.causal) {                   // single-direction operator: nothing wrote the reverse direction's terms

@@ -625,8 +625,8 @@ __global__ __launch_bounds__(SCAN_THREADS, 4) void chunk_scan_kernel(const bimam
 #pragma unroll
                 for (int d = 1; d < CPR; d <<= 1) rsum += __shfl_xor(rsum, d, 64);
                 if (id < 16 * CPR && r < limit && (id % CPR) == 0) {
-                    if (npt == 1) p.ddt_direct[o + r] = rsum;
-                    else atomicAdd(p.ddt_direct + o + r, rsum);   // several headdim tiles share a row
+                    // (several headdim tiles share a row: each writes the plane of its tile, the reader adds them)
+                    p.ddt_direct[(int64_t)pt * ((int64_t)p.batch * H * nc * Q) + o + r] = rsum;
                 }
             }
         }
@@ -664,8 +664,7 @@ static inline bool al16(const void *ptr) { return (reinterpret_cast<uintptr_t>(p
 
 static inline int scan_col_tile(const bimamba2_params *p) {
     // headdim tile: the widest the LDS image allows (64 columns for 16-bit types, 32 for float32)
-    const int njmax = p->dtype == BIMAMBA2_F32 ? 2 : 4;
-    return p->headdim <= 16 ? 16 : (p->headdim <= 32 || njmax == 2) ? 32 : 64;
+    return scan_col_tile_of(p->headdim, p->dtype);
 }
 
 // whether the kernels without guarded fallbacks apply (vs = elements per 16 bytes)
@@ -690,6 +689,10 @@ bool scan_recomputes_cb(const bimamba2_params *p, bool bwd) {
     return scan_fast(p, bwd, 64, 8) && al16(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al16(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg);
 }
 
+bool chunk_scan_uses_scan16(const bimamba2_params *p, bool bwd) {
+    return scan_recomputes_cb(p, bwd) && (p->headdim == 64 || p->headdim == 128) && p->dstate == 64;
+}
+
 template <typename T, int NJMAX, bool BWD>
 static int launch_scan_t(const bimamba2_params *p) {
     const int nc = nchunks(p);
@@ -710,13 +713,10 @@ static int launch_scan_t(const bimamba2_params *p) {
     const void *c16f = BWD ? p->dstates16_f : p->states16_f, *c16b = BWD ? p->dstates16_b : p->states16_b;
     if (c16f && (!al16(c16f) || !al16(c16b) || !(p->causal || c16b))) return BIMAMBA2_EINVAL;
     if constexpr (sizeof(T) == 2 && NJMAX == 4) {
-#ifndef BM2_SCAN_V1
         // the shapes of the 16-bit kernel with transposed products and a raw operand tile: it needs the 16-bit copies of the
         // entering states (the composites keep them at these shapes) and no CB
-        if (c16f && (BWD ? p->CBT : p->CB) == nullptr && scan_recomputes_cb(p, BWD) && (P == 64 || P == 128) && N == 64 &&
-            (p->causal || c16b))
+        if (c16f && (BWD ? p->CBT : p->CB) == nullptr && chunk_scan_uses_scan16(p, BWD) && (p->causal || c16b))
             return launch_chunk_scan16(p, BWD);
-#endif
         if (p->causal) {                                // single-direction comparator: the fused kernels only
             if (!scan_recomputes_cb(p, BWD)) return BIMAMBA2_EUNSUPPORTED;
             if (qt == 1) hipLaunchKernelGGL((chunk_scan_kernel<T, 1, 4, BWD, true, 2, true>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);

@@ -599,9 +599,8 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 rsum += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((ln ^ 16) << 2, __builtin_bit_cast(int, rsum)));
                 rsum += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((ln ^ 32) << 2, __builtin_bit_cast(int, rsum)));
                 if (lg == 0 && live) {
-                    float *dst = p.ddt_direct + ((((int64_t)b * H + hh) * nc + c) * Q + r_lane);
-                    if (npt == 1) *dst = rsum;
-                    else atomicAdd(dst, rsum);   // several headdim tiles share a row
+                    // (several headdim tiles share a row: each writes the plane of its tile, the reader adds them)
+                    p.ddt_direct[(int64_t)pt * ((int64_t)p.batch * H * nc * Q) + ((((int64_t)b * H + hh) * nc + c) * Q + r_lane)] = rsum;
                 }
             }
         }
@@ -688,6 +687,10 @@ static int scan16_heads_per_block(const bimamba2_params *p, int nc) {
         if (k == 1 || cost <= best_cost) { best = k; best_cost = cost; }
     }
     return best;
+}
+
+int chunk_scan16_heads_per_workgroup(const bimamba2_params *p) {
+    return scan16_heads_per_block(p, (p->seqlen + p->chunk_size - 1) / p->chunk_size);
 }
 
 // Launches the kernel above; the caller (launch_chunk_scan) has checked that the problem is one of its shapes:

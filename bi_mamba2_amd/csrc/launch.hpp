@@ -8,6 +8,17 @@ namespace bm2 {
 
 static inline int check_launch() { return hipGetLastError() == hipSuccess ? BIMAMBA2_OK : BIMAMBA2_ELAUNCH; }
 
+// Width of the headdim column tile of the chunk-scan kernels (64 columns for 16-bit types, 32 for float32, less for narrow
+// heads), and with it the number of planes of ddt_direct: every column tile of the dx kernel writes the row sums of its own
+// columns to its own (batch, nheads, nchunks, chunk_size) plane, and the reader adds the planes in order (no atomics).
+__host__ __device__ inline int scan_col_tile_of(int headdim, int dtype) {
+    return headdim <= 16 ? 16 : (headdim <= 32 || dtype == BIMAMBA2_F32) ? 32 : 64;
+}
+__host__ __device__ inline int ddt_direct_planes(const bimamba2_params &p) {
+    const int pw = scan_col_tile_of(p.headdim, p.dtype);
+    return (p.headdim + pw - 1) / pw;
+}
+
 int launch_chunk_cumsum_fwd(const bimamba2_params *p);
 int launch_bmm_chunk_fwd(const bimamba2_params *p);
 int launch_chunk_state(const bimamba2_params *p, bool dstates, bool cumsum = false);   // cumsum: also does the chunk cumsum
@@ -16,6 +27,10 @@ int launch_state_passing_fwd(const bimamba2_params *p);
 int launch_chunk_scan(const bimamba2_params *p, bool bwd);
 // the 16-bit kernel of kernels_scan16.hip (launch_chunk_scan picks it where it applies)
 int launch_chunk_scan16(const bimamba2_params *p, bool bwd);
+// heads of one group that a workgroup of that kernel walks through (they share one C.B^T product)
+int chunk_scan16_heads_per_workgroup(const bimamba2_params *p);
+// whether launch_chunk_scan() would pick that kernel for this problem (the 16-bit copies of the entering states given)
+bool chunk_scan_uses_scan16(const bimamba2_params *p, bool bwd);
 // true when that launch recomputes CB (bwd: CB^T) from the C and B rows instead of reading it
 bool scan_recomputes_cb(const bimamba2_params *p, bool bwd);
 // true when the dCB launch can rebuild its CB tiles from the C and B rows (then CB may be NULL)

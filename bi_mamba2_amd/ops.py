@@ -392,12 +392,15 @@ def _chunk_scan_chunk_state_bwd_dx(x, dt, dA_cumsum_f, dA_cumsum_b, B, CB, dout,
     c.put("cs_f", dA_cumsum_f, torch.float32); c.put("cs_b", dA_cumsum_b, torch.float32)
     c.put("dstates_f", dstates_f, torch.float32); c.put("dstates_b", dstates_b, torch.float32)
     dx = c.put("dx", dx) if dx is not None else c.new("dx", x.shape, x.dtype)
-    ddt = c.new("ddt_direct", _bhcq(c))
+    # one plane per headdim column tile of the kernel, added up here in a fixed order
+    planes = int(_lib.load().bimamba2_ddt_direct_planes(c.p))
+    ddt = c.new("ddt_direct", (planes,) + _bhcq(c))
     dD = None
     if D is not None:
         dD = c.new("dD", tuple(D.shape))
         c.new("red", (batch * nchunks * nheads * headdim,))
     c.run("bimamba2_chunk_scan_bwd_dx")
+    ddt = ddt[0] if planes == 1 else ddt.sum(0)
     return dx, ddt, (dD.to(D.dtype) if dD is not None else None)
 
 
@@ -543,6 +546,42 @@ def _point_into(c, blob, offs, fields=_BLOB_FIELDS):
     for field, o in zip(fields, offs):
         setattr(c.p, field, base + 4 * o)
     c.keep.append(blob)
+
+
+# Sequence boundaries that one chunk may hold.  The kernels separate packed sequences by an offset of BIMAMBA2_SEQ_CUT (-20)
+# per boundary in the chunk's cumulative decay sums (include/bimamba2.h), whose float32 resolution therefore falls with
+# the number of boundaries inside ONE chunk: 1.2e-6 relative per boundary, i.e. 4e-5 at 32 - inside the float32 contract
+# of 1e-4 - and beyond it from about 40.  The result does not depend on the chunk size, so a call whose seq_idx puts more
+# boundaries than this into some chunk runs with a smaller chunk (a chunk of 32 positions cannot hold more than 32).
+MAX_SEQ_BOUNDARIES_PER_CHUNK = 32
+
+
+def seq_boundaries_per_chunk(seq_idx, chunk_size):
+    """Largest number of sequence boundaries that fall into one chunk of `chunk_size` positions, as the kernels count
+    them: a change of seq_idx between positions l - 1 and l offsets the forward sums of the chunk of l and the reverse
+    sums of the chunk of l - 1."""
+    change = seq_idx[:, 1:] != seq_idx[:, :-1]                      # (batch, L - 1): entry l - 1 is the boundary in front of l
+    if change.numel() == 0:
+        return 0
+    batch, n = change.shape
+    pos = torch.arange(1, n + 1, device=seq_idx.device)
+    nch = (n + 1 + chunk_size - 1) // chunk_size
+    ones = change.to(torch.int32)
+    fwd = torch.zeros(batch, nch, dtype=torch.int32, device=seq_idx.device).scatter_add_(1, (pos // chunk_size).expand(batch, n), ones)
+    rev = torch.zeros(batch, nch, dtype=torch.int32, device=seq_idx.device).scatter_add_(1, ((pos - 1) // chunk_size).expand(batch, n), ones)
+    return int(torch.maximum(fwd.max(), rev.max()).item())
+
+
+def chunk_size_for_seq_idx(seq_idx, chunk_size):
+    """The chunk size a call with this seq_idx runs with: `chunk_size` if no chunk holds more than
+    MAX_SEQ_BOUNDARIES_PER_CHUNK boundaries, else the largest of 128, 64, 32 below it for which that is true.  Costs one
+    device-to-host synchronisation (the count is taken on the device)."""
+    for q in [chunk_size] + [c for c in (128, 64, 32) if c < chunk_size]:
+        if seq_boundaries_per_chunk(seq_idx, q) <= MAX_SEQ_BOUNDARIES_PER_CHUNK:
+            return q
+    # (not reached with chunk sizes down to 32; kept so that a change of the limit cannot make the mechanism fail silently)
+    raise ValueError(f"seq_idx puts more than {MAX_SEQ_BOUNDARIES_PER_CHUNK} sequence boundaries into every chunk size down "
+                     "to 32 positions: beyond the accuracy of the packed-sequence mechanism")
 
 
 def _set_seq_idx(c, seq_idx, x):
@@ -744,8 +783,14 @@ class MambaChunkScanCombinedFn(torch.autograd.Function):
             # kernels' layout is not used
             for name, like in (("dx", x), ("dB", B), ("dC", C)):
                 t = ctx.grad_places[name]() if ctx.grad_places.get(name) else None
-                if (t is not None and tuple(t.shape) == tuple(like.shape) and t.dtype == x.dtype and like.dtype == x.dtype
-                        and t.stride(3) == 1 and t.stride(2) == like.shape[3] and t.device == x.device):
+                fits = (t is not None and tuple(t.shape) == tuple(like.shape) and t.dtype == x.dtype and like.dtype == x.dtype
+                        and t.stride(3) == 1 and t.stride(2) == like.shape[3] and t.device == x.device)
+                # The forward pass of a 16-bit problem keeps only the 16-bit copies of the entering states, which the
+                # kernels for 16-byte aligned operands read: a destination that is not aligned that way (an odd offset into
+                # a wider buffer) is not used - the kernel writes a fresh tensor and the caller copies it.
+                if fits and x.element_size() == 2 and (t.data_ptr() % 16 or t.stride(0) % 8 or t.stride(1) % 8):
+                    fits = False
+                if fits:
                     given[name] = t
         res = _mamba_chunk_scan_combined_bwd(
             dout, x, dt, A, B, C, out_x, ctx.chunk_size, D=D, z=z, dt_bias=dt_bias, dt_softplus=ctx.dt_softplus,
@@ -783,10 +828,16 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
             neighbouring pieces of a longer sequence).  Gradients flow into them and through the final states.
         seq_idx: (batch, seqlen) integers, optional - not in the bidirectional reference (its causal sibling has it):
             constant over each of several sequences packed one behind the other; positions with different seq_idx do
-            not interact in either direction.
+            not interact in either direction.  When some chunk would hold more than MAX_SEQ_BOUNDARIES_PER_CHUNK (32)
+            sequence boundaries the call runs with a smaller chunk size (the result does not depend on it), which costs
+            one device-to-host synchronisation per call with seq_idx (chunk_size_for_seq_idx).
         grad_places: {"dx": f, "dB": f, "dC": f}, optional - not in the reference: callables asked in the backward pass for
             the tensors these gradients are to be written into (shaped like x / B / C, the two inner dimensions contiguous;
-            e.g. slices of one buffer, which saves concatenating them when x, B, C are pieces of one tensor).
+            e.g. slices of one buffer, which saves concatenating them when x, B, C are pieces of one tensor).  A destination
+            the kernels cannot write (wrong shape or type, inner dimensions not contiguous, for 16-bit types a base or
+            batch / position stride that is not a multiple of 16 bytes) is not used, and neither are any on the routes for
+            headdim > 128 and dstate > 256 (torch glue around several kernel calls): the caller then receives freshly
+            allocated gradients through autograd as without this argument and copies them where it wants them.
     Return:
         out: (batch, seqlen, nheads, headdim), or (out, final_states_f, final_states_b) with
         return_final_states=True (final states are (batch, nheads, headdim, dstate) float32)
@@ -794,6 +845,9 @@ def bimamba_chunk_scan_combined(x, dt, A, B, C, chunk_size, D=None, z=None, dt_b
     # The result does not depend on the chunk size (it only sets where the kernels cut the sequence), and the kernels'
     # chunks hold at most 256 positions: a larger chunk_size, which the reference accepts, runs with 256.
     chunk_size = min(chunk_size, MAX_CHUNK_SIZE)
+    if seq_idx is not None:
+        # many short packed sequences: a smaller chunk keeps the boundaries per chunk inside what the mechanism resolves
+        chunk_size = chunk_size_for_seq_idx(seq_idx, chunk_size)
     headdim = x.shape[-1]
     if headdim > MAX_HEADDIM:
         # The channels of a head only share dt, A and the head's group, so a head wider than the kernels' 128 channels

@@ -95,7 +95,7 @@ typedef struct bimamba2_params {
     float *states_f, *states_b;     /* chunk states, overwritten in place by the inter-chunk scan */
     float *dstates_f, *dstates_b;
     void *dout_x;                   /* dout * silu(z), element type `dtype` */
-    float *ddt_direct, *u_f, *u_b, *v_f, *v_b;
+    float *ddt_direct, *u_f, *u_b, *v_f, *v_b;     /* ddt_direct: bimamba2_ddt_direct_planes() planes of (B, H, nc, Q) */
     float *da_intra;                    /* (B, H, nc, T*T, 2, 64), T = ceil(Q/64): per-tile column / row sums */
     float *ddA_chunk_f, *ddA_chunk_b;   /* (B, H, nc, ceil(P*N/1024)) partial sums */
     float *dBs, *dCs;                   /* (S, B, L, G, N) float32 partial gradients, S = ceil(H/G/8) head slices */
@@ -172,6 +172,19 @@ int bimamba2_state_copies(const bimamba2_params *p);
  * the first three are 0, bimamba2_bmm_chunk_fwd is not needed at all.  Fuses _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208)
  * into its consumers for those shapes. */
 int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which);
+
+/* Planes of ddt_direct: the dx kernel works on headdim column tiles (64 columns for 16-bit types, 32 for float32) and
+ * every tile writes the row sums of its own columns into its own (B, H, nc, Q) plane, plane k at ddt_direct + k*B*H*nc*Q;
+ * bimamba2_chunk_cumsum_bwd called with the same headdim adds them in order.  1 for headdim <= 64 (16-bit) / 32 (float32).
+ * (The reference adds the tiles with atomics, src/ssd/bi/ssd_combined.py:232.) */
+int bimamba2_ddt_direct_planes(const bimamba2_params *p);
+
+/* Heads of one group that one workgroup of bimamba2_chunk_scan_fwd (bwd = 0) or bimamba2_chunk_scan_bwd_dx (bwd = 1)
+ * works through when it rebuilds C.B^T itself: the product is formed once per workgroup and shared by these heads, so the
+ * flops a launch executes for it are (batch * nchunks * nheads / this) * 2 * Q * Q * N.  1 for the kernels that read CB or
+ * rebuild it per head.  A measurement aid (the reference has no counterpart: its _bmm_chunk_fwd computes CB once per group,
+ * src/ssd/bi/ssd_bmm.py:163-208). */
+int bimamba2_chunk_scan_heads_per_workgroup(const bimamba2_params *p, int bwd);
 
 /* Whole forward; replaces _mamba_chunk_scan_combined_fwd (src/ssd/bi/ssd_combined.py:297-331).
  * Needs: x dt A Bm Cm [D z dt_bias] out [out_x when has_z] [final_f final_b] workspace.  Intermediates given as

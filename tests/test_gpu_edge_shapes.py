@@ -126,3 +126,31 @@ def test_offsets_beyond_32_bits(case):
         assert torch.isfinite(a.float()).all(), name
         assert a.float().abs().max() > 0, name
         assert torch.equal(f[last], a), f"{name}: the last batch row differs from the same row computed alone"
+
+
+def test_gradient_destinations_that_break_the_kernels_alignment_are_not_used():
+    """grad_places at a 16-bit fast-path shape: slices of a wider buffer at an odd element offset (not 16-byte aligned) for
+    dx, dB and dC.  The forward kept only the 16-bit copies of the entering states, which the aligned kernels read, so such
+    a destination must be declined (fresh gradients through autograd), not turned into an unsupported-kernel error; aligned
+    slices of the same buffer are written in place.  Both against the oracle."""
+    from bi_mamba2_amd import ops
+    b, L, H, P, G, N, Q, dtype = 1, 300, 2, 64, 1, 64, 256, torch.bfloat16
+    inp = make_case(b, L, H, P, G, N, dtype, with_z=True)
+    r = to64(inp)
+    dout = torch.randn(b, L, H, P, generator=torch.Generator().manual_seed(5)).to(dtype)
+    ref = O.bimamba2_grads(dout.double(), r["x"], r["dt"], r["A"], r["B"], r["C"], D=r["D"], z=r["z"], dt_bias=r["dt_bias"],
+                           dt_softplus=True)
+    width = H * P + 2 * G * N
+    for shift, in_place in ((3, False), (8, True)):
+        d = to_dev(inp)
+        leaves = {k: (v.clone().requires_grad_(True) if v is not None else None) for k, v in d.items()}
+        buf = torch.zeros(b, L, width + 16, device="cuda", dtype=dtype)
+        cuts = {"dx": (shift, H * P, (H, P)), "dB": (shift + H * P, G * N, (G, N)), "dC": (shift + H * P + G * N, G * N, (G, N))}
+        places = {k: (lambda o=o, n=n, sh=sh: buf[..., o:o + n].unflatten(-1, sh)) for k, (o, n, sh) in cuts.items()}
+        out = ops.bimamba_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], Q, D=leaves["D"],
+                                              z=leaves["z"], dt_bias=leaves["dt_bias"], dt_softplus=True, grad_places=places)
+        out.backward(dout.cuda())
+        for k in ("x", "B", "C", "z", "dt", "A", "D", "dt_bias"):
+            assert_close(leaves[k].grad, ref["d" + k], dtype, f"d{k} (offset {shift})", scaled=is_reduced("d" + k, dtype) or k == "x")
+        for k, name in (("x", "dx"), ("B", "dB"), ("C", "dC")):
+            assert (leaves[k].grad.data_ptr() == places[name]().data_ptr()) == in_place, (name, shift)

@@ -33,6 +33,10 @@ CASES = [
     # chunk's cumulative sums
     (2, 512, 4, 32, 2, 16, 256, torch.float32, False, [tuple(range(8, 264, 8)), tuple(range(4, 512, 8))]),
     (1, 512, 4, 64, 1, 64, 256, torch.bfloat16, True, [tuple(range(6, 510, 6))]),
+    # more boundaries per 256 positions than the mechanism resolves in one chunk (64: sequences of 4 tokens; 255: every token
+    # a sequence of its own): the host side runs these with a smaller chunk, float32 still held to the plain 1e-4
+    (1, 512, 4, 32, 2, 16, 256, torch.float32, False, [tuple(range(4, 512, 4))]),
+    (2, 256, 2, 16, 1, 8, 256, torch.float32, True, [tuple(range(1, 256)), tuple(range(2, 256, 2))]),
 ]
 
 

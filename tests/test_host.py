@@ -176,3 +176,26 @@ def test_state_copies_are_for_the_fast_path_only():
     # the generic state passing (float32 problem) does not know the copies
     p = _params(cs_f=256, cs_b=256, states_f=256, states_b=256, states16_f=256, states16_b=256, dtype=_lib.F32)
     assert lib.bimamba2_state_passing_fwd(ctypes.byref(p)) == -2
+
+
+def test_chunk_size_follows_the_number_of_sequence_boundaries():
+    """Packed sequences: the host lowers the chunk size until no chunk holds more boundaries than the float32 cumulative sums
+    resolve (runs on CPU tensors: only the count is taken here)."""
+    import torch
+    from bi_mamba2_amd import ops
+    lim = ops.MAX_SEQ_BOUNDARIES_PER_CHUNK
+    one = torch.zeros(2, 300, dtype=torch.int32)
+    assert ops.seq_boundaries_per_chunk(one, 256) == 0 and ops.chunk_size_for_seq_idx(one, 256) == 256
+    # a boundary in front of position l counts for the chunk of l (forward sums) and for the chunk of l - 1 (reverse sums)
+    edge = torch.zeros(1, 512, dtype=torch.int32)
+    edge[0, 256:] = 1
+    assert ops.seq_boundaries_per_chunk(edge, 256) == 1
+    four = torch.arange(512)[None].div(4, rounding_mode="floor")            # 64 boundaries per 256 positions
+    assert ops.seq_boundaries_per_chunk(four, 256) == 64 and ops.seq_boundaries_per_chunk(four, 128) == 32
+    assert ops.chunk_size_for_seq_idx(four, 256) == 128
+    single = torch.arange(256)[None]                                        # every token its own sequence
+    assert ops.chunk_size_for_seq_idx(single, 256) == 32
+    assert ops.seq_boundaries_per_chunk(single, 32) <= lim
+    mixed = torch.cat([torch.zeros(1, 256, dtype=torch.int64), 1 + torch.arange(256)[None].div(5, rounding_mode="floor")], dim=1)
+    assert ops.chunk_size_for_seq_idx(mixed, 256) == 128                    # the densest chunk decides
+    assert ops.chunk_size_for_seq_idx(four, 64) == 64                       # never above what the caller asked for
