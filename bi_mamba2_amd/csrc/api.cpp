@@ -17,6 +17,12 @@ inline hipStream_t stream_of(const bimamba2_params *p) { return reinterpret_cast
 inline size_t elem_size(int dtype) { return dtype == BIMAMBA2_F32 ? 4 : 2; }
 inline int sp_nsplit(const bimamba2_params *p) { return (p->headdim * p->dstate + 1023) / 1024; }
 
+// the forward scan kernel that rebuilds C.B^T from the 16-bit copies' side: it exists beyond state dimension 64 (128) and
+// runs where the entering states are given as copies
+inline bool fwd_scan_rebuilds_cb(const bimamba2_params *p) {
+    return chunk_scan_uses_scan16(p, false) && p->states16_f && (p->causal || p->states16_b);
+}
+
 int check_problem(const bimamba2_params *p) {
     if (!p) return BIMAMBA2_EINVAL;
     if (p->batch <= 0 || p->seqlen <= 0 || p->nheads <= 0 || p->headdim <= 0 || p->ngroups <= 0 || p->dstate <= 0)
@@ -65,8 +71,6 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     need_f(q->dt_out, bhcq);
     need_f(q->cs_f, bhcq);
     need_f(q->cs_b, bhcq);
-    // CB: read by the forward scan and by the dCB kernel unless they rebuild it; CB^T: by the dx kernel, likewise
-    if (is_bwd ? !(scan_recomputes_cb(q, true) && dcb_recomputes_cb(q)) : !scan_recomputes_cb(q, false)) need_f(q->CB, cbn);
     // 16-bit copies of the entering states (see states16_f in the header): used where the kernels know them and the
     // caller does not ask for the float32 entering states; a backward pass that got the copies from the forward pass
     // needs no float32 states at all
@@ -79,7 +83,12 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
     const bool fwd_only_copies = !is_bwd && !q->causal && (q->dtype == BIMAMBA2_BF16 || q->dtype == BIMAMBA2_F16) &&
                                  (q->headdim * q->dstate) % 4 == 0 && al16(q->final_f) && al16(q->final_b) &&
                                  al16(q->initial_f) && al16(q->initial_b) && !q->states_b && !q->states16_b;
-    if ((copies || fwd_only_copies) && !q->states_f && !q->states16_f) {
+    const bool carve16 = (copies || fwd_only_copies) && !q->states_f && !q->states16_f;
+    // CB: read by the forward scan and by the dCB kernel unless they rebuild it; CB^T: by the dx kernel, likewise.  (The
+    // forward scan kernel for state dimension 128 rebuilds it as well, and runs where the entering states travel as copies.)
+    const bool fwd_scan16 = !is_bwd && chunk_scan_uses_scan16(q, false) && (carve16 || q->states16_f) && (q->causal || carve16 || q->states16_b);
+    if (is_bwd ? !(scan_recomputes_cb(q, true) && dcb_recomputes_cb(q)) : !(scan_recomputes_cb(q, false) || fwd_scan16)) need_f(q->CB, cbn);
+    if (carve16) {
         q->states16_f = cv.take<char>(stn * 2);
         q->states16_b = cv.take<char>(stn * 2);
     }
@@ -183,6 +192,7 @@ int bimamba2_chunk_scan_reads_cb(const bimamba2_params *p, int which) {
     if (check_problem(p)) return 1;
     if (which == 2) return dcb_recomputes_cb(p) ? 0 : 1;
     if (which == 3) return chunk_state_does_cumsum(p) ? 0 : 1;
+    if (which == 0 && fwd_scan_rebuilds_cb(p)) return 0;
     return scan_recomputes_cb(p, which != 0) ? 0 : 1;
 }
 
@@ -225,7 +235,7 @@ int bimamba2_state_passing_fwd(const bimamba2_params *p) {
 int bimamba2_chunk_scan_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->x); REQUIRE(p->Cm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
-    if (!p->CB && !(p->Bm && scan_recomputes_cb(p, false))) return BIMAMBA2_EINVAL;   // without CB the kernel rebuilds it from Cm, Bm
+    if (!p->CB && !(p->Bm && (scan_recomputes_cb(p, false) || fwd_scan_rebuilds_cb(p)))) return BIMAMBA2_EINVAL;   // without CB the kernel rebuilds it from Cm, Bm
     if (!p->states16_f) { REQUIRE(p->states_f); REQUIRE(p->states_b); }
     REQUIRE(p->out);
     if (p->has_D) REQUIRE(p->D);
@@ -340,7 +350,7 @@ int bimamba2_fwd(const bimamba2_params *p) {
     TRY(forward_cumsum_and_states(&q));
     if (q.CB) TRY(bimamba2_bmm_chunk_fwd(&q));     // given by the caller, or carved because the scan kernel reads it
     TRY(bimamba2_state_passing_fwd(&q));
-    if (scan_recomputes_cb(&q, false)) q.CB = nullptr;
+    if (scan_recomputes_cb(&q, false) || fwd_scan_rebuilds_cb(&q)) q.CB = nullptr;
     TRY(bimamba2_chunk_scan_fwd(&q));
     return BIMAMBA2_OK;
 }

@@ -681,16 +681,20 @@ static bool scan_fast(const bimamba2_params *p, bool bwd, int pw, int vs) {
     return fast;
 }
 
-bool scan_recomputes_cb(const bimamba2_params *p, bool bwd) {
-    if (p->dtype == BIMAMBA2_F32 || p->dstate != 64 || scan_col_tile(p) != 64) return false;
+// the conditions of the kernels that rebuild C.B^T, apart from the state dimension
+static bool scan_rebuild_shape(const bimamba2_params *p, bool bwd) {
+    if (p->dtype == BIMAMBA2_F32 || scan_col_tile(p) != 64) return false;
     auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
     if (p->B_sl <= 0 || p->C_sl <= 0 || p->B_sl > (1 << 21) || p->C_sl > (1 << 21)) return false;   // 256 rows in 32-bit byte offsets
     if (!(bwd ? al16(p->dstates_f) && al16(p->dstates_b) : al16(p->states_f) && al16(p->states_b))) return false;
     return scan_fast(p, bwd, 64, 8) && al16(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al16(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg);
 }
 
+bool scan_recomputes_cb(const bimamba2_params *p, bool bwd) { return p->dstate == 64 && scan_rebuild_shape(p, bwd); }
+
 bool chunk_scan_uses_scan16(const bimamba2_params *p, bool bwd) {
-    return scan_recomputes_cb(p, bwd) && (p->headdim == 64 || p->headdim == 128) && p->dstate == 64;
+    // state dimension 64, or 128 in the forward kernel
+    return scan_rebuild_shape(p, bwd) && (p->headdim == 64 || p->headdim == 128) && (p->dstate == 64 || (p->dstate == 128 && !bwd));
 }
 
 template <typename T, int NJMAX, bool BWD>
@@ -723,7 +727,8 @@ static int launch_scan_t(const bimamba2_params *p) {
             else hipLaunchKernelGGL((chunk_scan_kernel<T, 2, 4, BWD, true, 2, true>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
             return check_launch();
         }
-        if ((BWD ? p->CBT : p->CB) == nullptr) {        // the caller checked scan_recomputes_cb()
+        if ((BWD ? p->CBT : p->CB) == nullptr) {
+            if (!scan_recomputes_cb(p, BWD)) return BIMAMBA2_EINVAL;   // (the kernels below rebuild C.B^T at state dimension 64 only)
             if (qt == 1) hipLaunchKernelGGL((chunk_scan_kernel<T, 1, 4, BWD, true, 2>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
             else hipLaunchKernelGGL((chunk_scan_kernel<T, 2, 4, BWD, true, 2>), grid, dim3(SCAN_THREADS), 0, s, *p, nc, npt);
             return check_launch();

@@ -55,16 +55,29 @@ constexpr int S16_ROWS = 16 * S16_WAVES;          // rows the workgroup covers (
 constexpr int S16_NSTEP = S16_ROWS / 32;          // K steps at most
 constexpr int S16_MAX_HEADS = 4;                  // heads a workgroup walks through at most
 
-// LDS map (bytes)
-constexpr int S16_XR = 0;                                     // 2 x raw K-operand tile (x, resp. dy): [256][64] 16-bit, tile64 swizzle
-constexpr int S16_ST = S16_XR + 2 * 32768;                    // 2 x 2 state tiles [p][n], 16-byte chunks ^ (p % 8)
-constexpr int S16_KT = S16_ST + 2 * 2 * 8192;                 // K rows (B, resp. C) of the chunk, chunks ^ (row % 8); afterwards
-                                                              // the z (resp. x) rows of the head in hand, tile64 swizzle
-constexpr int S16_RAW = S16_KT + 32768;                       // 2 x (cs_f, cs_b, dt) of a head as they lie in memory
-constexpr int S16_TAB = S16_RAW + 2 * 3 * 1024;               // lo, up, glo, gup, dtl of the head in hand
-constexpr int S16_RED = S16_TAB + 5 * 1024;                   // mirror: per-wave column sums of dy * x
-constexpr int S16_DT = S16_RED + S16_WAVES * 64 * 4;           // D of the workgroup's heads, one value per headdim column
-constexpr int S16_LDS = S16_DT + S16_MAX_HEADS * 64 * 4;
+// LDS map (bytes), by the state dimension DS (64 or 128).
+// DS = 64: two buffers of x (dy) tiles, two buffers of state tiles, the K rows (32 KB) whose place takes the z (x) rows later.
+// DS = 128: the K rows take 64 KB and a pair of state tiles 32 KB, so the state tiles are single-buffered (the requests for
+// the next head's pair go out behind a barrier that follows this head's state products) and the K rows, needed only in
+// front of the first head, lie over the second x-tile buffer and the z-row area, which are filled later.
+template <int DS> struct S16Map {
+    static constexpr int ROWB = DS * 2;                                   // bytes of a K row / of a state-tile row
+    static constexpr int ST_TILE = 64 * ROWB;                             // one state tile [p][n], 16-byte chunks ^ (p % 8)
+    static constexpr int ST_BUFS = DS == 64 ? 2 : 1;
+    static constexpr int XR0 = 0;                                         // raw K-operand tile (x, resp. dy) of buffer 0: [256][64] 16-bit, tile64 swizzle
+    static constexpr int ST = XR0 + 32768;                                // ST_BUFS x 2 state tiles
+    static constexpr int XR1 = ST + ST_BUFS * 2 * ST_TILE;                // K-operand tile of buffer 1
+    static constexpr int XR_STRIDE = XR1 - XR0;
+    static constexpr int ZR = XR1 + 32768;                                // z (resp. x) rows of the head in hand, tile64 swizzle
+    static constexpr int KT = DS == 64 ? ZR : XR1;                        // K rows (B, resp. C) of the chunk, chunks ^ (row % 8)
+    static constexpr int RAW = ZR + 32768;                                // 2 x (cs_f, cs_b, dt) of a head as they lie in memory
+    static constexpr int TAB = RAW + 2 * 3 * 1024;                        // lo, up, glo, gup, dtl of the head in hand
+    static constexpr int RED = TAB + 5 * 1024;                            // mirror: per-wave column sums of dy * x
+    static constexpr int DT = RED + S16_WAVES * 64 * 4;                   // D of the workgroup's heads, one value per headdim column
+    static constexpr int LDS = DT + S16_MAX_HEADS * 64 * 4;
+    static_assert(KT + 256 * ROWB <= RAW, "the K rows must end in front of the tables");
+    static_assert(LDS <= 160 * 1024, "LDS of a CU");
+};
 
 // byte offset of the elements (r, n ..), n a multiple of 4, in a raw [rows][64] 16-bit tile whose 16-byte chunks are swizzled
 // by tile64_swz (the layout tile64_request leaves)
@@ -109,14 +122,20 @@ __device__ __forceinline__ const char *uniform_ptr(const void *ptr) {
 // diagonal and the far half of the diagonal step are left out.
 // hpw: heads per workgroup (divides nheads / ngroups, <= S16_MAX_HEADS); blockIdx.x = ((pt * nslices + slice) * nbc + bc).
 // DCOLS (mirror): dD per (head, headdim column); else one value per head.
-template <typename T, bool BWD, bool UNI, bool DCOLS = false>
+// DS: the state dimension, 64 or 128 (128: forward only).
+template <typename T, bool BWD, bool UNI, bool DCOLS = false, int DS = 64>
 __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba2_params p, int nc, int npt, int hpw) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
+    typedef S16Map<DS> L;
     static_assert(sizeof(T) == 2, "16-bit operands");
+    static_assert(DS == 64 || (DS == 128 && !BWD), "state dimension 64, or 128 in the forward kernel");
     constexpr int KSTEP = 32, NSTEP = S16_NSTEP;
+    constexpr int NF = DS / 32;                    // MFMA K steps over the state dimension
+    constexpr int ROWB = L::ROWB;
+    constexpr bool ST_SINGLE = L::ST_BUFS == 1;
     // (aligned: the fragment addresses below flip bit 6 of an absolute LDS address)
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[S16_LDS];
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[L::LDS];
     const unsigned sbase = lds_addr(smem);
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lr = lane & 15, lg = lane >> 4;
@@ -162,21 +181,32 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             kp = uniform_ptr(kp);
             // (rows behind the last K step are never read; their requests go to the clamped, valid row all the same)
             // (the mirror is the last kernel of the pass that reads dout_x and the gradients of the entering states)
-            load16_to_lds_at<BWD>(kp, tile_off(ln, part, ks_bytes), smem + S16_XR + buf * 32768 + wave * 2048 + part * 1024);
+            load16_to_lds_at<BWD>(kp, tile_off(ln, part, ks_bytes), smem + L::XR0 + buf * L::XR_STRIDE + wave * 2048 + part * 1024);
         } else if (part == 2) {
             const int dir = wave >> 3;
             if (!(UNI && dir)) {
-                const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * 64 + (int64_t)p0 * 64;
+                const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * DS + (int64_t)p0 * DS;
                 const T *src = reinterpret_cast<const T *>(BWD ? (dir ? p.dstates16_b : p.dstates16_f) : (dir ? p.states16_b : p.states16_f));
-                // thread t of a half brings row t/8, chunk position t%8 <- chunk (t%8) ^ (row%8)
-                const int row = (wave & 7) * 8 + (ln >> 3);
-                const unsigned soff = (unsigned)((row * 64 + (((ln & 7) ^ (row & 7)) << 3)) * sizeof(T));
-                load16_to_lds_at<BWD>(uniform_ptr(src + so), soff, smem + S16_ST + (buf * 2 + dir) * 8192 + (wave & 7) * 1024);
+                const int sbuf = ST_SINGLE ? 0 : buf;
+                if constexpr (DS == 64) {
+                    // thread t of a half brings row t/8, chunk position t%8 <- chunk (t%8) ^ (row%8)
+                    const int row = (wave & 7) * 8 + (ln >> 3);
+                    const unsigned soff = (unsigned)((row * 64 + (((ln & 7) ^ (row & 7)) << 3)) * sizeof(T));
+                    load16_to_lds_at<BWD>(uniform_ptr(src + so), soff, smem + L::ST + (sbuf * 2 + dir) * L::ST_TILE + (wave & 7) * 1024);
+                } else {
+                    // rows of 256 bytes: a wave of a half brings 8 rows in two loads of 4, chunk position l%16 <- chunk (l%16) ^ (row%8)
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const int row = ((wave & 7) * 2 + u) * 4 + (ln >> 4);
+                        const unsigned soff = (unsigned)(row * ROWB + (((ln & 15) ^ (row & 7)) << 4));
+                        load16_to_lds_at<BWD>(uniform_ptr(src + so), soff, smem + L::ST + (sbuf * 2 + dir) * L::ST_TILE + ((wave & 7) * 2 + u) * 1024);
+                    }
+                }
             }
         } else if (wave < 3) {
             // cs_f, cs_b, dt (waves 0, 1, 2): 256 floats each (entries past chunk_size are never used: clamped to stay inside)
             const float *src = (wave == 0 ? p.cs_f : wave == 1 ? p.cs_b : p.dt_out) + (((int64_t)b * H + h) * nc + c) * Q;
-            load16_to_lds_at(uniform_ptr(src), (unsigned)min(ln * 4, Q - 4) * 4u, smem + S16_RAW + (buf * 3 + wave) * 1024);
+            load16_to_lds_at(uniform_ptr(src), (unsigned)min(ln * 4, Q - 4) * 4u, smem + L::RAW + (buf * 3 + wave) * 1024);
         }
     };
     auto request_head = [&](int h, int buf) __attribute__((always_inline)) {
@@ -184,7 +214,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         for (int part = 0; part < 4; ++part) request_part(h, buf, part);
     };
     // requests of a head this wave issues (the vmcnt a wait for something older has to leave outstanding)
-    const int head_requests = 2 + ((UNI && wave >= 8) ? 0 : 1) + (wave < 3 ? 1 : 0);
+    const int head_requests = 2 + ((UNI && wave >= 8) ? 0 : (DS == 64 ? 1 : 2)) + (wave < 3 ? 1 : 0);
 
     // ---- prologue: the K rows of the chunk (B, resp. C), this lane's own rows (C, resp. B), the first head's operands.  The
     // products below wait for the first two only; the head's operands land meanwhile.  (LDS accesses are raw from here on.)
@@ -193,21 +223,23 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         int64_t krs;
         if (BWD) { krs = p.C_sl; kr = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * krs + g * p.C_sg; }
         else { krs = p.B_sl; kr = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * krs + g * p.B_sg; }
+        // units of 1 KB: 8 rows of 128 bytes (DS = 64) or 4 rows of 256 bytes (DS = 128), 16-byte chunk ^ (row % 8)
+        constexpr int UR = 1024 / ROWB, UC = ROWB / 16, NU = 256 / UR / S16_WAVES;
 #pragma unroll
-        for (int uu = 0; uu < 2; ++uu) {
-            const int u = wave * 2 + uu, row = u * 8 + (lane >> 3);
-            if (u * 8 < nsteps * KSTEP)
-                load16_to_lds_at(uniform_ptr(kr), (unsigned)min(row, limit - 1) * (unsigned)(krs * sizeof(T)) + (((lane & 7) ^ (row & 7)) << 4), smem + S16_KT + u * 1024);
+        for (int uu = 0; uu < NU; ++uu) {
+            const int u = wave * NU + uu, row = u * UR + lane / UC;
+            if (u * UR < nsteps * KSTEP)
+                load16_to_lds_at(uniform_ptr(kr), (unsigned)min(row, limit - 1) * (unsigned)(krs * sizeof(T)) + (((lane & (UC - 1)) ^ (row & 7)) << 4), smem + L::KT + u * 1024);
         }
     }
-    Frag own[2];
+    Frag own[NF];
     {
         const T *ap;
         int64_t as;
         if (BWD) { as = p.B_sl; ap = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * as + g * p.B_sg; }
         else { as = p.C_sl; ap = reinterpret_cast<const T *>(p.Cm) + b * p.C_sb + (int64_t)c * Q * as + g * p.C_sg; }
 #pragma unroll
-        for (int f = 0; f < 2; ++f) own[f] = M::load(ap + (int64_t)rc_own * as + f * KSTEP + lg * 8);
+        for (int f = 0; f < NF; ++f) own[f] = M::load(ap + (int64_t)rc_own * as + f * KSTEP + lg * 8);
     }
     float d_val = 0.f;                             // D of head h0 + tid / 64, headdim column tid % 64
     if ((int)threadIdx.x < hpw * 64 && p.has_D) {
@@ -218,7 +250,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
     // everything older than this wave's last two requests has landed (a wave issues at least two per head): the K rows it
     // brought, its own rows, its D values
     wait_vmcnt<2>();
-    if ((int)threadIdx.x < hpw * 64) raw_lds_write_at<0>(sbase + S16_DT + threadIdx.x * 4, d_val);
+    if ((int)threadIdx.x < hpw * 64) raw_lds_write_at<0>(sbase + L::DT + threadIdx.x * 4, d_val);
     raw_lds_wait();
     raw_lds_barrier();
     // CB (resp. CB^T) of this wave's rows against every column of the chunk, in operand layout: D[m][n] = sum_d Krow[k(m)][d]
@@ -230,20 +262,24 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
     float cb_unscale;                              // 1 / (the power of two the entries were scaled by)
     {
         f32x4 cb1[NSTEP], cb2[NSTEP];
-        const int kfb = (8 * (lr >> 2) + (lr & 3)) * 64 + (lg ^ (lr & 3)) * 8;
-        const unsigned kt = sbase + S16_KT + kfb * 2;
+        // (in bytes, rows of ROWB: fragment (hh, f) of step s sits at s*32*ROWB + hh*4*ROWB + 64*((f&1)^hh) + 128*(f>>1) from here)
+        const unsigned kt = sbase + L::KT + (8 * (lr >> 2) + (lr & 3)) * ROWB + (lg ^ (lr & 3)) * 16;
         static_for<0, NSTEP>([&](auto S) __attribute__((always_inline)) {
             constexpr int s = decltype(S)::value;
             cb1[s] = cb2[s] = f32x4{0.f, 0.f, 0.f, 0.f};
             if (active && s < nsteps) {
-                Frag kf00 = raw_lds_read_at<Frag, s * 4096>(kt), kf01 = raw_lds_read_at<Frag, s * 4096 + 64>(kt);
-                Frag kf10 = raw_lds_read_at<Frag, s * 4096 + 512 + 64>(kt), kf11 = raw_lds_read_at<Frag, s * 4096 + 512>(kt);
-                raw_lds_wait();
-                raw_lds_use(kf00); raw_lds_use(kf01); raw_lds_use(kf10); raw_lds_use(kf11);
-                cb1[s] = M::mma(kf00, own[0], cb1[s]);
-                cb2[s] = M::mma(kf10, own[0], cb2[s]);
-                cb1[s] = M::mma(kf01, own[1], cb1[s]);
-                cb2[s] = M::mma(kf11, own[1], cb2[s]);
+                static_for<0, NF / 2>([&](auto F2) __attribute__((always_inline)) {
+                    constexpr int f2 = decltype(F2)::value, O = s * 32 * ROWB + 128 * f2;
+                    Frag kf00 = raw_lds_read_at<Frag, O>(kt), kf01 = raw_lds_read_at<Frag, O + 64>(kt);
+                    Frag kf10 = raw_lds_read_at<Frag, O + 4 * ROWB + 64>(kt), kf11 = raw_lds_read_at<Frag, O + 4 * ROWB>(kt);
+                    raw_lds_wait();
+                    raw_lds_use(kf00); raw_lds_use(kf01); raw_lds_use(kf10); raw_lds_use(kf11);
+                    cb1[s] = M::mma(kf00, own[2 * f2], cb1[s]);
+                    cb2[s] = M::mma(kf10, own[2 * f2], cb2[s]);
+                    cb1[s] = M::mma(kf01, own[2 * f2 + 1], cb1[s]);
+                    cb2[s] = M::mma(kf11, own[2 * f2 + 1], cb2[s]);
+                    return true;
+                });
             }
             return true;
         });
@@ -255,12 +291,12 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(fabsf(cb1[s][i]), fabsf(cb2[s][i])));
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
-        if (lane == 0) raw_lds_write_at<0>(sbase + S16_RED + wave * 4, mx);
+        if (lane == 0) raw_lds_write_at<0>(sbase + L::RED + wave * 4, mx);
         raw_lds_wait();
         wait_vmcnt<0>();                           // the first head's operands (this wave's share; the barrier makes it everybody's)
         raw_lds_barrier();                         // (everybody is done with the K rows as well: their place takes the z / x rows)
         {
-            float wm = raw_lds_read_at<float, 0>(sbase + S16_RED + (lane & (S16_WAVES - 1)) * 4);
+            float wm = raw_lds_read_at<float, 0>(sbase + L::RED + (lane & (S16_WAVES - 1)) * 4);
             raw_lds_wait();
             raw_lds_use(wm);
             mx = wm;
@@ -282,7 +318,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
     }
 
     // per-lane LDS addresses
-    const unsigned tab = sbase + S16_TAB;          // lo +0, up +1024, glo +2048 (mlo +2560), gup +3072 (mup +3584), dtl +4096
+    const unsigned tab = sbase + L::TAB;          // lo +0, up +1024, glo +2048 (mlo +2560), gup +3072 (mup +3584), dtl +4096
     const unsigned lg32 = lg * 32;                 // this lane's 8 columns inside a step of the float tables
     // column factors of this lane's 8 columns (8 float16 = 16 bytes) and the reference exponent of their block of 16
     unsigned g_l = tab + 2048 + lg * 16, m_l = tab + 2048 + 512 + (lg >> 1) * 4;
@@ -295,7 +331,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
     {
         const int kk = 8 * lg + (lr >> 2);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) xo[j] = sbase + S16_XR + tile64_tr_offset(kk, s16_col(j, 4 * (lr & 3)));
+        for (int j = 0; j < 4; ++j) xo[j] = sbase + L::XR0 + tile64_tr_offset(kk, s16_col(j, 4 * (lr & 3)));
     }
     const int cq = 8 * lg;                         // first of this lane's eight columns inside a 32-column half
 
@@ -329,7 +365,8 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         const bool more = hi + 1 < hpw;
         int hn = h + 1;
         asm volatile("" : "+s"(hn));
-        if (more && !active) request_head(hn, cur ^ 1);
+        // (single-buffered state tiles: theirs go out behind the barrier that follows the state products)
+        if (!ST_SINGLE && more && !active) request_head(hn, cur ^ 1);
         if (BWD || p.has_z) {
             const char *row2 = uniform_ptr(
                 BWD ? reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh + p0
@@ -337,8 +374,8 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             if (active) {
                 int ln = lane;
                 asm volatile("" : "+v"(ln));
-                load16_to_lds_at(row2, tile_off(ln, 0, s2_bytes), smem + S16_KT + wave * 2048);
-                load16_to_lds_at(row2, tile_off(ln, 1, s2_bytes), smem + S16_KT + wave * 2048 + 1024);
+                load16_to_lds_at(row2, tile_off(ln, 0, s2_bytes), smem + L::ZR + wave * 2048);
+                load16_to_lds_at(row2, tile_off(ln, 1, s2_bytes), smem + L::ZR + wave * 2048 + 1024);
             }
         }
         // ---- tables of this head
@@ -348,7 +385,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         // between k and r), 2^{lo[r]-lo[k]} = 2^{lo[r]-m} * glo[k], glo[k] = 2^{m-lo[k]}, both factors <= 1 for A <= 0;
         // likewise gup[k] = 2^{up[first of k's block] - up[k]}.  The column factors also carry dt[k] (forward) and the zero
         // of the rows behind the end of the sequence, which the raw tile holds as copies of its last row.
-        const unsigned raw_a = sb + S16_RAW + cur * 3072;        // cs_f +0, cs_b +1024, dt +2048
+        const unsigned raw_a = sb + L::RAW + cur * 3072;        // cs_f +0, cs_b +1024, dt +2048
         if (threadIdx.x < S16_ROWS) {
             int q = threadIdx.x;
             asm volatile("" : "+v"(q));             // (the addresses below are rebuilt per head, not kept across the loop)
@@ -363,7 +400,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             fe *= BWD ? -LOG2E : LOG2E; rs *= BWD ? -LOG2E : LOG2E;
             if (q >= limit) dtq = 0.f;
             const float l = BWD ? -r : f, u = BWD ? -f : r;
-            const unsigned ta = sb + S16_TAB + q * 4;
+            const unsigned ta = sb + L::TAB + q * 4;
             raw_lds_write_at<0>(ta, l);
             raw_lds_write_at<1024>(ta, u);
             raw_lds_write_at<4096>(ta, dtq);
@@ -375,11 +412,11 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             const bool okl = exl > 0 && exl < 254, oku = exu > 0 && exu < 254;       // (zero or denormal maximum: left as it is)
             const _Float16 hl = (_Float16)(okl ? gl * __uint_as_float((253u - exl) << 23) : gl);
             const _Float16 hu = (_Float16)(oku ? gu * __uint_as_float((253u - exu) << 23) : gu);
-            const unsigned tg = sb + S16_TAB + q * 2;
+            const unsigned tg = sb + L::TAB + q * 2;
             raw_lds_write16_at<2048>(tg, hl);
             raw_lds_write16_at<3072>(tg, hu);
             if ((q & 15) == 0) {
-                const unsigned tm = sb + S16_TAB + (q >> 4) * 4;
+                const unsigned tm = sb + L::TAB + (q >> 4) * 4;
                 raw_lds_write_at<2048 + 512>(tm, fe - (okl ? (float)((int)exl - 126) : 0.f));
                 raw_lds_write_at<3072 + 512>(tm, rs - (oku ? (float)((int)exu - 126) : 0.f));
             }
@@ -397,8 +434,10 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         raw_lds_barrier();                         // #1: the tables are there (everybody's requests for this head landed before #2)
 
         f32x4 acc[4];
+        float lor = 0.f, upr = 0.f;
         if (active) {
-            float lor = raw_lds_read_at<float, 0>(tab + r_own * 4), upr = raw_lds_read_at<float, 1024>(tab + r_own * 4);
+            lor = raw_lds_read_at<float, 0>(tab + r_own * 4);
+            upr = raw_lds_read_at<float, 1024>(tab + r_own * 4);
             // ---- part 1: states.  D[p][r] = sum_n S[p][n] Own[r][n], scaled by this lane's row factor, one direction after the other
 #pragma unroll
             for (int dir = 0; dir < (UNI ? 1 : 2); ++dir) {
@@ -407,23 +446,26 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 for (int j = 0; j < 4; ++j) tmp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int jj = 0; jj < 4; jj += 2) {
-                    Frag sf[2][2];
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        // row s16_col(jj + j, lr) of the tile, chunk (4 s + lg) ^ (row % 8)
-                        const int pr = s16_col(jj + j, lr);
-                        const unsigned ra = sbase + S16_ST + (cur * 2 + dir) * 8192 + pr * 128;
-                        sf[j][0] = raw_lds_read_at<Frag, 0>(ra + ((lg ^ (pr & 7)) << 4));
-                        sf[j][1] = raw_lds_read_at<Frag, 0>(ra + (((4 + lg) ^ (pr & 7)) << 4));
-                    }
-                    raw_lds_wait();
+                    for (int s0 = 0; s0 < NF; s0 += 2) {
+                        Frag sf[2][2];
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
-#pragma unroll
-                        for (int s = 0; s < 2; ++s) {
-                            raw_lds_use(sf[j][s]);
-                            tmp[jj + j] = M::mma(sf[j][s], own[s], tmp[jj + j]);
+                        for (int j = 0; j < 2; ++j) {
+                            // row s16_col(jj + j, lr) of the tile, chunk (4 s + lg) ^ (row % 8)
+                            const int pr = s16_col(jj + j, lr);
+                            const unsigned ra = sbase + L::ST + ((ST_SINGLE ? 0 : cur * 2) + dir) * L::ST_TILE + pr * ROWB;
+                            sf[j][0] = raw_lds_read_at<Frag, 0>(ra + (((4 * s0 + lg) ^ (pr & 7)) << 4));
+                            sf[j][1] = raw_lds_read_at<Frag, 0>(ra + (((4 * s0 + 4 + lg) ^ (pr & 7)) << 4));
                         }
+                        raw_lds_wait();
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)
+#pragma unroll
+                            for (int s = 0; s < 2; ++s) {
+                                raw_lds_use(sf[j][s]);
+                                tmp[jj + j] = M::mma(sf[j][s], own[s0 + s], tmp[jj + j]);
+                            }
+                    }
                 }
                 raw_lds_use(lor); raw_lds_use(upr);
                 // forward: e^{cs_f[r]} = 2^{lo[r]}, e^{cs_b[r]} = 2^{up[r]}; mirror: e^{cs_f[Q-1]-cs_f[r]} = 2^{e_f+up[r]}, e^{cs_b[0]-cs_b[r]} = 2^{e_b+lo[r]}
@@ -431,6 +473,15 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[j] = dir ? tmp[j] * e + acc[j] : tmp[j] * e;
             }
+        }
+        if constexpr (ST_SINGLE) {
+            // the one pair of state tiles: every wave is done with it here, so the next head's pair may be requested (the
+            // active waves do that at their third K step)
+            raw_lds_wait();
+            raw_lds_barrier();
+            if (more && !active) request_head(hn, cur ^ 1);
+        }
+        if (active) {
             // ---- part 2: inside the chunk.  Per K step of 32 columns: CB (resp. CB^T) times the decay factors, times the K operand
             auto k_step = [&](auto STEP) __attribute__((always_inline)) -> bool {
                 constexpr int step = decltype(STEP)::value;
@@ -504,7 +555,8 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         if (!more) wait_vmcnt<0>();
         else if (head_requests == 2) wait_vmcnt<2>();
         else if (head_requests == 3) wait_vmcnt<3>();
-        else wait_vmcnt<4>();
+        else if (head_requests == 4) wait_vmcnt<4>();
+        else wait_vmcnt<5>();
         // ---- epilogue.  acc[2t][i], acc[2t+1][i] = row wr0 + lr, headdim columns p0 + 32 t + 8 lg + i, + 4 + i ----
         f32x4 res_a[2], res_b[2];                  // packed results of the two column halves: out / dx, and out_x
         float rsum = 0.f, dsum = 0.f;
@@ -512,7 +564,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         const bool live = r_own < limit;
         if (active) {
             const bool need_d = p.has_D;
-            const unsigned d_a = sb + S16_DT + hi * 256 + cq * 4;
+            const unsigned d_a = sb + L::DT + hi * 256 + cq * 4;
             float dtr = 0.f;                       // mirror: dt of this lane's row
             if (BWD) dtr = raw_lds_read_at<float, 2048>(raw_a + min(r_lane, Q - 1) * 4);
 #pragma unroll
@@ -520,8 +572,8 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 // the D term's row (forward: x, mirror: dy) from the raw tile, z (resp. x) from the rows this wave brought
                 const unsigned eo = sb + tile64_row_offset(min(r_lane, limit - 1), t * 32 + cq);
                 // (read whether used or not: the addresses are valid, and a conditional read needs its registers cleared first)
-                f32x4 kx4 = raw_lds_read_at<f32x4, S16_XR>(eo + cur * 32768);
-                f32x4 g24 = raw_lds_read_at<f32x4, 0>(eo + S16_KT);
+                f32x4 kx4 = raw_lds_read_at<f32x4, L::XR0>(eo + cur * L::XR_STRIDE);
+                f32x4 g24 = raw_lds_read_at<f32x4, L::ZR>(eo);
                 f32x4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
                 if (!BWD || need_d) {                  // (the mirror is out of registers: there the read stays conditional)
                     d0 = t ? raw_lds_read_at<f32x4, 128>(d_a) : raw_lds_read_at<f32x4, 0>(d_a);
@@ -608,7 +660,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             if (d_cols) {
                 // dD partial of this (b, c, h): column sums of dy * x over the rows; a lane holds columns s16_col(j, 4 lg + i) of
                 // row lr: add the 16 lanes of a row group, then the waves
-                const unsigned red_a = sb + S16_RED + (wave * 64 + 8 * lg) * 4;
+                const unsigned red_a = sb + L::RED + (wave * 64 + 8 * lg) * 4;
                 static_for<0, 16>([&](auto JI) __attribute__((always_inline)) {
                     constexpr int j = decltype(JI)::value >> 2, i = decltype(JI)::value & 3;
                     const float v = row16_sum(active ? acc[j][i] : 0.f);
@@ -622,7 +674,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 float v = row16_sum((active && live) ? dsum : 0.f);
                 v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((ln ^ 16) << 2, __builtin_bit_cast(int, v)));
                 v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((ln ^ 32) << 2, __builtin_bit_cast(int, v)));
-                if (ln == 0) raw_lds_write_at<0>(sb + S16_RED + wave * 4, v);
+                if (ln == 0) raw_lds_write_at<0>(sb + L::RED + wave * 4, v);
             }
         }
         // #2: everybody is done with this head's tiles, tables and z rows (a bare barrier: the stores just issued need not
@@ -633,7 +685,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             float pv[S16_WAVES];
             // per column: the waves' sums of this thread's column; per head: the waves' sums, kept by thread 0 (the partial sums
             // have the same layout either way, [(b, c)][h][P]: the other columns of the head then hold zeros)
-            const unsigned red_a = sb + S16_RED + (d_cols ? threadIdx.x * 4 : 0u);
+            const unsigned red_a = sb + L::RED + (d_cols ? threadIdx.x * 4 : 0u);
             if (d_cols) {
                 static_for<0, S16_WAVES>([&](auto WV) __attribute__((always_inline)) {
                     pv[decltype(WV)::value] = raw_lds_read_at<float, decltype(WV)::value * 256>(red_a);
@@ -654,7 +706,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         }
         // the fragment addresses move on to the other buffer
 #pragma unroll
-        for (int j = 0; j < 4; ++j) xo[j] = cur ? xo[j] - 32768u : xo[j] + 32768u;
+        for (int j = 0; j < 4; ++j) xo[j] = cur ? xo[j] - (unsigned)L::XR_STRIDE : xo[j] + (unsigned)L::XR_STRIDE;
     }
 }
 
@@ -700,7 +752,15 @@ static int launch_scan16_t(const bimamba2_params *p, int nc) {
     const int npt = p->headdim / 64, hpw = scan16_heads_per_block(p, nc);
     dim3 grid(p->batch * nc * (p->nheads / hpw) * npt);
     hipStream_t s = reinterpret_cast<hipStream_t>(p->stream);
-    if (BWD && p->has_D && p->D_has_hdim) {
+    if (p->dstate == 128) {
+        // the forward kernel only (launch_chunk_scan sends the mirror of this shape elsewhere)
+        if constexpr (!BWD) {
+            if (p->causal) hipLaunchKernelGGL((chunk_scan16_kernel<T, false, true, false, 128>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
+            else hipLaunchKernelGGL((chunk_scan16_kernel<T, false, false, false, 128>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
+        } else {
+            return BIMAMBA2_EUNSUPPORTED;
+        }
+    } else if (BWD && p->has_D && p->D_has_hdim) {
         if (p->causal) hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, true, BWD>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
         else hipLaunchKernelGGL((chunk_scan16_kernel<T, BWD, false, BWD>), grid, dim3(S16_THREADS), 0, s, *p, nc, npt, hpw);
     } else {
