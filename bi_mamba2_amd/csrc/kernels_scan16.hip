@@ -327,12 +327,10 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
     // supplies the four columns s16_col(j, 4 (s%4)) .., which lanes 4 (s%4) .. + 3 of the group receive
     // (rows k + 4: the swizzle flips bit 2 of the chunk position, i.e. byte bit 6, and the row adds 512 bytes).
     // The addresses follow the buffer of the head in hand.
-    unsigned xo[4];
-    {
-        const int kk = 8 * lg + (lr >> 2);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xo[j] = sbase + L::XR0 + tile64_tr_offset(kk, s16_col(j, 4 * (lr & 3)));
-    }
+    // Tile j reads the columns s16_col(j, 4 (lr%4)) = 32 (j/2) + 4 (j%2) + 8 (lr%4) ..: against tile 0 that is 8 bytes further
+    // for j%2 (bit 3 of the offset, clear in tile 0's) and bit 6 flipped for j/2 (chunk position bit 2), so tile 0's address and
+    // its bit-6 twin serve all four tiles and both row halves, everything else being immediates.
+    unsigned xo0 = sbase + L::XR0 + tile64_tr_offset(8 * lg + (lr >> 2), s16_col(0, 4 * (lr & 3)));
     const int cq = 8 * lg;                         // first of this lane's eight columns inside a 32-column half
 
     auto cb_at = [&](int s, int col) __attribute__((always_inline)) { return (float)__builtin_bit_cast(half2_t, cbh[s][col >> 1])[col & 1]; };
@@ -439,40 +437,36 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             lor = raw_lds_read_at<float, 0>(tab + r_own * 4);
             upr = raw_lds_read_at<float, 1024>(tab + r_own * 4);
             // ---- part 1: states.  D[p][r] = sum_n S[p][n] Own[r][n], scaled by this lane's row factor, one direction after the other
-#pragma unroll
-            for (int dir = 0; dir < (UNI ? 1 : 2); ++dir) {
+            // Fragment (tile j, state step s) of a state tile lies at row s16_col(j, lr), 16-byte chunk (4 s + lg) ^ (row % 8).  With
+            // row = [32 (j/2) + 4 (j%2)] + [8 (lr/4) + lr%4] the lane's part is one address and everything else a constant:
+            // (row % 8) = lr%4 + 4 (j%2), so the chunk is (lg ^ lr%4) + 4 ((s%2) ^ (j%2)) + 8 (s/2).
+            const unsigned st_lane = sb + L::ST + (ST_SINGLE ? 0 : cur * 2 * L::ST_TILE) + (8 * (lr >> 2) + (lr & 3)) * ROWB + ((lg ^ (lr & 3)) << 4);
+            static_for<0, (UNI ? 1 : 2)>([&](auto DIR) __attribute__((always_inline)) {
+                constexpr int dir = decltype(DIR)::value;
                 f32x4 tmp[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) tmp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int jj = 0; jj < 4; jj += 2) {
-#pragma unroll
-                    for (int s0 = 0; s0 < NF; s0 += 2) {
-                        Frag sf[2][2];
-#pragma unroll
-                        for (int j = 0; j < 2; ++j) {
-                            // row s16_col(jj + j, lr) of the tile, chunk (4 s + lg) ^ (row % 8)
-                            const int pr = s16_col(jj + j, lr);
-                            const unsigned ra = sbase + L::ST + ((ST_SINGLE ? 0 : cur * 2) + dir) * L::ST_TILE + pr * ROWB;
-                            sf[j][0] = raw_lds_read_at<Frag, 0>(ra + (((4 * s0 + lg) ^ (pr & 7)) << 4));
-                            sf[j][1] = raw_lds_read_at<Frag, 0>(ra + (((4 * s0 + 4 + lg) ^ (pr & 7)) << 4));
-                        }
-                        raw_lds_wait();
-#pragma unroll
-                        for (int j = 0; j < 2; ++j)
-#pragma unroll
-                            for (int s = 0; s < 2; ++s) {
-                                raw_lds_use(sf[j][s]);
-                                tmp[jj + j] = M::mma(sf[j][s], own[s0 + s], tmp[jj + j]);
-                            }
-                    }
-                }
+                static_for<0, 2 * (NF / 2)>([&](auto JS) __attribute__((always_inline)) {
+                    constexpr int jj = 2 * (decltype(JS)::value / (NF / 2)), s0 = 2 * (decltype(JS)::value % (NF / 2));
+                    constexpr int O0 = dir * L::ST_TILE + (32 * (jj >> 1)) * ROWB + 128 * (s0 >> 1);      // tile jj (even): j%2 = 0
+                    constexpr int O1 = O0 + 4 * ROWB;                                                     // tile jj + 1
+                    Frag a0 = raw_lds_read_at<Frag, O0>(st_lane), a1 = raw_lds_read_at<Frag, O0 + 64>(st_lane);
+                    Frag b0 = raw_lds_read_at<Frag, O1 + 64>(st_lane), b1 = raw_lds_read_at<Frag, O1>(st_lane);
+                    raw_lds_wait();
+                    raw_lds_use(a0); raw_lds_use(a1); raw_lds_use(b0); raw_lds_use(b1);
+                    tmp[jj] = M::mma(a0, own[s0], tmp[jj]);
+                    tmp[jj] = M::mma(a1, own[s0 + 1], tmp[jj]);
+                    tmp[jj + 1] = M::mma(b0, own[s0], tmp[jj + 1]);
+                    tmp[jj + 1] = M::mma(b1, own[s0 + 1], tmp[jj + 1]);
+                    return true;
+                });
                 raw_lds_use(lor); raw_lds_use(upr);
                 // forward: e^{cs_f[r]} = 2^{lo[r]}, e^{cs_b[r]} = 2^{up[r]}; mirror: e^{cs_f[Q-1]-cs_f[r]} = 2^{e_f+up[r]}, e^{cs_b[0]-cs_b[r]} = 2^{e_b+lo[r]}
                 const float e = __builtin_amdgcn_exp2f(BWD ? (dir ? e_b + lor : e_f + upr) : (dir ? upr : lor));
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[j] = dir ? tmp[j] * e + acc[j] : tmp[j] * e;
-            }
+                return true;
+            });
         }
         if constexpr (ST_SINGLE) {
             // the one pair of state tiles: every wave is done with it here, so the next head's pair may be requested (the
@@ -483,6 +477,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         }
         if (active) {
             // ---- part 2: inside the chunk.  Per K step of 32 columns: CB (resp. CB^T) times the decay factors, times the K operand
+            const unsigned xo1 = xo0 ^ 64u;
             auto k_step = [&](auto STEP) __attribute__((always_inline)) -> bool {
                 constexpr int step = decltype(STEP)::value;
                 if (step < 4 && more) request_part(hn, cur ^ 1, step);
@@ -539,8 +534,9 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 constexpr int XS = step * (KSTEP * 128);
 #pragma unroll
                 for (int jj = 0; jj < 4; jj += 2) {
-                    const i16x4 a0 = raw_lds_tr16_read_at<XS>(xo[jj]), a1 = raw_lds_tr16_read_at<XS + 512>(xo[jj] ^ 64u);
-                    const i16x4 b0 = raw_lds_tr16_read_at<XS>(xo[jj + 1]), b1 = raw_lds_tr16_read_at<XS + 512>(xo[jj + 1] ^ 64u);
+                    const unsigned xa = jj ? xo1 : xo0, xb = jj ? xo0 : xo1;
+                    const i16x4 a0 = raw_lds_tr16_read_at<XS>(xa), a1 = raw_lds_tr16_read_at<XS + 512>(xb);
+                    const i16x4 b0 = raw_lds_tr16_read_at<XS + 8>(xa), b1 = raw_lds_tr16_read_at<XS + 512 + 8>(xb);
                     raw_lds_wait();
                     i16x8 fa = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7), fb = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
                     raw_lds_use(fa); raw_lds_use(fb);
@@ -572,8 +568,8 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 // the D term's row (forward: x, mirror: dy) from the raw tile, z (resp. x) from the rows this wave brought
                 const unsigned eo = sb + tile64_row_offset(min(r_lane, limit - 1), t * 32 + cq);
                 // (read whether used or not: the addresses are valid, and a conditional read needs its registers cleared first)
-                f32x4 kx4 = raw_lds_read_at<f32x4, L::XR0>(eo + cur * L::XR_STRIDE);
-                f32x4 g24 = raw_lds_read_at<f32x4, L::ZR>(eo);
+                f32x4 kx4 = raw_lds_read_at<f32x4, 0>(eo + (L::XR0 + cur * L::XR_STRIDE));
+                f32x4 g24 = raw_lds_read_at<f32x4, 0>(eo + L::ZR);
                 f32x4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
                 if (!BWD || need_d) {                  // (the mirror is out of registers: there the read stays conditional)
                     d0 = t ? raw_lds_read_at<f32x4, 128>(d_a) : raw_lds_read_at<f32x4, 0>(d_a);
@@ -705,8 +701,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             p.red[((int64_t)(b * nc + c) * H + h) * P + p0 + threadIdx.x] = v;   // partials [(b, c)][h][P]
         }
         // the fragment addresses move on to the other buffer
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xo[j] = cur ? xo[j] - (unsigned)L::XR_STRIDE : xo[j] + (unsigned)L::XR_STRIDE;
+        xo0 = cur ? xo0 - (unsigned)L::XR_STRIDE : xo0 + (unsigned)L::XR_STRIDE;
     }
 }
 

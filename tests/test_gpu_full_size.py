@@ -98,4 +98,8 @@ def test_long_sequence_forward_against_chunked_oracle_sample(ops):
     r = {k: (v.double() if v is not None else None) for k, v in inp.items()}
     ref = O.bimamba2_naive_chunked(r["x"][:1, :, hs], r["dt"][:1, :, hs], r["A"][hs], r["B"][:1], r["C"][:1], 256,
                                    D=r["D"][hs], dt_bias=r["dt_bias"][hs], dt_softplus=True)[0]
-    assert_close(out[:1, :, hs], ref, torch.bfloat16, "long forward")
+    # 3 million outputs of magnitude up to 25 from operands with 8 bits of mantissa: the largest error sits at 0.9 - 1.05 x the
+    # plain bound depending on the kernel's summation order (one element at 1.03 x with the persistent kernel, none with the
+    # generic one), hence the form with the absolute part in units of the RMS (1.06 here) and its tail allowance, as for the
+    # other full-size outputs
+    assert_close(out[:1, :, hs], ref, torch.bfloat16, "long forward", scaled=True)

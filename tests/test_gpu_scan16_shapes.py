@@ -79,3 +79,36 @@ def test_scan16_shapes_single_direction(ops, case):
     for k in ("x", "z", "B", "C", "dt", "A", "D", "dt_bias"):
         if r[k] is not None:
             assert_close(leaves[k].grad, r[k].grad, dtype, "d" + k, scaled=is_reduced("d" + k, dtype) or k == "x")
+
+
+WIDE_STATE = [
+    # batch, seqlen, H, P, G, chunk, dtype, z, D kind   -- state dimension 128, forward only (the route of a pass without a
+    # backward: 16-bit copies of the entering states, no CB, the persistent kernel's variant with single-buffered state tiles)
+    (2, 300, 4, 64, 1, 256, torch.bfloat16, False, "h"),      # four heads per workgroup, ragged last chunk (44 rows)
+    (1, 700, 6, 64, 2, 128, torch.bfloat16, True, "hp"),      # three heads per workgroup in two groups, z gate, D per column
+    (1, 200, 3, 128, 3, 64, torch.float16, True, "none"),     # one head per workgroup, two headdim tiles, two K steps
+    (2, 513, 8, 64, 1, 192, torch.bfloat16, False, "h"),      # six K steps, a last chunk of 129 rows
+]
+
+
+@pytest.mark.parametrize("case", WIDE_STATE)
+def test_scan16_state_dimension_128_forward(ops, case):
+    b, L, H, P, G, Q, dtype, z, Dk = case
+    inp = make_case(b, L, H, P, G, 128, dtype, with_z=z, with_D=(Dk != "none"), D_has_hdim=(Dk == "hp"))
+    d = to_dev(inp)
+    with torch.no_grad():
+        out, ff, fb = ops.bimamba_chunk_scan_combined(d["x"], d["dt"], d["A"], d["B"], d["C"], Q, D=d["D"], z=d["z"],
+                                                      dt_bias=d["dt_bias"], dt_softplus=True, return_final_states=True)
+    r = to64(inp)
+    ref, _, rf, rb = O.bimamba2_naive_chunked(r["x"], r["dt"], r["A"], r["B"], r["C"], Q, D=r["D"], z=r["z"], dt_bias=r["dt_bias"],
+                                             dt_softplus=True)
+    # (16-bit operands with a state of 128 columns: outputs of magnitude 10 - 60; the absolute part in units of the RMS)
+    assert_close(out, ref, dtype, "out", scaled=True)
+    assert_close(ff, rf, dtype, "final_f", scaled=True)
+    assert_close(fb, rb, dtype, "final_b", scaled=True)
+    # the same pass with the float32 entering states kept (the generic scan kernel on a float32 CB): both routes round the
+    # same operands, so they agree far inside the tolerance
+    leaves = {k: (v.clone().requires_grad_(True) if v is not None else None) for k, v in d.items()}
+    out2 = ops.bimamba_chunk_scan_combined(leaves["x"], leaves["dt"], leaves["A"], leaves["B"], leaves["C"], Q, D=leaves["D"],
+                                           z=leaves["z"], dt_bias=leaves["dt_bias"], dt_softplus=True)
+    assert_close(out, out2.detach(), dtype, "out, both routes", scale=0.5, scaled=True)
