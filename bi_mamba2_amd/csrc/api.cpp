@@ -92,7 +92,11 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
         q->states16_f = cv.take<char>(stn * 2);
         q->states16_b = cv.take<char>(stn * 2);
     }
-    if (!saved_copies) {
+    // a forward pass whose caller asks for no float32 states at all keeps the per-chunk states in the 16-bit copies' place
+    // too (the chunk-state kernel writes them there, the inter-chunk scan replaces them by the entering states)
+    const bool states16_only = !is_bwd && !q->states_f && !q->states_b && (carve16 || (q->states16_f && q->states16_b)) &&
+                               chunk_states_in_16bit(q);
+    if (!saved_copies && !states16_only) {
         need_f(q->states_f, stn);
         need_f(q->states_b, stn);
     }
@@ -222,13 +226,14 @@ int bimamba2_bmm_chunk_fwd(const bimamba2_params *p) {
 int bimamba2_chunk_state_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->x); REQUIRE(p->Bm); REQUIRE(p->dt_out); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
-    REQUIRE(p->states_f); REQUIRE(p->states_b);
+    if (p->states_f || !p->states16_f) { REQUIRE(p->states_f); REQUIRE(p->states_b); }   // (else: 16-bit per-chunk states in states16_*)
     return launch_chunk_state(p, false);
 }
 
 int bimamba2_state_passing_fwd(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->states_f); REQUIRE(p->states_b);
+    REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (p->states_f || !p->states16_f) { REQUIRE(p->states_f); REQUIRE(p->states_b); }
     return launch_state_passing_fwd(p);
 }
 

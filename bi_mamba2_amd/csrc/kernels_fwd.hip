@@ -205,7 +205,10 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_kernel(const bimamba2_pa
 // dt and scans it while the tiles are under way - and the first tile's workgroup writes dt_out, cs_f, cs_b for the later
 // kernels: one launch less in front of the forward pass.
 // UNI: forward direction only (single-direction comparator).
-template <typename T, bool DSTATES, bool CUMSUM, bool UNI = false>
+// OUT16 (chunk states of the forward pass only): the per-chunk states leave in the inputs' 16-bit type, into states16_f/b
+// (where the inter-chunk scan turns them into the entering states in place) - half the bytes of the float32 tensors; the
+// tile passes through LDS so that it is written as 16-byte vectors, a whole 128-byte row piece per eight lanes.
+template <typename T, bool DSTATES, bool CUMSUM, bool UNI = false, bool OUT16 = false>
 __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bimamba2_params p, int nc) {
     typedef Mma<T> M;
     typedef typename M::Frag Frag;
@@ -428,6 +431,32 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     if (nsteps > 5) kstep(std::integral_constant<int, 5>());
     if (nsteps > 6) kstep(std::integral_constant<int, 6>());
     if (nsteps > 7) kstep(std::integral_constant<int, 7>());
+    if constexpr (OUT16 && !DSTATES) {
+        // the two 64 x 64 tiles as 16-bit values into the rings' LDS (everybody is done reading them behind the barrier): row
+        // r at r * 128 bytes, 16-byte chunk ch at position ch ^ ((r / 4) % 4), which keeps the four lane groups (rows 4 apart)
+        // off each other's banks; then every thread takes 32 contiguous bytes of a row of each tile to memory
+        __syncthreads();
+        unsigned char *stf = reinterpret_cast<unsigned char *>(xt), *stb = reinterpret_cast<unsigned char *>(bt);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = wave * 16 + lg * 4 + i, col = j * 16 + lr;
+                const int at = r * 128 + ((((col >> 3) ^ lg) << 4) | ((col & 7) << 1));
+                *reinterpret_cast<T *>(stf + at) = from_f<T>(accf[j][i]);
+                if (!UNI) *reinterpret_cast<T *>(stb + at) = from_f<T>(accb[j][i]);
+            }
+        __syncthreads();
+        const int r = threadIdx.x >> 2, c2 = (threadIdx.x & 3) * 2, sw = (r >> 2) & 3;
+        T *of = reinterpret_cast<T *>(p.states16_f) + (int64_t)bch * P * N + (int64_t)(pt * 64 + r) * N + nt * 64 + c2 * 8;
+        T *ob = reinterpret_cast<T *>(p.states16_b) + (int64_t)bch * P * N + (int64_t)(pt * 64 + r) * N + nt * 64 + c2 * 8;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int at = r * 128 + (((c2 + k) ^ sw) << 4);
+            *reinterpret_cast<f32x4 *>(of + k * 8) = *reinterpret_cast<const f32x4 *>(stf + at);
+            if (!UNI) *reinterpret_cast<f32x4 *>(ob + k * 8) = *reinterpret_cast<const f32x4 *>(stb + at);
+        }
+    } else {
     float *of = (DSTATES ? p.dstates_f : p.states_f) + (int64_t)bch * P * N;
     float *ob = (DSTATES ? p.dstates_b : p.states_b) + (int64_t)bch * P * N;
 #pragma unroll
@@ -438,6 +467,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
             of[(int64_t)pp * N + n] = accf[j][i];
             if (!UNI) ob[(int64_t)pp * N + n] = accb[j][i];
         }
+    }
     if constexpr (DO_CUMSUM) {
         if (wave == 0 && nt == 0 && pt == 0) {
 #pragma unroll
@@ -699,6 +729,17 @@ int launch_bmm_chunk_fwd(const bimamba2_params *p) {
     return check_launch();
 }
 
+// Whether the forward pass of this problem can keep its per-chunk states in the 16-bit type only, in states16_f/b: written
+// there by the chunk-state kernel with direct loads, turned into the entering states in place by the vector kernel of the
+// inter-chunk scan (bidirectional operator, 16-byte aligned operands; the pointers themselves are checked where they are used).
+bool chunk_states_in_16bit(const bimamba2_params *p) {
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
+    return p->dtype != BIMAMBA2_F32 && !p->causal && p->headdim % 64 == 0 && p->dstate % 64 == 0 && p->chunk_size % 32 == 0 &&
+           al(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh) && al(p->states16_f) &&
+           al(p->states16_b) && al(p->final_f) && al(p->final_b) && al(p->initial_f) && al(p->initial_b);
+}
+
 template <typename T>
 static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cumsum) {
     const int nc = nchunks(p);
@@ -721,6 +762,13 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cum
             else hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
             return check_launch();
         }
+        if (fast && p->chunk_size % 32 == 0 && !dstates && !p->states_f) {
+            // no float32 tensors for the per-chunk states: they go to states16_f/b in the 16-bit type
+            if (!p->states16_f || !p->states16_b || !chunk_states_in_16bit(p)) return BIMAMBA2_EINVAL;
+            if (cumsum) hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, true, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            else hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, false, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            return check_launch();
+        }
         if (fast && p->chunk_size % 32 == 0) {
             if (dstates) hipLaunchKernelGGL((chunk_state_direct_kernel<T, true, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
             else if (cumsum) hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
@@ -730,6 +778,7 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cum
     }
     if (p->causal) return BIMAMBA2_EUNSUPPORTED;
     if (cumsum) return BIMAMBA2_EINVAL;      // the caller checked chunk_state_does_cumsum()
+    if (!dstates && !(p->states_f && p->states_b)) return BIMAMBA2_EINVAL;   // (16-bit per-chunk states: the kernel above only)
     if (dstates) {
         if (fast) hipLaunchKernelGGL((chunk_state_kernel<T, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
         else hipLaunchKernelGGL((chunk_state_kernel<T, true, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
@@ -833,10 +882,68 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_fwd_vec_kernel(const b
     if (fin) *reinterpret_cast<f32x4 *>(fin + ((int64_t)b * p.nheads + h) * PN + e) = s;
 }
 
+// The same recurrences on per-chunk states that lie in states16_f/b in the 16-bit type (chunk_state_direct_kernel<.., OUT16>):
+// every state is read once and replaced by the state entering its chunk; the running state stays in float32 registers.
+// 8 elements (16 bytes) per thread, the loads of 8 chunks in flight.
+template <typename T16>
+__global__ __launch_bounds__(NTHREADS) void state_passing_fwd_inplace16_kernel(const bimamba2_params p, int nc) {
+    const int PN = p.headdim * p.dstate;
+    const int e = (blockIdx.x * NTHREADS + threadIdx.x) * 8;
+    const int h = blockIdx.y, b = blockIdx.z >> 1, dir = blockIdx.z & 1;
+    if (e >= PN) return;
+    const int Q = p.chunk_size;
+    const float *cs = (dir == 0 ? p.cs_f : p.cs_b) + ((int64_t)b * p.nheads + h) * nc * Q + (dir == 0 ? Q - 1 : 0);
+    const int64_t cstride = (int64_t)p.nheads * PN;
+    T16 *st = reinterpret_cast<T16 *>(dir == 0 ? p.states16_f : p.states16_b) + ((int64_t)b * nc * p.nheads + h) * PN + e;
+    const float *ini = dir == 0 ? p.initial_f : p.initial_b;
+    float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (ini) {
+        const f32x4 a = *reinterpret_cast<const f32x4 *>(ini + ((int64_t)b * p.nheads + h) * PN + e);
+        const f32x4 c4 = *reinterpret_cast<const f32x4 *>(ini + ((int64_t)b * p.nheads + h) * PN + e + 4);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { s[k] = a[k]; s[4 + k] = c4[k]; }
+    }
+    for (int s0 = 0; s0 < nc; s0 += 8) {
+        Vec16<T16> v[8];
+        float d[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int si = min(s0 + i, nc - 1), c = dir == 0 ? si : nc - 1 - si;
+            v[i] = *reinterpret_cast<const Vec16<T16> *>(st + c * cstride);
+            d[i] = cs[(int64_t)c * Q];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (s0 + i < nc) {
+                const int c = dir == 0 ? s0 + i : nc - 1 - (s0 + i);
+                Vec16<T16> o;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) o.v[k] = from_f<T16>(s[k]);
+                *reinterpret_cast<Vec16<T16> *>(st + c * cstride) = o;
+                const float dec = __expf(d[i]);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) s[k] = dec * s[k] + to_f(v[i].v[k]);
+            }
+    }
+    float *fin = dir == 0 ? p.final_f : p.final_b;
+    if (fin) {
+        *reinterpret_cast<f32x4 *>(fin + ((int64_t)b * p.nheads + h) * PN + e) = f32x4{s[0], s[1], s[2], s[3]};
+        *reinterpret_cast<f32x4 *>(fin + ((int64_t)b * p.nheads + h) * PN + e + 4) = f32x4{s[4], s[5], s[6], s[7]};
+    }
+}
+
 int launch_state_passing_fwd(const bimamba2_params *p) {
     const int nc = nchunks(p), PN = p->headdim * p->dstate;
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     const int ndir = p->causal ? 1 : 2;
+    if (!p->states_f) {
+        // the per-chunk states lie in states16_f/b (16-bit): in place
+        if (!p->states16_f || !p->states16_b || !chunk_states_in_16bit(p)) return BIMAMBA2_EINVAL;
+        dim3 grid((PN / 8 + NTHREADS - 1) / NTHREADS, p->nheads, p->batch * 2);
+        if (p->dtype == BIMAMBA2_BF16) hipLaunchKernelGGL(state_passing_fwd_inplace16_kernel<bf16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+        else hipLaunchKernelGGL(state_passing_fwd_inplace16_kernel<f16_t>, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc);
+        return check_launch();
+    }
     if (PN % 4 == 0 && al(p->states_f) && al(p->states_b) && al(p->final_f) && al(p->final_b) && al(p->initial_f) && al(p->initial_b)) {
         dim3 grid((PN / 4 + NTHREADS - 1) / NTHREADS, p->nheads, p->batch * ndir);
         if (p->states16_f) {

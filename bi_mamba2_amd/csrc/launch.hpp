@@ -23,6 +23,8 @@ int launch_chunk_cumsum_fwd(const bimamba2_params *p);
 int launch_bmm_chunk_fwd(const bimamba2_params *p);
 int launch_chunk_state(const bimamba2_params *p, bool dstates, bool cumsum = false);   // cumsum: also does the chunk cumsum
 bool chunk_state_does_cumsum(const bimamba2_params *p);
+// the forward pass may keep its per-chunk states in states16_f/b only (16-bit type, no float32 state tensors)
+bool chunk_states_in_16bit(const bimamba2_params *p);
 int launch_state_passing_fwd(const bimamba2_params *p);
 int launch_chunk_scan(const bimamba2_params *p, bool bwd);
 // the 16-bit kernel of kernels_scan16.hip (launch_chunk_scan picks it where it applies)
