@@ -152,6 +152,12 @@ template <bool RAW = true> __device__ __forceinline__ void raw_lds_write(float *
 template <bool RAW = true> __device__ __forceinline__ void raw_lds_wait() {
     if constexpr (RAW) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 }
+// at most N LDS operations of this wave outstanding (they complete in order): the oldest reads can be used while the
+// younger ones are still under way
+template <int N> __device__ __forceinline__ void raw_lds_wait_n() {
+    static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit field");
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+}
 // Workgroup barrier to go with them: __syncthreads() carries fences that drain every outstanding vector memory operation
 // when a direct global->LDS load is in flight; the bare barrier does not.  All LDS traffic around it must be raw and
 // settled with raw_lds_wait() (writes) resp. the caller's own vmcnt wait (direct loads) beforehand.

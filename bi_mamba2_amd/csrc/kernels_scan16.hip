@@ -53,7 +53,7 @@ namespace {
 constexpr int S16_WAVES = 16, S16_THREADS = 64 * S16_WAVES;
 constexpr int S16_ROWS = 16 * S16_WAVES;          // rows the workgroup covers (>= chunk_size)
 constexpr int S16_NSTEP = S16_ROWS / 32;          // K steps at most
-constexpr int S16_MAX_HEADS = 4;                  // heads a workgroup walks through at most
+constexpr int S16_MAX_HEADS = 12;                 // heads a workgroup walks through at most
 
 // LDS map (bytes), by the state dimension DS (64 or 128).
 // DS = 64: two buffers of x (dy) tiles, two buffers of state tiles, the K rows (32 KB) whose place takes the z (x) rows later.
@@ -487,14 +487,22 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 const int cls = (k0 + KSTEP - 1 < wr0_l) ? 0 : (k0 > wr0_l + 15) ? 1 : 2;   // below, above, across the diagonal
                 if (UNI && cls == (BWD ? 0 : 1)) return true;                              // far side of the diagonal
                 constexpr int TB = step * (KSTEP * 4);     // byte offset of the step inside the float tables
+                constexpr int XS = step * (KSTEP * 128);
                 Frag af;
+                // the K-operand fragments of the first two column tiles are asked for behind the step's table values and
+                // arrive while the decay factors are worked out
+                // (all of them in straight-line code in front of the branch: a value read from inline assembly must not pass
+                // through a merge of two definitions, whose copy could be placed in front of the wait; the step across the
+                // diagonal reads the column factors without using them)
+                const unsigned sel = cls == 1 ? 1024u : 0u;
+                typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+                u32x4 gq = raw_lds_read_at<u32x4, step * 64>(g_l + sel);
+                float mref = raw_lds_read_at<float, step * 8>(m_l + sel);
+                i16x4 xa0 = raw_lds_tr16_read_at<XS>(xo0), xa1 = raw_lds_tr16_read_at<XS + 512>(xo1);
+                i16x4 xb0 = raw_lds_tr16_read_at<XS + 8>(xo0), xb1 = raw_lds_tr16_read_at<XS + 512 + 8>(xo1);
+                raw_lds_wait_n<4>();
+                raw_lds_use(gq); raw_lds_use(mref);
                 if (cls != 2) {
-                    const unsigned sel = cls == 0 ? 0u : 1024u;
-                    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-                    u32x4 gq = raw_lds_read_at<u32x4, step * 64>(g_l + sel);
-                    float mref = raw_lds_read_at<float, step * 8>(m_l + sel);
-                    raw_lds_wait();
-                    raw_lds_use(gq); raw_lds_use(mref);
                     const float rf = __builtin_amdgcn_exp2f((cls == 0 ? lor : upr) - mref) * cb_unscale;
                     float v[8];
 #pragma unroll
@@ -531,17 +539,20 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                     af = M::pack(v);
                 }
                 // ---- the product with the K operand, transposed: D[p][r] += X[k][p] A[r][k]; two column tiles at a time
-                constexpr int XS = step * (KSTEP * 128);
-#pragma unroll
-                for (int jj = 0; jj < 4; jj += 2) {
-                    const unsigned xa = jj ? xo1 : xo0, xb = jj ? xo0 : xo1;
-                    const i16x4 a0 = raw_lds_tr16_read_at<XS>(xa), a1 = raw_lds_tr16_read_at<XS + 512>(xb);
-                    const i16x4 b0 = raw_lds_tr16_read_at<XS + 8>(xa), b1 = raw_lds_tr16_read_at<XS + 512 + 8>(xb);
+                {
+                    // tiles 2, 3 (the bit-6 twins of the addresses) are asked for before tiles 0, 1 are multiplied
+                    const i16x4 c0 = raw_lds_tr16_read_at<XS>(xo1), c1 = raw_lds_tr16_read_at<XS + 512>(xo0);
+                    const i16x4 d0 = raw_lds_tr16_read_at<XS + 8>(xo1), d1 = raw_lds_tr16_read_at<XS + 512 + 8>(xo0);
+                    raw_lds_wait_n<4>();
+                    raw_lds_use(xa0); raw_lds_use(xa1); raw_lds_use(xb0); raw_lds_use(xb1);
+                    i16x8 fa = __builtin_shufflevector(xa0, xa1, 0, 1, 2, 3, 4, 5, 6, 7), fb = __builtin_shufflevector(xb0, xb1, 0, 1, 2, 3, 4, 5, 6, 7);
+                    acc[0] = M::mma(__builtin_bit_cast(Frag, fa), af, acc[0]);
+                    acc[1] = M::mma(__builtin_bit_cast(Frag, fb), af, acc[1]);
                     raw_lds_wait();
-                    i16x8 fa = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7), fb = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7);
-                    raw_lds_use(fa); raw_lds_use(fb);
-                    acc[jj] = M::mma(__builtin_bit_cast(Frag, fa), af, acc[jj]);
-                    acc[jj + 1] = M::mma(__builtin_bit_cast(Frag, fb), af, acc[jj + 1]);
+                    i16x8 fc = __builtin_shufflevector(c0, c1, 0, 1, 2, 3, 4, 5, 6, 7), fd = __builtin_shufflevector(d0, d1, 0, 1, 2, 3, 4, 5, 6, 7);
+                    raw_lds_use(fc); raw_lds_use(fd);
+                    acc[2] = M::mma(__builtin_bit_cast(Frag, fc), af, acc[2]);
+                    acc[3] = M::mma(__builtin_bit_cast(Frag, fd), af, acc[3]);
                 }
                 return true;
             };
