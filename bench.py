@@ -688,8 +688,10 @@ def main():
             "ms_per_step": t_causal * 1e3, "Mtokens_s": tokens / t_causal / 1e6,
             "bidirectional_over_causal": t_step / t_causal,
             "what": "single-direction SSD (y = SS(x) + D x, z gate) forward + backward from the same kernels with the "
-                    "reverse direction compiled out, same shape and dtypes; the scan kernels skip the K steps (and the "
-                    "reverse state tiles) the single direction does not use but still load the whole K-operand tile"}
+                    "reverse direction compiled out, same shape and dtypes: one chunk state and one entering state per "
+                    "chunk, one state product, no K steps on the far side of the diagonal, no dCB tiles above it, no "
+                    "reverse terms in the dt gradient; the chunk's K-operand tile is loaded once per workgroup and is "
+                    "needed in full by the causal operator too (the chunk's last rows read all of it)"}
         result.update(extras)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w)
