@@ -55,6 +55,15 @@ __global__ __launch_bounds__(NTHREADS) void chunk_cumsum_fwd_kernel(const bimamb
     const float incl_s = wave_incl_suffix(tot_r, lane);
     const float after = incl_s - tot_r;
     const int64_t o = (((int64_t)b * p.nheads + h) * nc + c) * Q;
+    if (Q % 4 == 0) {
+        // a lane's four positions are contiguous: 16-byte stores (the three tensors are contiguous and Q * 4 bytes per row)
+        if (lane * 4 < Q) {
+            *reinterpret_cast<f32x4 *>(p.dt_out + o + lane * 4) = f32x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4 *>(p.cs_f + o + lane * 4) = f32x4{before + pf[0], before + pf[1], before + pf[2], before + pf[3]};
+            *reinterpret_cast<f32x4 *>(p.cs_b + o + lane * 4) = f32x4{after + sb[0], after + sb[1], after + sb[2], after + sb[3]};
+        }
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int q = lane * 4 + e;
@@ -740,6 +749,212 @@ bool chunk_states_in_16bit(const bimamba2_params *p) {
            al(p->states16_b) && al(p->final_f) && al(p->final_b) && al(p->initial_f) && al(p->initial_b);
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// The chunk states of several heads of one (batch, chunk) in one workgroup (16-bit inputs, 16-bit per-chunk states out,
+// state dimension NH * 64).  With many heads per group and a wide state the kernel above is made of thousands of short
+// workgroups, each a chain of waits (weights, first rows, eight barriers, stores), and reaches half the memory rate; here a
+// workgroup of 4 * NH waves keeps the B rows of the chunk in LDS (loaded once), walks through its heads with the x tile of
+// the next head under way while the current one is multiplied, and stores a head's states while the next one is worked on.
+//   wave w: rows 16 (w % 4) .. of the 64 channels, 64-column tile w / 4 of the state dimension.
+//   LDS: B tile NH x [256][64] (tile64 swizzle) | two x tiles [256][64] | raw cs_f, cs_b, dt vectors of two heads | wf, wb.
+//   The finished head's x tile serves as the staging area of its output (16-byte stores of whole 128-byte row pieces).
+// Needs dt_out, cs_f, cs_b from bimamba2_chunk_cumsum_fwd.  Requests complete in order; a wave waits for everything it has
+// in flight (vmcnt(0)) once per head, in front of that head's stores, when the next head's operands have long landed.
+// ---------------------------------------------------------------------------------------------------------
+template <int NH> struct CshMap {
+    static constexpr int BT = 0;                               // NH tiles of 32 KB
+    static constexpr int XT = BT + NH * 32768;                 // 2 x 32 KB
+    static constexpr int RAW = XT + 2 * 32768;                 // 2 x (cs_f, cs_b, dt) x 1 KB
+    static constexpr int WT = RAW + 2 * 3 * 1024;              // wf, wb
+    static constexpr int LDS = WT + 2 * 1024;
+};
+
+template <typename T, int NH>
+__global__ __launch_bounds__(NH * NTHREADS) void chunk_state_heads_kernel(const bimamba2_params p, int nc, int hpw) {
+    typedef Mma<T> M;
+    typedef typename M::Frag Frag;
+    typedef CshMap<NH> L;
+    static_assert(sizeof(T) == 2, "16-bit operands");
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[L::LDS];
+    const unsigned sbase = lds_addr(smem);
+    constexpr int NW = 4 * NH;
+    const int lane = threadIdx.x & 63, wave8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = wave8 & 3, nh = wave8 >> 2;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int pt = blockIdx.x, slice = blockIdx.y, bc = blockIdx.z, c = bc % nc, b = bc / nc;
+    const int Q = p.chunk_size, N = p.dstate, P = p.headdim, H = p.nheads;
+    const int h0 = slice * hpw, g = h0 / (H / p.ngroups);
+    const int limit = min(Q, p.seqlen - c * Q);
+    const int nsteps = (limit + 31) >> 5;
+    // ---- the B rows of the chunk: tile t (64 columns) row r at t * 32 KB + r * 128, 16-byte chunk ^ tile64_swz(r)
+    {
+        const T *bp = reinterpret_cast<const T *>(p.Bm) + b * p.B_sb + (int64_t)c * Q * p.B_sl + g * p.B_sg;
+        for (int u = wave8; u < NH * 32; u += NW) {                  // units of 8 rows x 128 bytes
+            const int t = u >> 5, row = (u & 31) * 8 + (lane >> 3);
+            if ((u & 31) * 8 < nsteps * 32)
+                load16_to_lds(bp + t * 64 + (int64_t)min(row, limit - 1) * p.B_sl + (((lane & 7) ^ tile64_swz(row)) << 3), smem + L::BT + u * 1024);
+        }
+    }
+    // requests of a head: its x tile (32 units of 8 rows) and its three vectors, into buffer `buf`
+    auto request_head = [&](int h, int buf) __attribute__((always_inline)) {
+        const T *xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh + pt * 64;
+        for (int u = wave8; u < 32; u += NW) {
+            const int row = u * 8 + (lane >> 3);
+            if (u * 8 < nsteps * 32)
+                load16_to_lds(xp + (int64_t)min(row, limit - 1) * p.x_sl + (((lane & 7) ^ tile64_swz(row)) << 3), smem + L::XT + buf * 32768 + u * 1024);
+        }
+        if (wave8 < 3) {
+            const float *src = (wave8 == 0 ? p.cs_f : wave8 == 1 ? p.cs_b : p.dt_out) + (((int64_t)b * H + h) * nc + c) * Q;
+            load16_to_lds(src + min(lane * 4, Q - 4), smem + L::RAW + (buf * 3 + wave8) * 1024);
+        }
+    };
+    request_head(h0, 0);
+    // lane parts of the fragment addresses (see tile64_tr_frag): rows kk and kk + 4 of a step, 4 columns from nn on
+    const int kk = 8 * lg + (lr >> 2), nn = 4 * (lr & 3);
+    const unsigned xa_lo0 = sbase + L::XT + tile64_tr_offset(kk, wave * 16 + nn), xa_hi0 = sbase + L::XT + tile64_tr_offset(kk + 4, wave * 16 + nn);
+    unsigned ba_lo[4], ba_hi[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        ba_lo[j] = sbase + L::BT + nh * 32768 + tile64_tr_offset(kk, j * 16 + nn);
+        ba_hi[j] = sbase + L::BT + nh * 32768 + tile64_tr_offset(kk + 4, j * 16 + nn);
+    }
+    const unsigned wfl = sbase + L::WT + 32 * lg, wbl = sbase + L::WT + 1024 + 32 * lg;
+    wait_vmcnt<0>();
+    for (int hi = 0; hi < hpw; ++hi) {
+        const int h = h0 + hi, cur = hi & 1;
+        // #1: this head's x tile and vectors have landed for everybody (each wave waited for its own requests in front of the
+        // previous head's stores, or above); everybody is done with the other x buffer (the previous head's staging area)
+        raw_lds_barrier();
+        if (hi + 1 < hpw) request_head(h + 1, cur ^ 1);
+        if (threadIdx.x < NTHREADS) {
+            const int q = threadIdx.x, qq = min(q, Q - 1);
+            const unsigned ra = sbase + L::RAW + cur * 3072;
+            float cf = raw_lds_read_at<float, 0>(ra + qq * 4), cb = raw_lds_read_at<float, 1024>(ra + qq * 4);
+            float d = raw_lds_read_at<float, 2048>(ra + qq * 4);
+            float ef = raw_lds_read_at<float, 0>(ra + (Q - 1) * 4), eb = raw_lds_read_at<float, 1024>(ra);
+            raw_lds_wait();
+            raw_lds_use(cf); raw_lds_use(cb); raw_lds_use(d); raw_lds_use(ef); raw_lds_use(eb);
+            const bool in = q < limit;
+            raw_lds_write_at<0>(sbase + L::WT + q * 4, in ? __expf(ef - cf) * d : 0.f);
+            raw_lds_write_at<1024>(sbase + L::WT + q * 4, in ? __expf(eb - cb) * d : 0.f);
+            raw_lds_wait();
+        }
+        raw_lds_barrier();                          // #2: the weights are there
+        f32x4 accf[4] = {}, accb[4] = {};
+        const unsigned xa_lo = xa_lo0 + cur * 32768, xa_hi = xa_hi0 + cur * 32768;
+        auto kstep = [&](auto S) __attribute__((always_inline)) {
+            constexpr int s = decltype(S)::value;
+            constexpr int TO = s * 32 * 128, WO = s * 32 * 4;
+            i16x4 alo = raw_lds_tr16_read_at<TO>(xa_lo), ahi = raw_lds_tr16_read_at<TO>(xa_hi);
+            f32x4 f0 = raw_lds_read_at<f32x4, WO>(wfl), f1 = raw_lds_read_at<f32x4, WO + 16>(wfl);
+            f32x4 r0 = raw_lds_read_at<f32x4, WO>(wbl), r1 = raw_lds_read_at<f32x4, WO + 16>(wbl);
+            i16x4 blo[4], bhi[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { blo[j] = raw_lds_tr16_read_at<TO>(ba_lo[j]); bhi[j] = raw_lds_tr16_read_at<TO>(ba_hi[j]); }
+            raw_lds_wait();
+            raw_lds_use(alo); raw_lds_use(ahi); raw_lds_use(f0); raw_lds_use(f1); raw_lds_use(r0); raw_lds_use(r1);
+            const Frag a = __builtin_bit_cast(Frag, __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7));
+            float vf[8], vb[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float v = to_f(a[i]);
+                vf[i] = v * (i < 4 ? f0[i & 3] : f1[i & 3]);
+                vb[i] = v * (i < 4 ? r0[i & 3] : r1[i & 3]);
+            }
+            const Frag af = M::pack(vf), ab = M::pack(vb);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                raw_lds_use(blo[j]); raw_lds_use(bhi[j]);
+                const Frag bfr = __builtin_bit_cast(Frag, __builtin_shufflevector(blo[j], bhi[j], 0, 1, 2, 3, 4, 5, 6, 7));
+                accf[j] = M::mma(af, bfr, accf[j]);
+                accb[j] = M::mma(ab, bfr, accb[j]);
+            }
+        };
+        kstep(std::integral_constant<int, 0>());
+        if (nsteps > 1) kstep(std::integral_constant<int, 1>());
+        if (nsteps > 2) kstep(std::integral_constant<int, 2>());
+        if (nsteps > 3) kstep(std::integral_constant<int, 3>());
+        if (nsteps > 4) kstep(std::integral_constant<int, 4>());
+        if (nsteps > 5) kstep(std::integral_constant<int, 5>());
+        if (nsteps > 6) kstep(std::integral_constant<int, 6>());
+        if (nsteps > 7) kstep(std::integral_constant<int, 7>());
+        raw_lds_barrier();                          // #3: everybody is done with this head's x tile: it becomes the staging area
+        // tile (direction d, column tile nh) at (d * NH + nh) * 8 KB: row r at r * 128, 16-byte chunk ch at ch ^ ((r / 4) % 4)
+        const unsigned st = sbase + L::XT + cur * 32768;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = wave * 16 + lg * 4 + i, col = j * 16 + lr;
+                const unsigned at = st + nh * 8192 + r * 128 + ((((col >> 3) ^ lg) << 4) | ((col & 7) << 1));
+                // (the 16 bits of the value, whatever the type: the accessor takes them as a _Float16)
+                raw_lds_write16_at<0>(at, __builtin_bit_cast(_Float16, from_f<T>(accf[j][i])));
+                raw_lds_write16_at<NH * 8192>(at, __builtin_bit_cast(_Float16, from_f<T>(accb[j][i])));
+            }
+        raw_lds_wait();
+        raw_lds_barrier();                          // #4
+        {
+            const int tid = threadIdx.x & 255, r = tid >> 2, c2 = (tid & 3) * 2, sw = (r >> 2) & 3;
+            const unsigned at = st + nh * 8192 + r * 128;
+            f32x4 vf0 = raw_lds_read_at<f32x4, 0>(at + ((c2 ^ sw) << 4)), vf1 = raw_lds_read_at<f32x4, 0>(at + (((c2 + 1) ^ sw) << 4));
+            f32x4 vb0 = raw_lds_read_at<f32x4, NH * 8192>(at + ((c2 ^ sw) << 4)), vb1 = raw_lds_read_at<f32x4, NH * 8192>(at + (((c2 + 1) ^ sw) << 4));
+            raw_lds_wait();
+            raw_lds_use(vf0); raw_lds_use(vf1); raw_lds_use(vb0); raw_lds_use(vb1);
+            // the next head's operands (this wave's share) have landed long ago; waited for here, in front of the stores
+            wait_vmcnt<0>();
+            const int64_t so = (((int64_t)(b * nc + c) * H + h) * P + pt * 64 + r) * N + nh * 64 + c2 * 8;
+            T *of = reinterpret_cast<T *>(p.states16_f) + so, *ob = reinterpret_cast<T *>(p.states16_b) + so;
+            *reinterpret_cast<f32x4 *>(of) = vf0;
+            *reinterpret_cast<f32x4 *>(of + 8) = vf1;
+            *reinterpret_cast<f32x4 *>(ob) = vb0;
+            *reinterpret_cast<f32x4 *>(ob + 8) = vb1;
+        }
+    }
+}
+
+// heads per workgroup of the kernel above: the divisor of the heads per group (at most 32) that brings the number of workgroups
+// closest to a whole number of rounds of one per CU, the larger on a tie
+static int csh_heads_per_block(const bimamba2_params *p, int nc) {
+    const int hpg = p->nheads / p->ngroups;
+    int cus = 256;
+    {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    }
+    const long long units = (long long)p->batch * nc * (p->headdim / 64) * p->nheads;
+    int best = 1;
+    double best_cost = 0;
+    for (int k = 1; k <= std::min(hpg, 32); ++k) {
+        if (hpg % k) continue;
+        const long long rounds = (units / k + cus - 1) / cus;
+        const double cost = rounds * (1.5 + k);          // a workgroup's start (B rows, first head's operands) costs about 1.5 heads
+        if (k == 1 || cost <= best_cost) { best = k; best_cost = cost; }
+    }
+    return best;
+}
+
+bool chunk_state_uses_heads_kernel(const bimamba2_params *p) {
+    // where it pays: a state of 128 columns and enough heads per group to share the B rows
+    return chunk_states_in_16bit(p) && p->dstate == 128 && p->headdim % 64 == 0 && p->nheads / p->ngroups >= 4 &&
+           p->x_sl > 0 && p->x_sl <= (1 << 21) && p->B_sl > 0 && p->B_sl <= (1 << 21);
+}
+
+template <typename T>
+static int launch_chunk_state_heads_t(const bimamba2_params *p) {
+    const int nc = nchunks(p), hpw = csh_heads_per_block(p, nc);
+    dim3 grid(p->headdim / 64, p->nheads / hpw, p->batch * nc);
+    hipLaunchKernelGGL((chunk_state_heads_kernel<T, 2>), grid, dim3(2 * NTHREADS), 0, stream_of(p), *p, nc, hpw);
+    return check_launch();
+}
+
+int launch_chunk_state_heads(const bimamba2_params *p) {
+    if (!p->states16_f || !p->states16_b || !chunk_state_uses_heads_kernel(p)) return BIMAMBA2_EINVAL;
+    if (p->dtype == BIMAMBA2_BF16) return launch_chunk_state_heads_t<bf16_t>(p);
+    if (p->dtype == BIMAMBA2_F16) return launch_chunk_state_heads_t<f16_t>(p);
+    return BIMAMBA2_EUNSUPPORTED;
+}
+
+
 template <typename T>
 static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cumsum) {
     const int nc = nchunks(p);
@@ -765,6 +980,7 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cum
         if (fast && p->chunk_size % 32 == 0 && !dstates && !p->states_f) {
             // no float32 tensors for the per-chunk states: they go to states16_f/b in the 16-bit type
             if (!p->states16_f || !p->states16_b || !chunk_states_in_16bit(p)) return BIMAMBA2_EINVAL;
+            if (!cumsum && chunk_state_uses_heads_kernel(p)) return launch_chunk_state_heads(p);
             if (cumsum) hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, true, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
             else hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, false, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
             return check_launch();
@@ -804,6 +1020,8 @@ bool chunk_state_does_cumsum(const bimamba2_params *p) {
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
     if (p->seq_idx) return false;                 // packed sequences: the stand-alone cumsum kernel applies the cuts
+    // (the kernel that walks through several heads per workgroup reads the cumulative sums: the stand-alone launch comes first)
+    if (!p->states_f && p->states16_f && p->states16_b && chunk_state_uses_heads_kernel(p)) return false;
     return p->dtype != BIMAMBA2_F32 && p->headdim % 64 == 0 && p->dstate % 64 == 0 && p->chunk_size % 32 == 0 && al(p->Bm) &&
            mult(p->B_sb, p->B_sl, p->B_sg) && al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh);
 }

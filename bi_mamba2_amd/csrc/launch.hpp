@@ -25,6 +25,9 @@ int launch_chunk_state(const bimamba2_params *p, bool dstates, bool cumsum = fal
 bool chunk_state_does_cumsum(const bimamba2_params *p);
 // the forward pass may keep its per-chunk states in states16_f/b only (16-bit type, no float32 state tensors)
 bool chunk_states_in_16bit(const bimamba2_params *p);
+// the chunk-state kernel whose workgroups walk through several heads of one (batch, chunk): where it is used, and its launch
+bool chunk_state_uses_heads_kernel(const bimamba2_params *p);
+int launch_chunk_state_heads(const bimamba2_params *p);
 int launch_state_passing_fwd(const bimamba2_params *p);
 int launch_chunk_scan(const bimamba2_params *p, bool bwd);
 // the 16-bit kernel of kernels_scan16.hip (launch_chunk_scan picks it where it applies)
