@@ -55,14 +55,15 @@ def stage_table(w, e, fused=(False, False, False), copies=False, heads_per_wg=(1
         # entry point: (flops, bytes)
         "bimamba2_chunk_cumsum_fwd": (0, 4 * B * L * H + 3 * 4 * T1),
         "bimamba2_bmm_chunk_fwd": (ug * 2 * Q * Q * N, 2 * e * T2 + cb),
-        "bimamba2_chunk_state_fwd": (u * 4 * P * N * Q, e * T4 + e * T2 + 3 * 4 * T1 + 2 * st),
-        "bimamba2_state_passing_fwd": (0, 2 * st + 2 * se),
+        # (with the 16-bit copies the per-chunk states and their gradients are 16-bit as well: se instead of st)
+        "bimamba2_chunk_state_fwd": (u * 4 * P * N * Q, e * T4 + e * T2 + 3 * 4 * T1 + 2 * se),
+        "bimamba2_state_passing_fwd": (0, 2 * se + 2 * se),
         "bimamba2_chunk_scan_fwd": (u * (2 * Q * Q * P + 4 * Q * P * N) + scan_cb[0][0],
                                     4 * e * T4 + e * T2 + 3 * 4 * T1 + 2 * se + scan_cb[0][1]),
         "bimamba2_chunk_scan_bwd_dz": (0, 5 * e * T4),
-        "bimamba2_chunk_scan_bwd_dstates": (u * 4 * P * N * Q, e * T4 + e * T2 + 2 * 4 * T1 + 2 * st),
-        "bimamba2_chunk_scan_bwd_dz_dstates": (u * 4 * P * N * Q, 5 * e * T4 + e * T2 + 2 * 4 * T1 + 2 * st),
-        "bimamba2_state_passing_bwd": (0, 2 * st + 4 * se),
+        "bimamba2_chunk_scan_bwd_dstates": (u * 4 * P * N * Q, e * T4 + e * T2 + 2 * 4 * T1 + 2 * se),
+        "bimamba2_chunk_scan_bwd_dz_dstates": (u * 4 * P * N * Q, 5 * e * T4 + e * T2 + 2 * 4 * T1 + 2 * se),
+        "bimamba2_state_passing_bwd": (0, 2 * se + 4 * se),
         "bimamba2_chunk_scan_bwd_dx": (u * (2 * Q * Q * P + 4 * Q * P * N) + scan_cb[1][0],
                                        3 * e * T4 + e * T2 + 4 * 4 * T1 + 2 * se + scan_cb[1][1]),
         "bimamba2_chunk_state_bwd_db": (u * 4 * Q * P * N, e * T4 + e * T2 + 5 * 4 * T1 + 2 * se + 4 * T2),
@@ -616,6 +617,15 @@ def main():
         if hidden and reads_cb[hidden[1]] == 0:
             kept = getattr(c.p, hidden[0])
             setattr(c.p, hidden[0], None)
+        # ... and without float32 state tensors where the composites keep the per-chunk states (their gradients) in the
+        # 16-bit copies' place
+        no_f32 = {"bimamba2_chunk_state_fwd": ("states_f", "states_b"), "bimamba2_state_passing_fwd": ("states_f", "states_b"),
+                  "bimamba2_chunk_scan_bwd_dstates": ("dstates_f", "dstates_b"),
+                  "bimamba2_chunk_scan_bwd_dz_dstates": ("dstates_f", "dstates_b"),
+                  "bimamba2_state_passing_bwd": ("dstates_f", "dstates_b")}.get(entry, ()) if copies else ()
+        kept_f32 = {f: getattr(c.p, f) for f in no_f32}
+        for f in no_f32:
+            setattr(c.p, f, None)
         for _ in range(3):
             c.run(entry)
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -626,6 +636,8 @@ def main():
         torch.cuda.synchronize()
         if kept is not None:
             setattr(c.p, hidden[0], kept)
+        for f, v in kept_f32.items():
+            setattr(c.p, f, v)
         us = ev0.elapsed_time(ev1) * 1e3 / reps
         kernels[entry] = {"us": round(us, 2), "gflop": round(flops / 1e9, 3), "mbytes": round(nbytes / 1e6, 2),
                           "tflops": round(flops / us / 1e6, 2), "gbs": round(nbytes / us / 1e3, 1)}

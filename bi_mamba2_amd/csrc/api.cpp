@@ -109,8 +109,15 @@ size_t carve(bimamba2_params *q, int is_bwd, void *ws) {
         need_f(q->dCB, cbn * dcb_slices(q));
         need_f(q->dCBT, cbn * dcb_slices(q));
         if (!scan_recomputes_cb(q, true)) need_f(q->CBT, cbn);
-        need_f(q->dstates_f, stn);
-        need_f(q->dstates_b, stn);
+        // where the 16-bit copies of the gradients exist and the caller asks for no float32 tensors, the per-chunk gradients
+        // live in the copies' place as well (written there by the dstates kernels, replaced in place by the backward
+        // inter-chunk scan): no float32 tensors at all
+        // (the in-place kernel of the backward inter-chunk scan reads the entering states from their copies as well)
+        const bool dstates16_only = copies && !q->dstates_f && !q->dstates_b && (carve16 || q->states16_f);
+        if (!dstates16_only) {
+            need_f(q->dstates_f, stn);
+            need_f(q->dstates_b, stn);
+        }
         if (q->has_z && !q->dout_x)
             q->dout_x = cv.take<char>((size_t)q->batch * q->seqlen * q->nheads * q->headdim * elem_size(q->dtype));
         need_f(q->ddt_direct, bhcq * ddt_direct_planes(*q));
@@ -257,7 +264,8 @@ int bimamba2_chunk_scan_bwd_dz(const bimamba2_params *p) {
 
 int bimamba2_chunk_scan_bwd_dstates(const bimamba2_params *p) {
     TRY(check_problem(p));
-    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->dstates_f); REQUIRE(p->dstates_b);
+    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (p->dstates_f || !p->dstates16_f) { REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); }   // (else: 16-bit per-chunk gradients in dstates16_*)
     if (p->has_z) REQUIRE(p->dout_x); else REQUIRE(p->dout);
     return launch_chunk_state(p, true);
 }
@@ -266,7 +274,8 @@ int bimamba2_chunk_scan_bwd_dz_dstates(const bimamba2_params *p) {
     TRY(check_problem(p));
     if (!p->has_z) return BIMAMBA2_EINVAL;
     REQUIRE(p->z); REQUIRE(p->dout); REQUIRE(p->out_x); REQUIRE(p->dz); REQUIRE(p->dout_x);
-    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b); REQUIRE(p->dstates_f); REQUIRE(p->dstates_b);
+    REQUIRE(p->Cm); REQUIRE(p->cs_f); REQUIRE(p->cs_b);
+    if (p->dstates_f || !p->dstates16_f) { REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); }
     return launch_bwd_dz_dstates(p);       // BIMAMBA2_EUNSUPPORTED where only the two separate kernels exist
 }
 
@@ -274,7 +283,8 @@ int bimamba2_state_passing_bwd(const bimamba2_params *p) {
     TRY(check_problem(p));
     REQUIRE(p->cs_f); REQUIRE(p->cs_b);
     if (!p->states16_f) { REQUIRE(p->states_f); REQUIRE(p->states_b); }
-    REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); REQUIRE(p->ddA_chunk_f); REQUIRE(p->ddA_chunk_b);
+    if (p->dstates_f || !p->dstates16_f) { REQUIRE(p->dstates_f); REQUIRE(p->dstates_b); }
+    REQUIRE(p->ddA_chunk_f); REQUIRE(p->ddA_chunk_b);
     return launch_state_passing_bwd(p);
 }
 
@@ -407,7 +417,8 @@ int bimamba2_bwd(const bimamba2_params *p) {
         TRY(bimamba2_chunk_scan_bwd_dc(&q));
         if (!dz_dstates) TRY(bimamba2_chunk_scan_bwd_dstates(&q));
         REQUIRE(q.x); REQUIRE(q.dt_out); REQUIRE(q.cs_f); REQUIRE(q.cs_b); REQUIRE(q.dCB); REQUIRE(q.dCBT); REQUIRE(q.da_intra);
-        REQUIRE(q.dstates_f); REQUIRE(q.ddA_chunk_f); REQUIRE(q.ddA_chunk_b);
+        if (!q.dstates16_f) REQUIRE(q.dstates_f);
+        REQUIRE(q.ddA_chunk_f); REQUIRE(q.ddA_chunk_b);
         if (q.has_z) REQUIRE(q.dout_x); else REQUIRE(q.dout);
         TRY(launch_bwd_dcb_sp(&q, dcb16));
     } else {

@@ -238,8 +238,10 @@ __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_kernel(const bimam
 // waited for at every link costs microseconds.  Needs P*N % 4 == 0 and 16-byte aligned tensors.
 // PREV16: the entering states are read from their 16-bit copies (states16_*); DS16: the gradients with respect to the
 // entering states go to dstates16_* and the per-chunk gradients in dstates_* stay as they are.
+// DP16 (with DS16): the per-chunk gradients lie in dstates16_* in the 16-bit type as well (no float32 tensors): every one is
+// read once and replaced in place by the gradient with respect to the state entering its chunk.
 constexpr int SP_CH = 8;
-template <typename T16, bool PREV16, bool DS16>
+template <typename T16, bool PREV16, bool DS16, bool DP16 = false>
 __device__ __forceinline__ void state_passing_bwd_vec_body(const bimamba2_params &p, int nc, int nsplit, int ndir, BlockId bid) {
     struct alignas(8) V4 { T16 v[4]; };
     __shared__ float red[SP_CH][4];
@@ -273,7 +275,13 @@ __device__ __forceinline__ void state_passing_bwd_vec_body(const bimamba2_params
             const int c = dir == 0 ? nc - 1 - sj : sj;
             dec[j] = cs[(int64_t)c * Q];
             // (both are read for the last time in the pass: past the caches)
-            dp[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(ds + c * cstride));
+            if constexpr (DP16) {
+                const V4 t = *reinterpret_cast<const V4 *>(ds16 + c * cstride);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) dp[j][k] = to_f(t.v[k]);
+            } else {
+                dp[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(ds + c * cstride));
+            }
             if constexpr (PREV16) {
                 typedef float f32x2 __attribute__((ext_vector_type(2)));
                 const V4 t = __builtin_bit_cast(V4, __builtin_nontemporal_load(reinterpret_cast<const f32x2 *>(prev16 + c * cstride)));
@@ -314,9 +322,9 @@ __device__ __forceinline__ void state_passing_bwd_vec_body(const bimamba2_params
     }
     if (dini && live) *reinterpret_cast<f32x4 *>(dini + bh) = g;
 }
-template <typename T16, bool PREV16, bool DS16>
+template <typename T16, bool PREV16, bool DS16, bool DP16 = false>
 __global__ __launch_bounds__(NTHREADS) void state_passing_bwd_vec_kernel(const bimamba2_params p, int nc, int nsplit, int ndir) {
-    state_passing_bwd_vec_body<T16, PREV16, DS16>(p, nc, nsplit, ndir, BlockId{(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z});
+    state_passing_bwd_vec_body<T16, PREV16, DS16, DP16>(p, nc, nsplit, ndir, BlockId{(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z});
 }
 
 int launch_state_passing_bwd(const bimamba2_params *p) {
@@ -331,6 +339,13 @@ int launch_state_passing_bwd(const bimamba2_params *p) {
         if (prev16 && (!(p->causal || p->states16_b) || !al(p->states16_f) || !al(p->states16_b))) return BIMAMBA2_EINVAL;
         if (ds16 && (!(p->causal || p->dstates16_b) || !al(p->dstates16_f) || !al(p->dstates16_b))) return BIMAMBA2_EINVAL;
         if ((prev16 || ds16) && p->dtype != BIMAMBA2_BF16 && p->dtype != BIMAMBA2_F16) return BIMAMBA2_EUNSUPPORTED;
+        if (!p->dstates_f) {
+            // the per-chunk gradients lie in dstates16_* (16-bit): in place; known with the 16-bit copies on both sides only
+            if (!(prev16 && ds16)) return BIMAMBA2_EINVAL;
+            if (p->dtype == BIMAMBA2_F16) hipLaunchKernelGGL((state_passing_bwd_vec_kernel<f16_t, true, true, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit, ndir);
+            else hipLaunchKernelGGL((state_passing_bwd_vec_kernel<bf16_t, true, true, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit, ndir);
+            return check_launch();
+        }
 #define BM2_SPB(TT, A, B) hipLaunchKernelGGL((state_passing_bwd_vec_kernel<TT, A, B>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit, ndir)
         if (p->dtype == BIMAMBA2_F16) {
             if (prev16 && ds16) BM2_SPB(f16_t, true, true); else if (prev16) BM2_SPB(f16_t, true, false);
@@ -344,6 +359,7 @@ int launch_state_passing_bwd(const bimamba2_params *p) {
     }
     if (p->states16_f || p->dstates16_f) return BIMAMBA2_EUNSUPPORTED;
     if (p->causal) return BIMAMBA2_EUNSUPPORTED;
+    if (!p->dstates_f || !p->dstates_b) return BIMAMBA2_EINVAL;
     dim3 grid(nsplit, p->nheads, p->batch);
     hipLaunchKernelGGL(state_passing_bwd_kernel, grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nsplit);
     return check_launch();
@@ -1708,7 +1724,9 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_sp_kernel(const bimamba2_par
         bwd_dcb_ring_body<T, UNI>(p, nc, nqt, BlockId{id % gdx, id / gdx, 0}, gdx, 1, out16);
     } else {
         const int k = id - ndcb;                  // grid (nsplit, nheads, batch * ndir) of the state passing
-        state_passing_bwd_vec_body<T, true, true>(p, nc, nsplit, ndir, BlockId{k % nsplit, (k / nsplit) % p.nheads, k / (nsplit * p.nheads)});
+        const BlockId sb{k % nsplit, (k / nsplit) % p.nheads, k / (nsplit * p.nheads)};
+        if (p.dstates_f == nullptr) state_passing_bwd_vec_body<T, true, true, true>(p, nc, nsplit, ndir, sb);
+        else state_passing_bwd_vec_body<T, true, true>(p, nc, nsplit, ndir, sb);
     }
 }
 

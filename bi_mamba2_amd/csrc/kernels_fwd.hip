@@ -440,7 +440,7 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     if (nsteps > 5) kstep(std::integral_constant<int, 5>());
     if (nsteps > 6) kstep(std::integral_constant<int, 6>());
     if (nsteps > 7) kstep(std::integral_constant<int, 7>());
-    if constexpr (OUT16 && !DSTATES) {
+    if constexpr (OUT16) {
         // the two 64 x 64 tiles as 16-bit values into the rings' LDS (everybody is done reading them behind the barrier): row
         // r at r * 128 bytes, 16-byte chunk ch at position ch ^ ((r / 4) % 4), which keeps the four lane groups (rows 4 apart)
         // off each other's banks; then every thread takes 32 contiguous bytes of a row of each tile to memory
@@ -457,8 +457,8 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
             }
         __syncthreads();
         const int r = threadIdx.x >> 2, c2 = (threadIdx.x & 3) * 2, sw = (r >> 2) & 3;
-        T *of = reinterpret_cast<T *>(p.states16_f) + (int64_t)bch * P * N + (int64_t)(pt * 64 + r) * N + nt * 64 + c2 * 8;
-        T *ob = reinterpret_cast<T *>(p.states16_b) + (int64_t)bch * P * N + (int64_t)(pt * 64 + r) * N + nt * 64 + c2 * 8;
+        T *of = reinterpret_cast<T *>(DSTATES ? p.dstates16_f : p.states16_f) + (int64_t)bch * P * N + (int64_t)(pt * 64 + r) * N + nt * 64 + c2 * 8;
+        T *ob = reinterpret_cast<T *>(DSTATES ? p.dstates16_b : p.states16_b) + (int64_t)bch * P * N + (int64_t)(pt * 64 + r) * N + nt * 64 + c2 * 8;
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
             const int at = r * 128 + (((c2 + k) ^ sw) << 4);
@@ -635,6 +635,32 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
     if (nsteps > 5) kstep(std::integral_constant<int, 5>());
     if (nsteps > 6) kstep(std::integral_constant<int, 6>());
     if (nsteps > 7) kstep(std::integral_constant<int, 7>());
+    if (p.dstates_f == nullptr) {
+        // no float32 tensors for the per-chunk gradients: they go to dstates16_f/b in the 16-bit type (where the backward
+        // inter-chunk scan replaces them in place), through LDS as 16-byte vectors - see chunk_state_direct_kernel<.., OUT16>
+        __syncthreads();
+        unsigned char *stf = reinterpret_cast<unsigned char *>(xt), *stb = reinterpret_cast<unsigned char *>(bt);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = wave * 16 + lg * 4 + i, cc = j * 16 + lr;
+                const int at = r * 128 + ((((cc >> 3) ^ lg) << 4) | ((cc & 7) << 1));
+                *reinterpret_cast<T *>(stf + at) = from_f<T>(accf[j][i]);
+                if (!UNI) *reinterpret_cast<T *>(stb + at) = from_f<T>(accb[j][i]);
+            }
+        __syncthreads();
+        const int r = threadIdx.x >> 2, c2 = (threadIdx.x & 3) * 2, sw = (r >> 2) & 3;
+        const int64_t so = (int64_t)blockIdx.z * P * N + (int64_t)(pt * 64 + r) * N + c2 * 8;
+        T *of = reinterpret_cast<T *>(p.dstates16_f) + so, *ob16 = reinterpret_cast<T *>(p.dstates16_b) + so;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int at = r * 128 + (((c2 + k) ^ sw) << 4);
+            *reinterpret_cast<f32x4 *>(of + k * 8) = *reinterpret_cast<const f32x4 *>(stf + at);
+            if (!UNI) *reinterpret_cast<f32x4 *>(ob16 + k * 8) = *reinterpret_cast<const f32x4 *>(stb + at);
+        }
+        return;
+    }
     float *of = p.dstates_f + (int64_t)blockIdx.z * P * N;
     float *obk = (UNI ? p.dstates_f : p.dstates_b) + (int64_t)blockIdx.z * P * N;
 #pragma unroll
@@ -971,6 +997,13 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cum
     }
     hipStream_t s = stream_of(p);
     if constexpr (sizeof(T) == 2) {
+        if (fast && p->chunk_size % 32 == 0 && dstates && !p->dstates_f) {
+            // no float32 tensors for the per-chunk gradients: 16-bit, into dstates16_f/b
+            if (!p->dstates16_f || !(p->causal || p->dstates16_b)) return BIMAMBA2_EINVAL;
+            if (p->causal) hipLaunchKernelGGL((chunk_state_direct_kernel<T, true, false, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            else hipLaunchKernelGGL((chunk_state_direct_kernel<T, true, false, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
+            return check_launch();
+        }
         if (fast && p->chunk_size % 32 == 0 && p->causal) {
             if (dstates) hipLaunchKernelGGL((chunk_state_direct_kernel<T, true, false, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
             else if (cumsum) hipLaunchKernelGGL((chunk_state_direct_kernel<T, false, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
@@ -995,6 +1028,7 @@ static int launch_chunk_state_t(const bimamba2_params *p, bool dstates, bool cum
     if (p->causal) return BIMAMBA2_EUNSUPPORTED;
     if (cumsum) return BIMAMBA2_EINVAL;      // the caller checked chunk_state_does_cumsum()
     if (!dstates && !(p->states_f && p->states_b)) return BIMAMBA2_EINVAL;   // (16-bit per-chunk states: the kernel above only)
+    if (dstates && !(p->dstates_f && p->dstates_b)) return BIMAMBA2_EINVAL;
     if (dstates) {
         if (fast) hipLaunchKernelGGL((chunk_state_kernel<T, true, true>), grid, dim3(NTHREADS), 0, s, *p, nc);
         else hipLaunchKernelGGL((chunk_state_kernel<T, true, false>), grid, dim3(NTHREADS), 0, s, *p, nc);
