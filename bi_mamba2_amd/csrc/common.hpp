@@ -479,4 +479,20 @@ struct ChunkIdx {
     int b, c, h, g, limit;
 };
 
+// Launch position -> (inner, outer) for a grid of nouter x ninner workgroups whose `ninner` workgroups of one outer index
+// share data: workgroups are dealt round-robin to the 8 XCDs (each with its own L2) in launch order, so eight outer indices
+// at a time, one per XCD, go through their inner indices; what is left when nouter is not a multiple of 8 shares the XCDs.
+__device__ __forceinline__ void xcd_order(int lin, int ninner, int nouter, int &inner, int &outer) {
+    const int full = nouter / 8, grp = lin / (8 * ninner);
+    if (grp < full) {
+        const int r = lin - grp * 8 * ninner;
+        inner = r >> 3;
+        outer = grp * 8 + (r & 7);
+    } else {
+        const int m = nouter - full * 8, r = lin - full * 8 * ninner;
+        inner = r / m;
+        outer = full * 8 + r % m;
+    }
+}
+
 }  // namespace bm2

@@ -1327,6 +1327,7 @@ __device__ __forceinline__ float lanegroup_sum_mfma(float v) {
 // Slots of the ring.  Two (the step being multiplied and the one after it, requested right after the barrier that frees
 // its slot) measured 60 us against 62 us for three slots requested two steps ahead.
 constexpr int DCB_RING = 2;
+constexpr int DCB_RESIDENT_BLOCKS = 1024;                 // a dCB grid up to this size is on the chip all at once
 constexpr int DCB_TILE_B = 64 * 64 * 2;                    // one 64 x 64 tile of 16-bit elements
 constexpr int DCB_CS_OFF = 2 * DCB_TILE_B;                 // cs_f[t], cs_b[t], cs_f[s], cs_b[s], dt[s]: 5 x 64 floats
 constexpr int DCB_SLOT_B = DCB_CS_OFF + 5 * 64 * 4;
@@ -1336,6 +1337,19 @@ constexpr int DCB_PART_B = 10 * 64 * 4;
 
 // UNI: the single-direction operator - tiles above the diagonal are empty, tiles on it keep the forward half.
 // bid / gdx / gdz: block index and grid extents (x: batch * chunks * groups, y: tiles, z: head slices)
+// Which (batch, chunk, group) and which tile the id-th workgroup of the dCB grid takes.  Workgroups are dealt round-robin to
+// the 8 XCDs in id order, and the tiles of one (b, c, g) read the same dout and x rows (each row tile four times at chunk
+// 256), so they belong on one XCD, close in time.  A grid that is resident all at once (two or three workgroups per CU)
+// has (b, c, g) fastest: equal ids modulo 8 share an XCD, and all diagonal tiles, which cost more, come first and spread
+// over the CUs.  A larger grid runs in several rounds, and with that order a row tile's readers are rounds apart and
+// each fetches it from memory again (768 MB of reads at 8 groups of 4 heads, batch 4 x 4096; 172 -> 155 us): there
+// eight (b, c, g) at a time, one per XCD, go through all their tiles before the next eight start.
+__device__ __forceinline__ BlockId dcb_block_of(int id, int gdx, int ntiles, int nblocks) {
+    if (nblocks <= DCB_RESIDENT_BLOCKS || gdx % 8) return BlockId{id % gdx, id / gdx, 0};
+    const int k = id >> 3;
+    return BlockId{(k / ntiles) * 8 + (id & 7), k % ntiles, 0};
+}
+
 template <typename T, bool UNI>
 __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int nc, int nqt, BlockId bid, int gdx, int gdz, bool out16 = false) {
     typedef Mma<T> M;
@@ -1709,7 +1723,9 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
 
 template <typename T, bool UNI = false>
 __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_params p, int nc, int nqt) {
-    bwd_dcb_ring_body<T, UNI>(p, nc, nqt, BlockId{(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z}, gridDim.x, gridDim.z);
+    BlockId bid = dcb_block_of(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x, gridDim.y, gridDim.x * gridDim.y);
+    bid.z = blockIdx.z;
+    bwd_dcb_ring_body<T, UNI>(p, nc, nqt, bid, gridDim.x, gridDim.z);
 }
 
 // The dCB kernel and the backward state passing as roles of one launch (16-bit copies of the entering states on both sides
@@ -1718,16 +1734,28 @@ __global__ __launch_bounds__(NTHREADS) void bwd_dcb_ring_kernel(const bimamba2_p
 // dCB tiles in the order of their own grid (so they are placed first, two per CU as when alone), the rest are the state
 // passing's blocks, which take what is left of each CU.
 template <typename T, bool UNI>
-__global__ __launch_bounds__(NTHREADS) void bwd_dcb_sp_kernel(const bimamba2_params p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir, bool out16) {
+__device__ __forceinline__ void bwd_dcb_sp_body(const bimamba2_params &p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir, bool out16) {
     const int id = blockIdx.x;
     if (id < ndcb) {
-        bwd_dcb_ring_body<T, UNI>(p, nc, nqt, BlockId{id % gdx, id / gdx, 0}, gdx, 1, out16);
+        bwd_dcb_ring_body<T, UNI>(p, nc, nqt, dcb_block_of(id, gdx, nqt * nqt, ndcb), gdx, 1, out16);
     } else {
         const int k = id - ndcb;                  // grid (nsplit, nheads, batch * ndir) of the state passing
         const BlockId sb{k % nsplit, (k / nsplit) % p.nheads, k / (nsplit * p.nheads)};
         if (p.dstates_f == nullptr) state_passing_bwd_vec_body<T, true, true, true>(p, nc, nsplit, ndir, sb);
         else state_passing_bwd_vec_body<T, true, true>(p, nc, nsplit, ndir, sb);
     }
+}
+
+template <typename T, bool UNI>
+__global__ __launch_bounds__(NTHREADS) void bwd_dcb_sp_kernel(const bimamba2_params p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir, bool out16) {
+    bwd_dcb_sp_body<T, UNI>(p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);
+}
+// The same with at most 128 registers, so that four workgroups fit a CU: for grids that run in several rounds of workgroups
+// of few heads each, where a workgroup's start (the C and B rows, the first tiles) and end (its dCB tile) are a large share
+// of its life and only other workgroups on the CU cover them.
+template <typename T, bool UNI>
+__global__ __launch_bounds__(NTHREADS, 4) void bwd_dcb_sp4_kernel(const bimamba2_params p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir, bool out16) {
+    bwd_dcb_sp_body<T, UNI>(p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);
 }
 
 template <typename T> static void launch_dcb_ring(dim3 grid, const bimamba2_params *p, int nc, int nqt) {
@@ -1791,9 +1819,11 @@ int launch_bwd_dcb_sp(const bimamba2_params *p, bool out16) {
     const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS), ndir = p->causal ? 1 : 2;
     const int gdx = p->batch * nc * p->ngroups, ndcb = gdx * nqt * nqt, nsp = nsplit * p->nheads * p->batch * ndir;
     dim3 grid(ndcb + nsp);
+    const bool four = ndcb > DCB_RESIDENT_BLOCKS;          // several rounds of workgroups: four per CU
 #define BM2_DS(TT)                                                                                                                     \
     do {                                                                                                                               \
         if (p->causal) hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);  \
+        else if (four) hipLaunchKernelGGL((bwd_dcb_sp4_kernel<TT, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);      \
         else hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);           \
     } while (0)
     if (p->dtype == BIMAMBA2_BF16) BM2_DS(bf16_t); else BM2_DS(f16_t);
@@ -2214,8 +2244,12 @@ __global__ __launch_bounds__(NTHREADS) void bwd_tail_kernel(const bimamba2_param
                                                             int bmm_gy, int cs_gx, bool in16) {
     const int id = blockIdx.x;
     if (id < nbmm) {
-        // bmm grid (1, bmm_gy, z)
-        bmm_chunk_bwd_body<T, 256, true, SLIM>(p, nc, nslices, BlockId{0, id % bmm_gy, id / bmm_gy}, in16);
+        // bmm grid (1, bmm_gy, z).  The bmm_gy row tiles of one z = (which, b, c, g) stage the same K operand (the chunk's C or
+        // B rows): consecutive ids are dealt round-robin to the 8 XCDs, so eight z at a time, one per XCD, go through their
+        // row tiles (with the row tile fastest every XCD fetched every K operand: +100 MB of reads at 8 groups)
+        const int nz = nbmm / bmm_gy, k = id >> 3;
+        const BlockId bb = nz % 8 == 0 ? BlockId{0, k % bmm_gy, (k / bmm_gy) * 8 + (id & 7)} : BlockId{0, id % bmm_gy, id / bmm_gy};
+        bmm_chunk_bwd_body<T, 256, true, SLIM>(p, nc, nslices, bb, in16);
     } else {
         const int k = id - nbmm;                  // cumsum grid (cs_gx, nc, batch)
         chunk_cumsum_bwd_body<DT>(p, nc, nqt, nsplit, BlockId{k % cs_gx, (k / cs_gx) % nc, k / (cs_gx * nc)});

@@ -228,18 +228,28 @@ __global__ __launch_bounds__(NTHREADS) void chunk_state_direct_kernel(const bima
     __shared__ __attribute__((aligned(16))) float wf[BIMAMBA2_MAX_CHUNK], wb[BIMAMBA2_MAX_CHUNK];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lr = lane & 15, lg = lane >> 4;
-    // Workgroups are dealt to the chip's eight dies in launch order, one after the other, and each die has its own L2.  With
-    // several tiles per (b, c, h) - which all read the same x rows - the launch order is remapped so that the tiles of one
-    // (b, c, h) are eight workgroups apart, i.e. on the same die: groups of eight (b, c, h), tile by tile.
+    // Workgroups are dealt to the chip's eight dies in launch order, one after the other, and each die has its own L2.
+    // Workgroups that read the same rows are therefore put eight launch positions apart, i.e. on one die.  With small
+    // groups (at most 8 heads) that is all the workgroups of one (b, c) - the tiles of a head share its x rows, the heads of
+    // a group the B (C) rows: eight (b, c) at a time, one per die, go through their heads and tiles (in plain launch order
+    // the 4 heads of a group of the 8-group benchmark shape sat on 4 dies and each fetched the B rows: 151 -> 100 MB read).
+    // With large groups only the tiles of one (b, c, h) are kept together: the heads of a (b, c) spread over the dies,
+    // a few per die, and the B rows are a small part of the traffic (all 32 heads of a one-group (b, c) on one die, asking
+    // for the same B tile at the same time, made the launch slower: 16.3 -> 18.7 us).
     int nt = blockIdx.x, pt = blockIdx.y, bch = blockIdx.z;
     {
-        const int tiles = gridDim.x * gridDim.y, nbch = gridDim.z;
-        if (tiles > 1) {
-            const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-            const int full = nbch / 8, grp = lin / (8 * tiles);
+        const int tiles = gridDim.x * gridDim.y;
+        const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        if (p.nheads <= 8 * p.ngroups) {
+            int inner, bc_;
+            xcd_order(lin, tiles * p.nheads, (int)gridDim.z / p.nheads, inner, bc_);
+            const int tile = inner % tiles;
+            bch = bc_ * p.nheads + inner / tiles;
+            nt = tile % (int)gridDim.x;
+            pt = tile / (int)gridDim.x;
+        } else if (tiles > 1) {
             int tile;
-            if (grp < full) { const int r = lin - grp * 8 * tiles; tile = r / 8; bch = grp * 8 + r % 8; }
-            else { const int m = nbch - full * 8, r = lin - full * 8 * tiles; tile = r / m; bch = full * 8 + r % m; }
+            xcd_order(lin, tiles, (int)gridDim.z, tile, bch);
             nt = tile % (int)gridDim.x;
             pt = tile / (int)gridDim.x;
         }
@@ -514,8 +524,17 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
     __shared__ __attribute__((aligned(16))) float wf[BIMAMBA2_MAX_CHUNK], wb[BIMAMBA2_MAX_CHUNK];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lr = lane & 15, lg = lane >> 4;
-    const int pt = blockIdx.y;
-    const int h = blockIdx.z % p.nheads, bc = blockIdx.z / p.nheads, c = bc % nc, b = bc / nc;
+    // with small groups the workgroups of one (b, c) run on one die, as in chunk_state_direct_kernel: the heads of a group
+    // share the C rows
+    int pt = blockIdx.y, bch = blockIdx.z;
+    if (p.nheads <= 8 * p.ngroups) {
+        const int lin = blockIdx.y + gridDim.y * blockIdx.z;
+        int inner, bc_;
+        xcd_order(lin, (int)gridDim.y * p.nheads, (int)gridDim.z / p.nheads, inner, bc_);
+        pt = inner % (int)gridDim.y;
+        bch = bc_ * p.nheads + inner / (int)gridDim.y;
+    }
+    const int h = bch % p.nheads, bc = bch / p.nheads, c = bc % nc, b = bc / nc;
     const int g = h / (p.nheads / p.ngroups);
     const int Q = p.chunk_size, N = p.dstate, P = p.headdim;
     const int limit = min(Q, p.seqlen - c * Q);
@@ -651,7 +670,7 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
             }
         __syncthreads();
         const int r = threadIdx.x >> 2, c2 = (threadIdx.x & 3) * 2, sw = (r >> 2) & 3;
-        const int64_t so = (int64_t)blockIdx.z * P * N + (int64_t)(pt * 64 + r) * N + c2 * 8;
+        const int64_t so = (int64_t)bch * P * N + (int64_t)(pt * 64 + r) * N + c2 * 8;
         T *of = reinterpret_cast<T *>(p.dstates16_f) + so, *ob16 = reinterpret_cast<T *>(p.dstates16_b) + so;
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
@@ -661,8 +680,8 @@ __global__ __launch_bounds__(NTHREADS) __attribute__((amdgpu_waves_per_eu(4, 4))
         }
         return;
     }
-    float *of = p.dstates_f + (int64_t)blockIdx.z * P * N;
-    float *obk = (UNI ? p.dstates_f : p.dstates_b) + (int64_t)blockIdx.z * P * N;
+    float *of = p.dstates_f + (int64_t)bch * P * N;
+    float *obk = (UNI ? p.dstates_f : p.dstates_b) + (int64_t)bch * P * N;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
