@@ -17,9 +17,9 @@
  *   Bm, Cm, dB, dC                   (B, L, G, N)   element type `dtype`; input strides given; outputs contiguous
  *   dt, ddt                          (B, L, H)      element type `dt_dtype`; strides given for dt; ddt contiguous
  *   A, D, dt_bias, dA, dD, ddt_bias  (H,) [D, dD may be (H, P)]   float32, contiguous
- *   dt_out, cs_f, cs_b, ddt_direct, u_f, u_b, v_f, v_b   (B, H, nc, Q)   float32
+ *   dt_out, cs_f, cs_b, u_f, u_b, v_f, v_b   (B, H, nc, Q)   float32; ddt_direct: bimamba2_ddt_direct_planes() such planes
  *   CB, CBT, dCB                     (B, nc, G, Q, Q)   float32, CB[.., l, s] = C_l . B_s, CBT its transpose
- *   states_f/b, dstates_f/b          (B, nc, H, P, N)   float32
+ *   states_f/b, dstates_f/b          (B, nc, H, P, N)   float32 (states16_*, dstates16_*: the same shape in `dtype`)
  *   final_f, final_b                 (B, H, P, N)       float32
  */
 #ifndef BIMAMBA2_H
@@ -52,7 +52,9 @@ enum {
 /* Added to the decay exponent across a change of seq_idx: every factor across a boundary carries e^-20 = 2e-9, below
  * float32 resolution next to the terms it is added to.  The cumulative sums of a chunk grow by this much per boundary
  * inside it, and their float32 resolution with them: relative accuracy of the in-sequence decays about 1.2e-6 per boundary
- * in the chunk (the float32 contract of 1e-4 holds up to about 40 boundaries per chunk). */
+ * in the chunk, so a float32 contract of 1e-4 holds up to about 40 boundaries per chunk.  The library does not count
+ * boundaries: a caller whose sequences can be shorter than chunk_size / 32 positions on average picks a smaller chunk_size
+ * (the result does not depend on it); the Python host does so for at most 32 boundaries per chunk. */
 #define BIMAMBA2_SEQ_CUT (-20.0f)
 
 typedef struct bimamba2_params {
@@ -135,6 +137,14 @@ typedef struct bimamba2_params {
        for the backward pass (fwd_saved) then passes states16_f / states16_b to both instead of states_f / states_b.
        bimamba2_fwd does so for every 16-bit problem (a forward pass without kept states has the scan stage as the only
        reader), bimamba2_bwd where bimamba2_state_copies() == 1.
+       Without the float32 tensors: with states_f = states_b = NULL and states16_* given (16-bit dtype, headdim and dstate
+       multiples of 64, chunk_size % 32 == 0, aligned operands, not causal), bimamba2_chunk_state_fwd writes the per-chunk
+       states to states16_* in `dtype` and bimamba2_state_passing_fwd turns them into the entering states in place; with
+       dstates_f = dstates_b = NULL and dstates16_* given (bimamba2_state_copies() == 1), bimamba2_chunk_scan_bwd_dstates /
+       _dz_dstates write the per-chunk gradients to dstates16_* and bimamba2_state_passing_bwd (which then needs states16_*
+       as well) replaces them in place.  The values are rounded to `dtype` once more than with the float32 tensors (the
+       per-chunk value before the inter-chunk scan adds it up in float32).  bimamba2_fwd and bimamba2_bwd work this way
+       whenever they own the state tensors: no float32 state tensor is written or read in a 16-bit pass.
        The reference keeps its entering states in the input dtype as well (out_dtype=C.dtype, src/ssd/bi/ssd_combined.py:324-327). */
     void *states16_f, *states16_b;
     void *dstates16_f, *dstates16_b;
@@ -163,8 +173,9 @@ size_t bimamba2_workspace_bytes(const bimamba2_params *p, int is_bwd);
 int bimamba2_state_copies(const bimamba2_params *p);
 
 /* Whether a kernel of this problem reads CB (1) or rebuilds the CB tiles it needs from the C and B rows with MFMAs (0):
- *   which = 0: bimamba2_chunk_scan_fwd reads CB      (0 for 16-bit dtype, dstate 64, headdim % 64 == 0, chunk_size % 32 == 0)
- *   which = 1: bimamba2_chunk_scan_bwd_dx reads CBT  (same conditions)
+ *   which = 0: bimamba2_chunk_scan_fwd reads CB      (0 for 16-bit dtype, dstate 64, headdim % 64 == 0, chunk_size % 32 == 0;
+ *              also 0 at dstate 128 when states16_* are set, i.e. when the persistent scan kernel runs)
+ *   which = 1: bimamba2_chunk_scan_bwd_dx reads CBT  (0 for 16-bit dtype, dstate 64, headdim % 64 == 0, chunk_size % 32 == 0)
  *   which = 2: bimamba2_chunk_scan_bwd_dcb reads CB  (0 for 16-bit dtype, dstate % 32 == 0, headdim % 64 == 0, chunk_size % 64 == 0)
  *   which = 3: (not about CB) 1 when bimamba2_fwd launches bimamba2_chunk_cumsum_fwd on its own, 0 when its chunk-state
  *              launch does the cumsum as well (16-bit dtype, headdim and dstate multiples of 64, chunk_size % 32 == 0)
@@ -216,7 +227,7 @@ int bimamba2_bwd(const bimamba2_params *p);
 int bimamba2_chunk_cumsum_fwd(const bimamba2_params *p);
 /* Cm, Bm -> CB (and CBT when that pointer is set).  Replaces _bmm_chunk_fwd (src/ssd/bi/ssd_bmm.py:163-208). */
 int bimamba2_bmm_chunk_fwd(const bimamba2_params *p);
-/* x, Bm, dt_out, cs_f, cs_b -> states_f, states_b.  Replaces _chunk_state_fwd
+/* x, Bm, dt_out, cs_f, cs_b -> states_f, states_b (or states16_f/b, see there).  Replaces _chunk_state_fwd
  * (src/ssd/bi/ssd_chunk_state.py:764-798). */
 int bimamba2_chunk_state_fwd(const bimamba2_params *p);
 /* states_f/b (chunk states) -> states_f/b (state entering each chunk), in place, both directions in one
