@@ -57,9 +57,10 @@ constexpr int S16_MAX_HEADS = 12;                 // heads a workgroup walks thr
 
 // LDS map (bytes), by the state dimension DS (64 or 128).
 // DS = 64: two buffers of x (dy) tiles, two buffers of state tiles, the K rows (32 KB) whose place takes the z (x) rows later.
-// DS = 128: the K rows take 64 KB and a pair of state tiles 32 KB, so the state tiles are single-buffered (the requests for
-// the next head's pair go out behind a barrier that follows this head's state products) and the K rows, needed only in
-// front of the first head, lie over the second x-tile buffer and the z-row area, which are filled later.
+// DS = 128: the K rows take 64 KB and a pair of state tiles 32 KB, so the map holds one pair of state tiles; the K rows, needed
+// only in front of the first head, lie over the second x-tile buffer and the z-row area, which are filled later.  With a z
+// gate the state tiles are single-buffered (the requests for the next head's pair go out behind a barrier that follows
+// this head's state products); without one the z-row area holds the second pair.
 template <int DS> struct S16Map {
     static constexpr int ROWB = DS * 2;                                   // bytes of a K row / of a state-tile row
     static constexpr int ST_TILE = 64 * ROWB;                             // one state tile [p][n], 16-byte chunks ^ (p % 8)
@@ -133,7 +134,12 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
     constexpr int KSTEP = 32, NSTEP = S16_NSTEP;
     constexpr int NF = DS / 32;                    // MFMA K steps over the state dimension
     constexpr int ROWB = L::ROWB;
-    constexpr bool ST_SINGLE = L::ST_BUFS == 1;
+    // One pair of state tiles where the map has room for one only (DS = 128) and the z-row area is in use; without a z gate
+    // that area (32 KB, free once the K rows are done with) holds the second pair.
+    const bool st_single = L::ST_BUFS == 1 && (BWD || p.has_z);
+    auto st_buf_off = [&](int buf) __attribute__((always_inline)) {
+        return L::ST_BUFS == 2 ? buf * 2 * L::ST_TILE : st_single ? 0 : buf * (L::ZR - L::ST);
+    };
     // (aligned: the fragment addresses below flip bit 6 of an absolute LDS address)
     __shared__ __attribute__((aligned(1024))) unsigned char smem[L::LDS];
     const unsigned sbase = lds_addr(smem);
@@ -187,19 +193,19 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             if (!(UNI && dir)) {
                 const int64_t so = ((int64_t)(b * nc + c) * H + h) * P * DS + (int64_t)p0 * DS;
                 const T *src = reinterpret_cast<const T *>(BWD ? (dir ? p.dstates16_b : p.dstates16_f) : (dir ? p.states16_b : p.states16_f));
-                const int sbuf = ST_SINGLE ? 0 : buf;
+                const int sboff = st_buf_off(buf);
                 if constexpr (DS == 64) {
                     // thread t of a half brings row t/8, chunk position t%8 <- chunk (t%8) ^ (row%8)
                     const int row = (wave & 7) * 8 + (ln >> 3);
                     const unsigned soff = (unsigned)((row * 64 + (((ln & 7) ^ (row & 7)) << 3)) * sizeof(T));
-                    load16_to_lds_at<BWD>(uniform_ptr(src + so), soff, smem + L::ST + (sbuf * 2 + dir) * L::ST_TILE + (wave & 7) * 1024);
+                    load16_to_lds_at<BWD>(uniform_ptr(src + so), soff, smem + L::ST + sboff + dir * L::ST_TILE + (wave & 7) * 1024);
                 } else {
                     // rows of 256 bytes: a wave of a half brings 8 rows in two loads of 4, chunk position l%16 <- chunk (l%16) ^ (row%8)
 #pragma unroll
                     for (int u = 0; u < 2; ++u) {
                         const int row = ((wave & 7) * 2 + u) * 4 + (ln >> 4);
                         const unsigned soff = (unsigned)(row * ROWB + (((ln & 15) ^ (row & 7)) << 4));
-                        load16_to_lds_at<BWD>(uniform_ptr(src + so), soff, smem + L::ST + (sbuf * 2 + dir) * L::ST_TILE + ((wave & 7) * 2 + u) * 1024);
+                        load16_to_lds_at<BWD>(uniform_ptr(src + so), soff, smem + L::ST + sboff + dir * L::ST_TILE + ((wave & 7) * 2 + u) * 1024);
                     }
                 }
             }
@@ -364,7 +370,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
         int hn = h + 1;
         asm volatile("" : "+s"(hn));
         // (single-buffered state tiles: theirs go out behind the barrier that follows the state products)
-        if (!ST_SINGLE && more && !active) request_head(hn, cur ^ 1);
+        if (!st_single && more && !active) request_head(hn, cur ^ 1);
         if (BWD || p.has_z) {
             const char *row2 = uniform_ptr(
                 BWD ? reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h * p.x_sh + p0
@@ -440,7 +446,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
             // Fragment (tile j, state step s) of a state tile lies at row s16_col(j, lr), 16-byte chunk (4 s + lg) ^ (row % 8).  With
             // row = [32 (j/2) + 4 (j%2)] + [8 (lr/4) + lr%4] the lane's part is one address and everything else a constant:
             // (row % 8) = lr%4 + 4 (j%2), so the chunk is (lg ^ lr%4) + 4 ((s%2) ^ (j%2)) + 8 (s/2).
-            const unsigned st_lane = sb + L::ST + (ST_SINGLE ? 0 : cur * 2 * L::ST_TILE) + (8 * (lr >> 2) + (lr & 3)) * ROWB + ((lg ^ (lr & 3)) << 4);
+            const unsigned st_lane = sb + L::ST + st_buf_off(cur) + (8 * (lr >> 2) + (lr & 3)) * ROWB + ((lg ^ (lr & 3)) << 4);
             static_for<0, (UNI ? 1 : 2)>([&](auto DIR) __attribute__((always_inline)) {
                 constexpr int dir = decltype(DIR)::value;
                 f32x4 tmp[4];
@@ -468,7 +474,7 @@ __global__ __launch_bounds__(S16_THREADS) void chunk_scan16_kernel(const bimamba
                 return true;
             });
         }
-        if constexpr (ST_SINGLE) {
+        if (st_single) {
             // the one pair of state tiles: every wave is done with it here, so the next head's pair may be requested (the
             // active waves do that at their third K step)
             raw_lds_wait();
