@@ -79,7 +79,7 @@ def test_forward_reference_grid(ops, shape):
 
 E2E = [
     # batch, seqlen, H, P, G, N, chunk, dtype, z, D ('none'|'h'|'hp'), bias, softplus, limit
-    (2, 256, 4, 32, 1, 16, 64, torch.float32, False, "h", True, True, (0.0, INF)),       # BASELINE config 0
+    (2, 256, 4, 32, 1, 16, 64, torch.float32, False, "h", True, True, (0.0, INF)),       # the reference’s own CPU-runnable benchmark shape
     (2, 250, 4, 32, 2, 16, 64, torch.float32, True, "hp", True, True, (0.0, INF)),
     (1, 130, 2, 64, 1, 64, 128, torch.float32, True, "h", False, False, (0.0, INF)),
     (2, 200, 4, 16, 4, 8, 32, torch.float32, False, "none", True, True, (0.01, 0.2)),
