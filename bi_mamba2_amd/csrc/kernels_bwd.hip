@@ -1387,19 +1387,25 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
             for (int i = threadIdx.x; i < DCB_VEC; i += NTHREADS) tv0[hh * tv_head + i] = 0.f;
     } else {
         const unsigned sbase = lds_addr(smem);
-        // ---- requests: unit u = i*256 + thread of a 64 x 64 tile is row r = u / 8, 16-byte chunk (u % 8) ^ (r % 8)
-        const T *ysrc[2], *xsrc[2];
+        // ---- requests: unit u = i*256 + thread of a 64 x 64 tile is row r = u / 8, 16-byte chunk (u % 8) ^ (r % 8).
+        // Addresses are a wave-uniform base (scalar registers, moved on from head to head) plus this lane's 32-bit byte offset
+        // (the launcher checks that the rows of a chunk lie within 32 bits of each other): six vector registers less than
+        // four per-lane pointers (126 registers instead of 138: four workgroups fit a CU where the grid has them).
+        const char *ybase, *xbase;
+        unsigned yoff[2], xoff[2];
         int64_t y_head, y_row;
         {
             const T *yp;
             if (p.has_z) { y_row = (int64_t)H * P; y_head = P; yp = reinterpret_cast<const T *>(p.dout_x) + ((int64_t)b * p.seqlen + (int64_t)c * Q) * y_row + (int64_t)h0 * P; }
             else { y_row = p.dout_sl; y_head = p.dout_sh; yp = reinterpret_cast<const T *>(p.dout) + b * p.dout_sb + (int64_t)c * Q * y_row + h0 * p.dout_sh; }
             const T *xp = reinterpret_cast<const T *>(p.x) + b * p.x_sb + (int64_t)c * Q * p.x_sl + h0 * p.x_sh;
+            ybase = uniform_ptr(yp);
+            xbase = uniform_ptr(xp);
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 const int u = i * NTHREADS + threadIdx.x, r = u >> 3, col = ((u & 7) ^ (r & 7)) * 8;
-                ysrc[i] = yp + (int64_t)min(t0 + r, limit - 1) * y_row + col;
-                xsrc[i] = xp + (int64_t)min(s0 + r, limit - 1) * p.x_sl + col;
+                yoff[i] = (unsigned)(((int64_t)min(t0 + r, limit - 1) * y_row + col) * (int64_t)sizeof(T));
+                xoff[i] = (unsigned)(((int64_t)min(s0 + r, limit - 1) * p.x_sl + col) * (int64_t)sizeof(T));
             }
         }
         const float *csrc;                                     // threads 0..79: 16-byte unit of the five decay vectors
@@ -1413,16 +1419,16 @@ __device__ __forceinline__ void bwd_dcb_ring_body(const bimamba2_params &p, int 
         // requests one step into `slot` and moves the source pointers on to the next step
         auto issue = [&](int slot) __attribute__((always_inline)) {
             unsigned char *sl = smem + slot * DCB_SLOT_B + wave * 1024;
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)ysrc[0], (lds_ptr_t)(sl), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)ysrc[1], (lds_ptr_t)(sl + 4096), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)xsrc[0], (lds_ptr_t)(sl + DCB_TILE_B), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)xsrc[1], (lds_ptr_t)(sl + DCB_TILE_B + 4096), 16, 0, 0);
+            load16_to_lds_at(ybase, yoff[0], sl);
+            load16_to_lds_at(ybase, yoff[1], sl + 4096);
+            load16_to_lds_at(xbase, xoff[0], sl + DCB_TILE_B);
+            load16_to_lds_at(xbase, xoff[1], sl + DCB_TILE_B + 4096);
             if (threadIdx.x < 80) __builtin_amdgcn_global_load_lds((gbl_ptr_t)csrc, (lds_ptr_t)(sl + DCB_CS_OFF), 16, 0, 0);
             const bool last = ++ikc == nkc;
             if (last) ikc = 0;
             const int64_t dy = last ? y_head - (nkc - 1) * KC : KC, dx = last ? x_head - (nkc - 1) * KC : KC;
-            ysrc[0] += dy; ysrc[1] += dy;
-            xsrc[0] += dx; xsrc[1] += dx;
+            ybase += dy * (int64_t)sizeof(T);
+            xbase += dx * (int64_t)sizeof(T);
             if (last) csrc += cs_head;
         };
         // ---- per-lane LDS byte offsets inside a slot
@@ -1750,14 +1756,6 @@ template <typename T, bool UNI>
 __global__ __launch_bounds__(NTHREADS) void bwd_dcb_sp_kernel(const bimamba2_params p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir, bool out16) {
     bwd_dcb_sp_body<T, UNI>(p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);
 }
-// The same with at most 128 registers, so that four workgroups fit a CU: for grids that run in several rounds of workgroups
-// of few heads each, where a workgroup's start (the C and B rows, the first tiles) and end (its dCB tile) are a large share
-// of its life and only other workgroups on the CU cover them.
-template <typename T, bool UNI>
-__global__ __launch_bounds__(NTHREADS, 4) void bwd_dcb_sp4_kernel(const bimamba2_params p, int nc, int nqt, int gdx, int ndcb, int nsplit, int ndir, bool out16) {
-    bwd_dcb_sp_body<T, UNI>(p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);
-}
-
 template <typename T> static void launch_dcb_ring(dim3 grid, const bimamba2_params *p, int nc, int nqt) {
     if constexpr (sizeof(T) == 2) {
         if (p->causal) hipLaunchKernelGGL((bwd_dcb_ring_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
@@ -1767,10 +1765,17 @@ template <typename T> static void launch_dcb_ring(dim3 grid, const bimamba2_para
 
 // whether the dCB kernel can do without CB (it rebuilds its tile from the C and B rows): the 16-bit ring variant, dstate a
 // multiple of 32, 16-byte aligned row matrices
+// the ring variant addresses the rows of a chunk with 32-bit byte offsets from a per-head base
+static bool dcb_rows_in_32bit(const bimamba2_params *p) {
+    // (a query that comes before dout is known - no pointer, no strides yet - is answered for the contiguous tensor)
+    const int64_t ys = (p->has_z || !p->dout) ? (int64_t)p->nheads * p->headdim : p->dout_sl;
+    return p->x_sl > 0 && p->x_sl < (1 << 22) && ys > 0 && ys < (1 << 22);
+}
+
 bool dcb_recomputes_cb(const bimamba2_params *p) {
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
     auto mult = [](int64_t a, int64_t b, int64_t c) { return a % 8 == 0 && b % 8 == 0 && c % 8 == 0; };
-    if (p->dtype == BIMAMBA2_F32 || p->headdim % 64 || p->chunk_size % 64 || p->dstate % 32) return false;
+    if (p->dtype == BIMAMBA2_F32 || p->headdim % 64 || p->chunk_size % 64 || p->dstate % 32 || !dcb_rows_in_32bit(p)) return false;
     if (!(al(p->x) && mult(p->x_sb, p->x_sl, p->x_sh))) return false;
     if (!(p->has_z ? al(p->dout_x) : (al(p->dout) && mult(p->dout_sb, p->dout_sl, p->dout_sh)))) return false;
     return al(p->Bm) && mult(p->B_sb, p->B_sl, p->B_sg) && al(p->Cm) && mult(p->C_sb, p->C_sl, p->C_sg);
@@ -1786,8 +1791,9 @@ static int launch_dcb_t(const bimamba2_params *p) {
     bool fast = p->headdim % (sizeof(T) == 2 ? 64 : 16) == 0 && al(p->x) && p->x_sb % VS == 0 && p->x_sl % VS == 0 && p->x_sh % VS == 0;
     fast = fast && (p->has_z ? al(p->dout_x) : (al(p->dout) && p->dout_sb % VS == 0 && p->dout_sl % VS == 0 && p->dout_sh % VS == 0));
     if (!p->CB && !dcb_recomputes_cb(p)) return BIMAMBA2_EINVAL;
-    if (p->causal && !(fast && sizeof(T) == 2 && p->chunk_size % 64 == 0)) return BIMAMBA2_EUNSUPPORTED;
-    if (fast && sizeof(T) == 2 && p->chunk_size % 64 == 0) launch_dcb_ring<T>(grid, p, nc, nqt);
+    const bool ring = fast && sizeof(T) == 2 && p->chunk_size % 64 == 0 && dcb_rows_in_32bit(p);
+    if (p->causal && !ring) return BIMAMBA2_EUNSUPPORTED;
+    if (ring) launch_dcb_ring<T>(grid, p, nc, nqt);
     else if (fast) hipLaunchKernelGGL((bwd_dcb_kernel<T, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
     else hipLaunchKernelGGL((bwd_dcb_kernel<T, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt);
     if (slices > 1) {
@@ -1819,11 +1825,9 @@ int launch_bwd_dcb_sp(const bimamba2_params *p, bool out16) {
     const int nsplit = (PN + SP_EPT * NTHREADS - 1) / (SP_EPT * NTHREADS), ndir = p->causal ? 1 : 2;
     const int gdx = p->batch * nc * p->ngroups, ndcb = gdx * nqt * nqt, nsp = nsplit * p->nheads * p->batch * ndir;
     dim3 grid(ndcb + nsp);
-    const bool four = ndcb > DCB_RESIDENT_BLOCKS;          // several rounds of workgroups: four per CU
 #define BM2_DS(TT)                                                                                                                     \
     do {                                                                                                                               \
         if (p->causal) hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, true>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);  \
-        else if (four) hipLaunchKernelGGL((bwd_dcb_sp4_kernel<TT, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);      \
         else hipLaunchKernelGGL((bwd_dcb_sp_kernel<TT, false>), grid, dim3(NTHREADS), 0, stream_of(p), *p, nc, nqt, gdx, ndcb, nsplit, ndir, out16);           \
     } while (0)
     if (p->dtype == BIMAMBA2_BF16) BM2_DS(bf16_t); else BM2_DS(f16_t);

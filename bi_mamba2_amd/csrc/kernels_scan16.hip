@@ -98,25 +98,6 @@ template <int I, int N, class F> __device__ __forceinline__ void static_for(F &&
     }
 }
 
-// load16_to_lds(base + off) with the address in the scalar-base form: `base` wave-uniform, `off` this lane's 32-bit byte
-// offset.  The offset passes through an empty asm right in front of the load, which keeps the 64-bit add next to the load
-// (hoisted into another block it could not be folded into the instruction and would cost two registers per address).
-// NT: the lines are not kept in the caches (data that no later kernel of the pass reads).
-template <bool NT = false>
-__device__ __forceinline__ void load16_to_lds_at(const char *base, unsigned off, void *lds_wave_base) {
-    asm volatile("" : "+v"(off));
-    if constexpr (NT) __builtin_amdgcn_global_load_lds((gbl_ptr_t)(base + off), (lds_ptr_t)lds_wave_base, 16, 0, 2);
-    else load16_to_lds(base + off, lds_wave_base);
-}
-
-// A wave-uniform pointer, made visibly so (through 64-bit address arithmetic the compiler loses sight of it and would build
-// the address per lane): base + 32-bit lane offset then takes the scalar-base form of the memory instructions.
-__device__ __forceinline__ const char *uniform_ptr(const void *ptr) {
-    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const char *>(((uint64_t)hi << 32) | lo);
-}
-
 }  // namespace
 
 // UNI: the single-direction (causal) operator: the reverse direction's state product, the K steps on the far side of the
