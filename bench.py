@@ -28,8 +28,8 @@ WORKLOAD = dict(batch=4, seqlen=2048, nheads=32, headdim=64, ngroups=1, dstate=6
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known
 # size); None until measured for the kernel in question.  Source: the summaries under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "bimamba2_chunk_scan_bwd_dcb": 101.0e6, "bimamba2_chunk_scan_bwd_dc": 64.7e6, "bimamba2_chunk_state_bwd_db": 65.3e6,
-    "bimamba2_chunk_scan_fwd": 169.1e6, "bimamba2_chunk_scan_bwd_dx": 126.1e6,
+    "bimamba2_chunk_scan_bwd_dcb": 100.2e6, "bimamba2_chunk_scan_bwd_dc": 64.4e6, "bimamba2_chunk_state_bwd_db": 65.3e6,
+    "bimamba2_chunk_scan_fwd": 169.5e6, "bimamba2_chunk_scan_bwd_dx": 126.1e6,
     "bimamba2_state_passing_bwd": 51.6e6, "bimamba2_bmm_chunk_bwd": 44.2e6, "bimamba2_chunk_state_fwd": 62.0e6,
     "bimamba2_state_passing_fwd": 34.1e6, "bimamba2_chunk_cumsum_bwd": 24.4e6,
     "bimamba2_bmm_chunk_fwd": 23.1e6, "bimamba2_chunk_scan_bwd_dz_dstates": 195.5e6,
